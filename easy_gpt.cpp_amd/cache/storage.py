@@ -1,0 +1,43 @@
+"""Device memory behind the cache manager: key/value slabs per group and per-request state records."""
+from __future__ import annotations
+
+import torch
+
+from ..parts.base import CacheNeed, StateNeed
+
+
+class KVStorage:
+    """For each group, keys and values as [slabs, num_pages, n_kv_heads, page_size, head_dim].
+
+    Within a page one head's tokens are contiguous (page_size * head_dim elements), which
+    is what the attention kernels stream.  Pages are never cleared: a kernel reads only
+    positions below a request's length."""
+
+    def __init__(self, groups, slabs_per_group, num_pages, page_size: int, dtype: torch.dtype, device):
+        self.page_size = page_size
+        self.k: list[torch.Tensor] = []
+        self.v: list[torch.Tensor] = []
+        for need, n_slabs, pages in zip(groups, slabs_per_group, num_pages):
+            shape = (n_slabs, pages, need.n_kv_heads, page_size, need.head_dim)
+            self.k.append(torch.zeros(shape, dtype=dtype, device=device))
+            self.v.append(torch.zeros(shape, dtype=dtype, device=device))
+
+    def slab(self, group: int, index: int):
+        return self.k[group][index], self.v[group][index]
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.k + self.v)
+
+
+class StateStorage:
+    """One record per request slot for every state id a model declares."""
+
+    def __init__(self, needs: dict[int, StateNeed], max_requests: int, device):
+        self.data = {
+            sid: torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+            for sid, need in needs.items()
+        }
+
+    def reset(self, slot: int) -> None:
+        for t in self.data.values():
+            t[slot].zero_()

@@ -1,0 +1,58 @@
+"""What one step hands to the model: the flattened tokens of all requests and where their cache lies."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..parts.base import CacheView, StateView
+
+
+@dataclass
+class GroupTables:
+    block_table: torch.Tensor   # int32 [B, W], -1 where there is no page
+    slots: torch.Tensor         # int32 [T], page * page_size + offset of each token of the step
+
+
+@dataclass
+class StepContext:
+    """T tokens of B requests, request after request.
+
+    token_ids, positions   int32 [T]; a token's position is the number of tokens before it in its request
+    q_start, q_len         int32 [B]: where each request's tokens start in the flat arrays, and how many
+    kv_len                 int32 [B]: tokens of the request in the cache once this step's are stored
+    want_rows              int32 [R]: flat indices of the tokens whose logits are wanted, or None
+    *_host                 the same numbers as Python lists, for parts that plan on the host
+    """
+
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor
+    positions: torch.Tensor
+    q_start: torch.Tensor
+    q_len: torch.Tensor
+    kv_len: torch.Tensor
+    want_rows: torch.Tensor | None
+    max_q_len: int
+    max_kv_len: int
+    q_start_host: list[int]
+    q_len_host: list[int]
+    kv_len_host: list[int]
+    state_slots: torch.Tensor
+    state_slots_host: list[int]
+    groups: list[GroupTables] = field(default_factory=list)
+    page_size: int = 0
+    kv_storage: object = None
+    state_storage: object = None
+    cache_location: dict = field(default_factory=dict)
+    group_windows: list = field(default_factory=list)
+
+    def cache_view(self, cache_id: int, writes: bool) -> CacheView:
+        g, j = self.cache_location[cache_id]
+        k, v = self.kv_storage.slab(g, j)
+        t = self.groups[g]
+        return CacheView(k, v, self.page_size, t.block_table, t.slots, self.group_windows[g], writes)
+
+    def state_view(self, state_id: int) -> StateView:
+        fresh = [kv == q for kv, q in zip(self.kv_len_host, self.q_len_host)]
+        return StateView(self.state_storage.data[state_id], self.state_slots, self.state_slots_host, fresh)

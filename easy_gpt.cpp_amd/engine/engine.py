@@ -1,0 +1,215 @@
+"""The engine: a loaded model, its cache, and the one step function.
+
+`step` takes a batch of (request, its next tokens): portions of prompts beside
+single decoded tokens, cut anywhere.  It runs only those tokens, as one batch,
+against what earlier steps left in the cache, and returns float32 logits at the
+wanted places.  The reference has two separate rectangular calls for this
+(/root/reference/src/models/gpt_model.cpp:375-419: sample_prefill_continuous and
+sample_decode_continuous, positions as offsets -pad_len / pos_len from
+/root/reference/src/models/generation_invariants.cpp:25-51); here positions are
+the true positions and nothing is padded.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, KVStorage, OutOfPages, RequestCache, StateStorage
+from ..config.registry import load_model_config
+from ..parts.model import Model, build_model
+from ..weights.loader import CheckedWeights
+from .context import GroupTables, StepContext
+
+DTYPES = {
+    "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+    "float32": torch.float32, "fp32": torch.float32,
+}
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one request and the places among them whose logits are wanted."""
+
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)
+
+
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> Model:
+    """Model folder -> model on the device: config.json picks the architecture, the weights
+    are checked by name and shape and then taken by the parts."""
+    arch, cfg = load_model_config(model_dir)
+    spec = arch.build_spec(cfg)
+    model = build_model(spec)
+    weights = CheckedWeights(model_dir, model.param_specs(), spec.ignorable_tensors)
+    try:
+        for name in weights.ignored:
+            print(f"[weights] tensor '{name}' is not used by this model and was ignored", flush=True)
+        torch_dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype
+        model.load(weights.get, torch_dtype, torch.device(device))
+    finally:
+        weights.close()
+    model.config = cfg
+    return model
+
+
+class Engine:
+    def __init__(
+        self,
+        model: Model,
+        *,
+        page_size: int = 16,
+        max_tokens: int | None = None,
+        num_pages: int | None = None,
+        max_requests: int = 64,
+    ):
+        """max_tokens: the most tokens live requests hold at any time (each request's count
+        rounded up to a page); the pools are made for that many.  num_pages sets the page
+        count directly."""
+        if model.device is None:
+            raise RuntimeError("the model has no weights yet (Model.load)")
+        self.model = model
+        self.device = model.device
+        self.page_size = int(page_size)
+        if num_pages is None:
+            if max_tokens is None:
+                raise ValueError("give max_tokens or num_pages")
+            num_pages = -(-int(max_tokens) // self.page_size)
+        groups = [g.need for g in model.cache_groups]
+        self.cache = CacheManager(groups, self.page_size, int(num_pages), max_requests)
+        self.kv = KVStorage(
+            groups, [len(g.cache_ids) for g in model.cache_groups], [num_pages] * len(groups),
+            self.page_size, model.dtype, self.device,
+        )
+        self.states = StateStorage(model.state_needs, max_requests, self.device)
+        self.vocab_size = model.spec.vocab_size
+        self.max_position = model.spec.max_position
+
+    @classmethod
+    def from_dir(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        return cls(load_model(model_dir, dtype, device), **kw)
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, request_id) -> RequestCache:
+        rc = self.cache.admit(request_id)
+        self.states.reset(rc.slot)
+        return rc
+
+    def finish(self, request_id) -> None:
+        self.cache.release(self.cache.requests[request_id])
+
+    def has_request(self, request_id) -> bool:
+        return request_id in self.cache.requests
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
+        of each entry's `want`, or None if nothing is wanted.  Raises OutOfPages (with the cache
+        unchanged) if the tokens do not fit."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return None
+        rcs = self._check(entries)
+        self._reserve_all(rcs, entries)
+        ctx = self._build_context(rcs, entries)
+        logits = self.model.forward(ctx)
+        for rc, e in zip(rcs, entries):
+            self.cache.commit(rc, len(e.tokens))
+        return logits
+
+    def _check(self, entries) -> list[RequestCache]:
+        rcs, seen = [], set()
+        for e in entries:
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            if e.request_id not in self.cache.requests:
+                raise KeyError(f"request {e.request_id!r} is not live (add_request first)")
+            rc = self.cache.requests[e.request_id]
+            n = len(e.tokens)
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise IndexError(f"token id {t} of request {e.request_id!r} is outside [0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise IndexError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
+            if rc.num_tokens + n > self.max_position:
+                raise ValueError(
+                    f"request {e.request_id!r} would reach {rc.num_tokens + n} tokens, "
+                    f"max_position_embeddings is {self.max_position}"
+                )
+            rcs.append(rc)
+        return rcs
+
+    def _reserve_all(self, rcs, entries) -> None:
+        before = [[len(t) for t in rc.tables] for rc in rcs]
+        try:
+            for rc, e in zip(rcs, entries):
+                self.cache.reserve(rc, len(e.tokens))
+        except OutOfPages:
+            for rc, lens in zip(rcs, before):       # give back what this step took
+                for pool, table, n in zip(self.cache.pools, rc.tables, lens):
+                    extra = [p for p in table[n:] if p >= 0]
+                    if extra:
+                        pool.give_back(extra)
+                    del table[n:]
+            raise
+
+    def _build_context(self, rcs, entries) -> StepContext:
+        ps = self.page_size
+        n_groups = len(self.cache.groups)
+        b = len(entries)
+        q_len = [len(e.tokens) for e in entries]
+        q_start = [0] * b
+        for i in range(1, b):
+            q_start[i] = q_start[i - 1] + q_len[i - 1]
+        t = q_start[-1] + q_len[-1]
+        kv_len = [rc.num_tokens + n for rc, n in zip(rcs, q_len)]
+        token_ids = np.empty(t, dtype=np.int32)
+        positions = np.empty(t, dtype=np.int32)
+        slots = np.empty((max(n_groups, 1), t), dtype=np.int32)
+        widths = [max((len(rc.tables[g]) for rc in rcs), default=1) or 1 for g in range(n_groups)]
+        tables = [np.full((b, widths[g]), -1, dtype=np.int32) for g in range(n_groups)]
+        want_rows: list[int] = []
+        for i, (rc, e) in enumerate(zip(rcs, entries)):
+            s, n = q_start[i], q_len[i]
+            token_ids[s : s + n] = np.asarray(e.tokens, dtype=np.int64)
+            pos = np.arange(rc.num_tokens, rc.num_tokens + n, dtype=np.int64)
+            positions[s : s + n] = pos
+            for g in range(n_groups):
+                tab = np.asarray(rc.tables[g], dtype=np.int64)
+                tables[g][i, : len(tab)] = tab
+                pages = tab[pos // ps]
+                if (pages < 0).any():
+                    raise RuntimeError("a token of this step would be stored in a page that was given back")
+                slots[g, s : s + n] = pages * ps + pos % ps
+            want_rows.extend(s + int(w) for w in e.want)
+        # one packed upload for everything
+        parts = [token_ids, positions, np.asarray(q_start, np.int32), np.asarray(q_len, np.int32),
+                 np.asarray(kv_len, np.int32), np.asarray([rc.slot for rc in rcs], np.int32),
+                 np.asarray(want_rows, np.int32)]
+        parts += [slots[g] for g in range(n_groups)] + [tables[g].reshape(-1) for g in range(n_groups)]
+        sizes = [p.size for p in parts]
+        packed = torch.from_numpy(np.concatenate([p.reshape(-1) for p in parts]).astype(np.int32, copy=False))
+        if self.device.type == "cuda":
+            packed = packed.pin_memory()
+        dev = packed.to(self.device, non_blocking=True)
+        views, off = [], 0
+        for n in sizes:
+            views.append(dev[off : off + n])
+            off += n
+        d_tok, d_pos, d_qs, d_ql, d_kv, d_slot, d_want = views[:7]
+        groups = []
+        for g in range(n_groups):
+            groups.append(GroupTables(views[7 + n_groups + g].view(b, widths[g]), views[7 + g]))
+        return StepContext(
+            num_tokens=t, num_seqs=b, token_ids=d_tok, positions=d_pos, q_start=d_qs, q_len=d_ql, kv_len=d_kv,
+            want_rows=d_want if want_rows else None, max_q_len=max(q_len), max_kv_len=max(kv_len),
+            q_start_host=q_start, q_len_host=q_len, kv_len_host=kv_len,
+            state_slots=d_slot, state_slots_host=[rc.slot for rc in rcs],
+            groups=groups, page_size=ps, kv_storage=self.kv, state_storage=self.states,
+            cache_location=self.model.cache_location, group_windows=[n.window for n in self.cache.groups],
+        )

@@ -1,0 +1,53 @@
+"""The kernel backend: the one place from which parts reach device code.
+
+`backend()` returns the object whose methods launch the hand-written HIP kernels
+(`kernels.hip.HipKernels`).  There is no CPU implementation in the product: if
+the compiled extension cannot be loaded on a machine with a GPU, `backend()`
+raises.  `use_backend` lets a test put an object with the same methods in its
+place (the tests' own slow emulation, to exercise the engine's bookkeeping on a
+machine without a GPU).
+
+Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
+
+  embed(token_ids i32[T], table act[V,H], out f32[T,H])
+  add_rmsnorm(h f32[T,H], delta act[T,H]|None, weight act[H], eps, out act[T,H])
+        h += delta in float32 (in place), out = h * rsqrt(mean(h^2) + eps) * weight
+  rows_add_rmsnorm(h, delta|None, rows i32[R], weight, eps, out act[R,H])
+        the same for rows `rows` only, h is not written
+  linear(x act[T,K], w act[N,K], bias act[N]|None, out act|f32 [T,N])      out = x w^T + bias
+  qkv_rope_store(qkv act[T,(nq+2nkv)*hd], bias|None, positions i32[T], inv_freq f32[rd/2]|None,
+                 rotary_dim, slots i32[T]|None, k_cache, v_cache, nq, nkv, hd, page_size)
+        adds bias, rotates the first rotary_dim features of every query and key head
+        (pairs (i, i + rotary_dim/2), angle = position * inv_freq[i]) in place, and stores
+        keys and values at `slots` (page * page_size + offset) of caches [P,nkv,page_size,hd]
+  paged_attention(qkv, out act[T,nq*hd], k_cache, v_cache, block_table i32[B,W], q_start i32[B],
+                  q_len i32[B], kv_len i32[B], nq, nkv, hd, page_size, scale, window,
+                  max_q_len, max_kv_len)
+        query i of request b stands at position p = kv_len[b] - q_len[b] + i and reads keys
+        j <= p (and j > p - window if window > 0) of that request through its block table
+  swiglu(gate_up act[T,2I], out act[T,I])        out = silu(gate_up[:, :I]) * gate_up[:, I:]
+  argmax(logits f32[R,V], out i32[R])            lowest index among equal maxima
+  sample(logits f32[R,V], temperature f32[R], top_k i32[R], top_p f32[R], uniform f32[R], out i32[R])
+"""
+from __future__ import annotations
+
+_backend = None
+
+
+class KernelsUnavailable(RuntimeError):
+    pass
+
+
+def backend():
+    global _backend
+    if _backend is None:
+        from .hip import HipKernels  # raises KernelsUnavailable with the reason
+
+        _backend = HipKernels()
+    return _backend
+
+
+def use_backend(obj) -> None:
+    """Install `obj` as the backend (None restores the default).  For tests."""
+    global _backend
+    _backend = obj

@@ -1,0 +1,125 @@
+"""Grouped-query softmax attention over the paged cache.
+
+As the reference computes it (/root/reference/src/models/self_attn.cpp:217-260 and
+the CUDA path /root/reference/src/cuda/ops/self_attn.cu:299-369,689-980):
+q = x Wq^T + bq, k = x Wk^T + bk, v = x Wv^T + bv; features h*hd + d belong to head h
+(/root/reference/src/tensor.cpp:101-114); queries and keys are rotated; keys and
+values of the new tokens join the cache before attention so a prompt portion
+attends to itself causally; query head h reads key/value head h // (nq/nkv)
+(/root/reference/src/cuda/ops/self_attn_detail.cuh:669); score = q.k / sqrt(hd),
+softmax in float32, output = sum_j p_j v_j; heads are concatenated and projected
+by Wo (no bias in Qwen2, bias used if the tensor exists: src/models/linear.cpp:30-39).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import kernels
+from .base import CacheNeed, Mixer, make_part, register_part
+from .spec import ParamSpec, PartSpec
+
+
+class GQAttention(Mixer):
+    def __init__(
+        self,
+        prefix: str,
+        hidden_size: int,
+        n_heads: int,
+        n_kv_heads: int,
+        head_dim: int,
+        qkv_bias: bool,
+        out_bias: bool,
+        position: PartSpec,
+        window: int | None = None,
+        scale: float | None = None,
+    ):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"n_heads ({n_heads}) must be a multiple of n_kv_heads ({n_kv_heads})")
+        self.prefix = prefix
+        self.hidden_size = int(hidden_size)
+        self.n_heads = int(n_heads)
+        self.n_kv_heads = int(n_kv_heads)
+        self.head_dim = int(head_dim)
+        self.qkv_bias = bool(qkv_bias)
+        self.out_bias = bool(out_bias)
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.position = make_part("position_encoding", position, head_dim=self.head_dim)
+        self.q_size = self.n_heads * self.head_dim
+        self.kv_size = self.n_kv_heads * self.head_dim
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    # ------------------------------------------------------------------ declaration
+    def cache_need(self):
+        return CacheNeed(self.n_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self):
+        p, h = self.prefix, self.hidden_size
+        specs = [
+            ParamSpec(p + "q_proj.weight", (self.q_size, h)),
+            ParamSpec(p + "k_proj.weight", (self.kv_size, h)),
+            ParamSpec(p + "v_proj.weight", (self.kv_size, h)),
+            ParamSpec(p + "o_proj.weight", (h, self.q_size)),
+        ]
+        if self.qkv_bias:
+            specs += [
+                ParamSpec(p + "q_proj.bias", (self.q_size,), role="bias"),
+                ParamSpec(p + "k_proj.bias", (self.kv_size,), role="bias"),
+                ParamSpec(p + "v_proj.bias", (self.kv_size,), role="bias"),
+            ]
+        if self.out_bias:
+            specs.append(ParamSpec(p + "o_proj.bias", (h,), role="bias"))
+        return specs + self.position.param_specs()
+
+    def load(self, get, dtype, device):
+        p = self.prefix
+        # q, k and v stay separate tensors in the file; on the device their rows are one
+        # matrix so that one product serves all three.
+        w = torch.cat([get(p + n + "_proj.weight").to(dtype) for n in "qkv"], dim=0)
+        self.w_qkv = w.to(device).contiguous()
+        if self.qkv_bias:
+            b = torch.cat([get(p + n + "_proj.bias").to(dtype) for n in "qkv"], dim=0)
+            self.b_qkv = b.to(device).contiguous()
+        self.w_o = self._to(get(p + "o_proj.weight"), "compute", dtype, device)
+        if self.out_bias:
+            self.b_o = self._to(get(p + "o_proj.bias"), "compute", dtype, device)
+        self.position.load(get, dtype, device)
+
+    # ------------------------------------------------------------------ computation
+    def forward(self, x, ctx, cache, state=None):
+        k = kernels.backend()
+        t = x.shape[0]
+        qkv = torch.empty((t, self.q_size + 2 * self.kv_size), dtype=x.dtype, device=x.device)
+        k.linear(x, self.w_qkv, None, qkv)
+        slots = cache.slots if cache.writes else None
+        rot = self.position.rotary(x.device)
+        common = dict(
+            k_cache=cache.k, v_cache=cache.v, nq=self.n_heads, nkv=self.n_kv_heads,
+            hd=self.head_dim, page_size=cache.page_size,
+        )
+        if rot is not None:
+            inv_freq, rotary_dim = rot
+            k.qkv_rope_store(qkv, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, **common)
+        else:
+            # bias, then the position encoding's own transform, then the store
+            if self.b_qkv is not None:
+                k.qkv_rope_store(qkv, self.b_qkv, ctx.positions, None, 0, None, **common)
+            q_view = qkv[:, : self.q_size].view(t, self.n_heads, self.head_dim)
+            k_view = qkv[:, self.q_size : self.q_size + self.kv_size].view(t, self.n_kv_heads, self.head_dim)
+            self.position.apply(q_view, k_view, ctx.positions)
+            if slots is not None:
+                k.qkv_rope_store(qkv, None, ctx.positions, None, 0, slots, **common)
+        attn = torch.empty((t, self.q_size), dtype=x.dtype, device=x.device)
+        k.paged_attention(
+            qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
+            nq=self.n_heads, nkv=self.n_kv_heads, hd=self.head_dim, page_size=cache.page_size,
+            scale=self.scale, window=self.window or 0, max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len,
+        )
+        out = torch.empty((t, self.hidden_size), dtype=x.dtype, device=x.device)
+        k.linear(attn, self.w_o, self.b_o, out)
+        return out
+
+
+register_part("mixer", "gq_attention", GQAttention)

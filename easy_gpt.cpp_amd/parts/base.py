@@ -1,0 +1,203 @@
+"""Interfaces of the parts a layer is made of, and the registries that name them.
+
+A part gets its sizes and constants as constructor parameters, declares the
+tensors it needs (`param_specs`), takes them (`load`) and computes (`forward`)
+through the kernel backend.  It never learns which model it belongs to.
+
+Shapes in the docstrings: T tokens of the step (all requests flattened), B
+requests of the step, H the model width.  "act" is the engine's activation
+dtype (bfloat16 or float32); the residual stream `h` is always float32.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable
+
+import torch
+
+from .spec import ParamSpec, PartSpec
+
+
+# --------------------------------------------------------------------------- needs
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer asks of the paged cache: keys and values per token.
+
+    window None: every earlier token stays readable.  window W: a token reads only
+    the last W tokens (itself included); pages wholly behind that are given back.
+    """
+
+    n_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: one record of `shape` and `dtype` per live request."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+# --------------------------------------------------------------------------- views handed to a mixer
+@dataclass
+class CacheView:
+    """One cache slab as a mixer sees it during a step.
+
+    k, v         [num_pages, n_kv_heads, page_size, head_dim], act
+    block_table  int32 [B, W]: page ids of each request in order (-1 where a page was given back)
+    slots        int32 [T]: page * page_size + offset where each token of the step is stored
+    """
+
+    k: torch.Tensor
+    v: torch.Tensor
+    page_size: int
+    block_table: torch.Tensor
+    slots: torch.Tensor
+    window: int | None
+    writes: bool = True
+
+
+@dataclass
+class StateView:
+    """Per-request state records: `data[slot]` belongs to the request that holds `slot`.
+
+    data       [max_requests, *shape]
+    slots      int32 [B] slot of each request of the step (device); slots_host the same on the host
+    fresh      list[bool]: True where the request has no tokens before this step (state must start anew)
+    """
+
+    data: torch.Tensor
+    slots: torch.Tensor
+    slots_host: list[int]
+    fresh: list[bool]
+
+
+# --------------------------------------------------------------------------- part interfaces
+class Part:
+    """Common interface: parameters declared, loaded, then used."""
+
+    def param_specs(self) -> list[ParamSpec]:
+        return []
+
+    def load(self, get: Callable[[str], torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        """Take the tensors declared by `param_specs`; `get(name)` returns the stored (CPU) tensor."""
+
+    @staticmethod
+    def _to(t: torch.Tensor, spec_dtype: str, dtype: torch.dtype, device) -> torch.Tensor:
+        if spec_dtype == "compute":
+            t = t.to(dtype)
+        return t.to(device).contiguous()
+
+
+class Norm(Part):
+    """forward(h, delta, out): h += delta (float32, in place, skipped when delta is None);
+    returns norm(h) as act [T, H].  forward_rows does the same for selected rows without
+    writing h back (used for the rows whose logits are wanted)."""
+
+    def forward(self, h: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_rows(self, h: torch.Tensor, delta: torch.Tensor | None, rows: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How token positions enter a mixer.
+
+    Either `rotary()` returns (inv_freq float32 [rotary_dim/2], rotary_dim) and the
+    mixer's fused kernel rotates queries and keys itself, or it returns None and
+    `apply(q, k, positions)` changes the [T, heads, head_dim] views in place.
+    """
+
+    def rotary(self, device) -> tuple[torch.Tensor, int] | None:
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request.
+
+    forward(x, ctx, cache, state) -> act [T, H]; x is the normed input act [T, H];
+    ctx is the engine's StepContext; cache a CacheView if `cache_need()` is not None;
+    state a StateView if `state_need()` is not None.
+    """
+
+    def cache_need(self) -> CacheNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: CacheView | None, state: StateView | None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(x) -> act [T, H] for x act [T, H]; tokens are independent."""
+
+    def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of one layer's parts around the residual stream.
+
+    forward(h, delta, ctx, cache, state) -> delta': `h` float32 [T, H] is updated in
+    place; `delta` is the not-yet-added output of the previous layer (None for the
+    first) and the return value the not-yet-added output of this one, so that the
+    addition fuses with the next norm.
+    """
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.feed_forward_norm = feed_forward_norm
+
+    def parts(self) -> list[Part]:
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def forward(self, h, delta, ctx, cache, state):
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registries
+MIXERS: dict[str, Callable[..., Mixer]] = {}
+FEED_FORWARDS: dict[str, Callable[..., FeedForward]] = {}
+NORMS: dict[str, Callable[..., Norm]] = {}
+POSITION_ENCODINGS: dict[str, Callable[..., PositionEncoding]] = {}
+BLOCKS: dict[str, Callable[..., Block]] = {}
+EMBEDDINGS: dict[str, Callable[..., Part]] = {}
+OUTPUT_HEADS: dict[str, Callable[..., Part]] = {}
+
+_REGISTRIES = {
+    "mixer": MIXERS,
+    "feed_forward": FEED_FORWARDS,
+    "norm": NORMS,
+    "position_encoding": POSITION_ENCODINGS,
+    "block": BLOCKS,
+    "embedding": EMBEDDINGS,
+    "output_head": OUTPUT_HEADS,
+}
+
+
+def register_part(family: str, kind: str, factory: Callable[..., Any], replace: bool = False) -> None:
+    """Add a part under `kind` to one of the families: mixer, feed_forward, norm,
+    position_encoding, block, embedding, output_head."""
+    reg = _REGISTRIES[family]
+    if kind in reg and not replace:
+        raise ValueError(f"{family} '{kind}' is already registered")
+    reg[kind] = factory
+
+
+def make_part(family: str, spec: PartSpec, **context) -> Any:
+    """Build the part `spec.kind` of `family` with `spec.params`, its name prefix and the
+    sizes the surrounding model gives every part (`context`, e.g. hidden_size)."""
+    reg = _REGISTRIES[family]
+    if spec.kind not in reg:
+        raise KeyError(f"unknown {family} kind '{spec.kind}' (registered: {', '.join(sorted(reg)) or 'none'})")
+    return reg[spec.kind](prefix=spec.prefix, **context, **dict(spec.params))

@@ -1,0 +1,96 @@
+"""Weights by tensor name, checked against what the model declares before anything is read.
+
+The reference validates required keys and shapes before loading and reports
+left-over keys afterwards (/root/reference/src/models/model_param_validation.cpp:84-218;
+fixtures in /root/reference/test/model_param_validation_test.cpp:345-426).  Here one
+error lists every missing tensor, every unexpected tensor and every wrong shape.
+
+Stored dtypes: BF16 stays bfloat16, F16 becomes bfloat16, F32 stays float32 (F64
+becomes float32), integer tables become int32.  Parts cast 'compute' parameters to
+the engine's dtype when they take them.
+"""
+from __future__ import annotations
+
+import os
+from typing import Iterable
+
+import torch
+
+from ..parts.spec import ParamSpec
+from .safetensors_io import SafetensorsFile
+
+
+class WeightsError(RuntimeError):
+    """The weights file does not hold what the model declares."""
+
+    def __init__(self, message: str, missing=(), unexpected=(), wrong_shape=()):
+        super().__init__(message)
+        self.missing = list(missing)
+        self.unexpected = list(unexpected)
+        self.wrong_shape = list(wrong_shape)
+
+
+def check_names_and_shapes(
+    available: dict[str, tuple[int, ...]],
+    specs: Iterable[ParamSpec],
+    ignorable: Iterable[str] = (),
+    where: str = "weights",
+) -> list[str]:
+    """Compare the tensors on offer with the declared ones.  Raises one WeightsError that
+    lists all problems; returns the ignorable names that were present (to warn about)."""
+    specs = list(specs)
+    declared = {s.name: s for s in specs}
+    missing = [s.name for s in specs if s.name not in available]
+    ignorable = set(ignorable)
+    unexpected = [n for n in available if n not in declared and n not in ignorable]
+    ignored = [n for n in available if n not in declared and n in ignorable]
+    wrong = []
+    for name, spec in declared.items():
+        if name in available:
+            shape = tuple(available[name])
+            if shape != tuple(spec.shape) and shape not in spec.alt_shapes:
+                wrong.append((name, shape, tuple(spec.shape)))
+    if missing or unexpected or wrong:
+        lines = [f"{where} does not match the model:"]
+        if missing:
+            lines.append(f"  missing tensors ({len(missing)}): " + ", ".join(missing))
+        if unexpected:
+            lines.append(f"  unexpected tensors ({len(unexpected)}): " + ", ".join(unexpected))
+        if wrong:
+            lines.append(
+                f"  wrong shapes ({len(wrong)}): "
+                + ", ".join(f"{n} is {list(got)}, expected {list(exp)}" for n, got, exp in wrong)
+            )
+        raise WeightsError("\n".join(lines), missing, unexpected, wrong)
+    return ignored
+
+
+_STORED_AS = {
+    torch.bfloat16: torch.bfloat16,
+    torch.float16: torch.bfloat16,
+    torch.float32: torch.float32,
+    torch.float64: torch.float32,
+    torch.int32: torch.int32,
+    torch.int64: torch.int32,
+}
+
+
+class CheckedWeights:
+    """A safetensors file whose names and shapes were checked; `get(name)` reads one tensor."""
+
+    def __init__(self, model_dir: str, specs: Iterable[ParamSpec], ignorable: Iterable[str] = ()):
+        self.path = os.path.join(model_dir, "model.safetensors")
+        self.file = SafetensorsFile(self.path)
+        available = {n: self.file.shape(n) for n in self.file.names()}
+        self.ignored = check_names_and_shapes(available, specs, ignorable, where=self.path)
+
+    def get(self, name: str) -> torch.Tensor:
+        t = self.file.read(name)
+        target = _STORED_AS[t.dtype]
+        if t.dtype == torch.int64 and t.numel():
+            if int(t.max()) > 2**31 - 1 or int(t.min()) < -(2**31):
+                raise WeightsError(f"{self.path}: integer tensor '{name}' does not fit int32")
+        return t if t.dtype == target else t.to(target)
+
+    def close(self) -> None:
+        self.file.close()
