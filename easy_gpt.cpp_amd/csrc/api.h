@@ -1,0 +1,37 @@
+// C entry points of the gfx950 kernel library.  Every function launches on `stream`
+// and returns 0, or one of the EGPT_* error codes without launching anything.
+// dtype: 0 = float32, 1 = bfloat16 (activations, weights and caches of one call share it).
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* egpt_error_string(int code);
+int egpt_abi_version(void);
+
+int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, int hidden, int vocab, int dtype,
+               void* stream);
+// h += delta (delta may be null); out = rmsnorm(h) * weight.  rows == null: every row, h written back.
+// rows != null: only the listed rows, gathered into out[n_rows], h untouched.
+int egpt_add_rmsnorm(float* h, const void* delta, const int32_t* rows, const void* weight, float eps, void* out,
+                     int n_rows, int hidden, int dtype, void* stream);
+int egpt_swiglu(const void* gate_up, void* out, int n_tokens, int inter, int dtype, void* stream);
+int egpt_qkv_rope_store(void* qkv, const void* bias, const int32_t* positions, const float* inv_freq, int rotary_dim,
+                        const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int hd,
+                        int page_size, int dtype, void* stream);
+// out = x w^T + bias; x [m,k], w [n,k], out [m,n]; out_f32 != 0 writes float32 whatever dtype is.
+int egpt_linear(const void* x, const void* w, const void* bias, void* out, int m, int n, int k, int dtype,
+                int out_f32, void* stream);
+int egpt_paged_attention(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                         const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
+                         const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int hd, int page_size,
+                         float scale, int window, int dtype, void* stream);
+int egpt_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
+int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
+                const float* uniform, int32_t* out, int n_rows, int vocab, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

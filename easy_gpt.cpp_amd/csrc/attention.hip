@@ -1,0 +1,125 @@
+// Softmax attention over the paged cache for a ragged batch: prompt portions and single decoded
+// tokens in one launch.
+//
+// Query i of request b stands at position p = kv_len[b] - q_len[b] + i and reads keys j <= p
+// (causal key limit as /root/reference/src/cuda/ops/self_attn_detail.cuh:695-751), and j > p - window
+// when a window is set.  score = (q . k) * scale, online softmax with float32 running maximum, sum and
+// accumulator (/root/reference/src/cuda/ops/self_attn_detail.cuh:299-383); query head h reads kv head
+// h / (nq / nkv) (:669).  Keys and values lie in pages [page][kv head][offset][hd] and are found
+// through the request's block table; nothing beyond kv_len is ever read, so pages need no clearing.
+#include "api.h"
+#include "common.h"
+
+namespace egpt {
+
+constexpr int kMaxHeadDim = 256;
+
+__device__ __forceinline__ int find_request(const int32_t* q_start, int n_seqs, int t) {
+    int lo = 0, hi = n_seqs - 1;  // last b with q_start[b] <= t
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) / 2;
+        if (q_start[mid] <= t) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+// One wavefront per (token, query head).  Keys are taken 64 at a time: each lane scores one key, the
+// wave agrees on the new maximum, then each lane owns head features lane, lane+64, ... of the output.
+template <typename T>
+__global__ __launch_bounds__(64) void paged_attention_generic_kernel(
+    const T* __restrict__ qkv, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int nq, int nkv, int hd,
+    int page_size, float scale, int window) {
+    __shared__ float q_s[kMaxHeadDim];
+    __shared__ float p_s[kWave];
+    __shared__ long v_off_s[kWave];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int b = find_request(q_start, n_seqs, t);
+    const int i = t - q_start[b];
+    const int p = kv_len[b] - q_len[b] + i;
+    const int hi = p + 1;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const int kvh = h / (nq / nkv);
+    const int row_width = (nq + 2 * nkv) * hd;
+    const T* q = qkv + static_cast<size_t>(t) * row_width + h * hd;
+    for (int d = lane; d < hd; d += kWave) q_s[d] = to_float(q[d]);
+    __syncthreads();
+    const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+    constexpr int kMaxOwn = kMaxHeadDim / kWave;
+    float acc[kMaxOwn] = {};
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int c = lo; c < hi; c += kWave) {
+        const int j = c + lane;
+        float s = -INFINITY;
+        long off = 0;
+        if (j < hi) {
+            const long page = table[j / page_size];
+            off = ((page * nkv + kvh) * page_size + (j % page_size)) * hd;
+            const T* kr = k_cache + off;
+            float dot = 0.f;
+            for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float(kr[d]), dot);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m_run, wave_max(s));   // finite: key c is always visible
+        const float pj = j < hi ? expf(s - m_new) : 0.f;
+        const float alpha = expf(m_run - m_new);          // exp(-inf) = 0 on the first chunk
+        l_run = l_run * alpha + wave_sum(pj);
+        m_run = m_new;
+        p_s[lane] = pj;
+        v_off_s[lane] = off;
+        __syncthreads();
+        const int n_valid = min(kWave, hi - c);
+#pragma unroll
+        for (int r = 0; r < kMaxOwn; ++r) {
+            const int d = lane + r * kWave;
+            if (d < hd) {
+                float a = acc[r] * alpha;
+                for (int jj = 0; jj < n_valid; ++jj) a = fmaf(p_s[jj], to_float(v_cache[v_off_s[jj] + d]), a);
+                acc[r] = a;
+            }
+        }
+        __syncthreads();
+    }
+    T* o = out + static_cast<size_t>(t) * nq * hd + h * hd;
+    const float inv_l = 1.0f / l_run;
+#pragma unroll
+    for (int r = 0; r < kMaxOwn; ++r) {
+        const int d = lane + r * kWave;
+        if (d < hd) o[d] = from_float<T>(acc[r] * inv_l);
+    }
+}
+
+}  // namespace egpt
+
+using namespace egpt;
+
+extern "C" int egpt_paged_attention(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                                    const int32_t* block_table, int table_width, const int32_t* q_start,
+                                    const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq,
+                                    int nkv, int hd, int page_size, float scale, int window, int dtype,
+                                    void* stream) {
+    if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
+        return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || hd <= 0 || page_size <= 0 ||
+        table_width <= 0 || window < 0)
+        return EGPT_BAD_ARGUMENT;
+    if (hd > kMaxHeadDim || nq > 65535) return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid(n_tokens, nq);
+    if (dtype == 0)
+        paged_attention_generic_kernel<float><<<grid, kWave, 0, s>>>(
+            static_cast<const float*>(qkv), static_cast<float*>(out), static_cast<const float*>(k_cache),
+            static_cast<const float*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
+            hd, page_size, scale, window);
+    else if (dtype == 1)
+        paged_attention_generic_kernel<bf16_t><<<grid, kWave, 0, s>>>(
+            static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
+            static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
+            hd, page_size, scale, window);
+    else
+        return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}

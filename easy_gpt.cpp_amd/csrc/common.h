@@ -1,0 +1,80 @@
+// Shared device helpers for the gfx950 kernels: element types, conversions, reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace egpt {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// bfloat16 as raw bits; arithmetic is always done in float.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(static_cast<uint32_t>(v.bits) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float v);
+template <>
+__device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  `scratch` holds >= 16 floats.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int n_waves = (blockDim.x + kWave - 1) / kWave;
+    v = wave_sum(v);
+    __syncthreads();  // scratch may still be read from an earlier call
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < n_waves; ++w) total += scratch[w];
+    return total;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int n_waves = (blockDim.x + kWave - 1) / kWave;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float m = scratch[0];
+    for (int w = 1; w < n_waves; ++w) m = fmaxf(m, scratch[w]);
+    return m;
+}
+
+}  // namespace egpt
+
+// Error codes returned by every entry point (0 = launched).
+#define EGPT_OK 0
+#define EGPT_BAD_ARGUMENT 1
+#define EGPT_UNSUPPORTED_SIZE 2
+#define EGPT_LAUNCH_FAILED 3
+
+#define EGPT_CHECK_LAUNCH()                                   \
+    do {                                                      \
+        hipError_t e_ = hipGetLastError();                    \
+        if (e_ != hipSuccess) return EGPT_LAUNCH_FAILED;      \
+    } while (0)

@@ -1,0 +1,202 @@
+// Embedding gather, residual-add + RMSNorm, SwiGLU, and the QKV epilogue
+// (bias + rotary position encoding + store of keys and values into cache pages).
+#include "api.h"
+#include "common.h"
+
+namespace egpt {
+
+// ----------------------------------------------------------------------------- embedding
+// x[t, :] = E[id_t, :]   (/root/reference/src/models/embedding.cpp:54-76); output float32.
+template <typename T>
+__global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+                             int hidden, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are range-checked on the host; never read outside
+    const T* row = table + static_cast<size_t>(id) * hidden;
+    float* o = out + static_cast<size_t>(t) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]);
+}
+
+// ----------------------------------------------------------------------------- add + RMSNorm
+// ss = sum x^2 (float32), inv = 1/sqrt(ss/H + eps), y = x * inv * w
+// (/root/reference/src/models/norm.cpp:47-59, /root/reference/src/cuda/ops/self_attn_detail.cuh:385-418).
+// The residual addition h += delta happens here too, in float32.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                   const int32_t* __restrict__ rows, const T* __restrict__ weight, float eps,
+                                   T* __restrict__ out, int hidden) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+    float* hrow = h + src * hidden;
+    const T* drow = delta ? delta + src * hidden : nullptr;
+    const bool write_back = (rows == nullptr) && (delta != nullptr);
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float v = hrow[j];
+        if (drow) v += to_float(drow[j]);
+        if (write_back) hrow[j] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
+    T* orow = out + static_cast<size_t>(r) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
+        float v = hrow[j];                       // already updated when written back
+        if (drow && !write_back) v += to_float(drow[j]);
+        orow[j] = from_float<T>(v * inv * to_float(weight[j]));
+    }
+}
+
+// ----------------------------------------------------------------------------- SwiGLU
+// out = up * gate / (1 + exp(-gate))   (/root/reference/src/cuda/ops/mlp.cu:152-162); [gate | up] per row.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int n_tokens, int inter) {
+    const size_t total = static_cast<size_t>(n_tokens) * inter;
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t t = i / inter, j = i % inter;
+        const float g = to_float(gate_up[t * 2 * inter + j]);
+        const float u = to_float(gate_up[t * 2 * inter + inter + j]);
+        out[i] = from_float<T>(u * (g / (1.0f + expf(-g))));
+    }
+}
+
+// ----------------------------------------------------------------------------- QKV epilogue
+// For each token: add bias; rotate the first rotary_dim features of every query and key head, pairs
+// (i, i + rotary_dim/2), angle = float(position) * inv_freq[i], cos/sin in float32
+// (/root/reference/src/ops.cpp:404-420, /root/reference/src/cuda/ops/self_attn_detail.cuh:512-541);
+// write the result back in place and store keys and values at their slot of the paged cache
+// [page][kv head][offset][hd].
+template <typename T>
+__global__ void qkv_rope_store_kernel(T* __restrict__ qkv, const T* __restrict__ bias,
+                                      const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                      int rotary_dim, const int32_t* __restrict__ slots, T* __restrict__ k_cache,
+                                      T* __restrict__ v_cache, int nq, int nkv, int hd, int page_size) {
+    const int t = blockIdx.x;
+    const int n_heads = nq + 2 * nkv;
+    T* row = qkv + static_cast<size_t>(t) * n_heads * hd;
+    const float pos = static_cast<float>(positions[t]);
+    const int half = rotary_dim / 2;
+    long slot = slots ? slots[t] : -1;
+    const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    for (int item = threadIdx.x; item < n_heads * hd; item += blockDim.x) {
+        const int head = item / hd, d = item % hd;
+        const bool rotated = head < nq + nkv && d < rotary_dim;
+        if (rotated && d >= half) continue;  // done by its partner
+        float a = to_float(row[item]) + (bias ? to_float(bias[item]) : 0.f);
+        float b = 0.f;
+        if (rotated) {
+            b = to_float(row[item + half]) + (bias ? to_float(bias[item + half]) : 0.f);
+            float s, c;
+            sincosf(pos * inv_freq[d], &s, &c);
+            const float ra = a * c - b * s, rb = a * s + b * c;
+            a = ra;
+            b = rb;
+        }
+        const T ta = from_float<T>(a), tb = from_float<T>(b);
+        row[item] = ta;
+        if (rotated) row[item + half] = tb;
+        if (slot >= 0 && head >= nq) {
+            const bool is_k = head < nq + nkv;
+            const int kvh = is_k ? head - nq : head - nq - nkv;
+            T* dst = (is_k ? k_cache : v_cache) + ((page * nkv + kvh) * page_size + off) * hd;
+            dst[d] = ta;
+            if (rotated) dst[d + half] = tb;
+        }
+    }
+}
+
+}  // namespace egpt
+
+using namespace egpt;
+
+extern "C" int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, int hidden, int vocab,
+                          int dtype, void* stream) {
+    if (!ids || !table || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0) return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        embed_kernel<float><<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), out, hidden, vocab);
+    else if (dtype == 1)
+        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), out, hidden, vocab);
+    else
+        return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_add_rmsnorm(float* h, const void* delta, const int32_t* rows, const void* weight, float eps,
+                                void* out, int n_rows, int hidden, int dtype, void* stream) {
+    if (!h || !weight || !out || n_rows < 0 || hidden <= 0) return EGPT_BAD_ARGUMENT;
+    if (n_rows == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int threads = hidden >= 2048 ? 512 : 256;
+    if (dtype == 0)
+        add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, static_cast<const float*>(delta), rows,
+                                                             static_cast<const float*>(weight), eps,
+                                                             static_cast<float*>(out), hidden);
+    else if (dtype == 1)
+        add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(h, static_cast<const bf16_t*>(delta), rows,
+                                                              static_cast<const bf16_t*>(weight), eps,
+                                                              static_cast<bf16_t*>(out), hidden);
+    else
+        return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_swiglu(const void* gate_up, void* out, int n_tokens, int inter, int dtype, void* stream) {
+    if (!gate_up || !out || n_tokens < 0 || inter <= 0) return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t total = static_cast<size_t>(n_tokens) * inter;
+    const int blocks = static_cast<int>(total / 256 + 1 > 8192 ? 8192 : total / 256 + 1);
+    if (dtype == 0)
+        swiglu_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out),
+                                                    n_tokens, inter);
+    else if (dtype == 1)
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
+                                                     n_tokens, inter);
+    else
+        return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" int egpt_qkv_rope_store(void* qkv, const void* bias, const int32_t* positions, const float* inv_freq,
+                                   int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens,
+                                   int nq, int nkv, int hd, int page_size, int dtype, void* stream) {
+    if (!qkv || !positions || n_tokens < 0 || nq <= 0 || nkv <= 0 || hd <= 0 || page_size <= 0)
+        return EGPT_BAD_ARGUMENT;
+    if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim % 2) != 0 || (rotary_dim > 0 && !inv_freq))
+        return EGPT_BAD_ARGUMENT;
+    if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        qkv_rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(
+            static_cast<float*>(qkv), static_cast<const float*>(bias), positions, inv_freq, rotary_dim, slots,
+            static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq, nkv, hd, page_size);
+    else if (dtype == 1)
+        qkv_rope_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(
+            static_cast<bf16_t*>(qkv), static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots,
+            static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
+    else
+        return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+extern "C" const char* egpt_error_string(int code) {
+    switch (code) {
+        case EGPT_OK: return "ok";
+        case EGPT_BAD_ARGUMENT: return "bad argument (null pointer, negative size or unknown dtype)";
+        case EGPT_UNSUPPORTED_SIZE: return "size not supported by this kernel";
+        case EGPT_LAUNCH_FAILED: return "kernel launch failed";
+        default: return "unknown error";
+    }
+}
+
+extern "C" int egpt_abi_version(void) { return 1; }

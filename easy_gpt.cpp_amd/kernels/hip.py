@@ -1,0 +1,206 @@
+"""ctypes binding of the gfx950 kernel library: shape and dtype checks on the host, then the launch.
+
+Every operand is checked against what the kernel and its grid assume before anything is
+launched; a mismatch raises here instead of faulting on the device.  Launches go to torch's
+current stream, so they order with torch's own work and can be captured into a graph.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import KernelsUnavailable
+
+_F32, _BF16, _I32 = torch.float32, torch.bfloat16, torch.int32
+_DT = {_F32: 0, _BF16: 1}
+
+
+def _load_library() -> ctypes.CDLL:
+    if not torch.cuda.is_available():
+        raise KernelsUnavailable(
+            "no GPU is visible to torch; this engine has no CPU path (its kernels are HIP code for gfx950)"
+        )
+    from ..csrc import build
+
+    try:
+        path = build.ensure_built()
+        lib = ctypes.CDLL(path)
+    except (build.BuildError, OSError) as e:
+        raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
+    if lib.egpt_abi_version() != 1:
+        raise KernelsUnavailable(f"{path} has an unexpected ABI version")
+    return lib
+
+
+class HipKernels:
+    name = "hip-gfx950"
+
+    def __init__(self):
+        lib = _load_library()
+        self.lib = lib
+        vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+        lib.egpt_error_string.restype = ctypes.c_char_p
+        lib.egpt_error_string.argtypes = [i]
+        sigs = {
+            "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
+            "egpt_add_rmsnorm": [vp, vp, vp, vp, f, vp, i, i, i, vp],
+            "egpt_swiglu": [vp, vp, i, i, i, vp],
+            "egpt_qkv_rope_store": [vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
+            "egpt_argmax": [vp, vp, i, i, vp],
+            "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
+        }
+        for name, argtypes in sigs.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = i
+
+    # ------------------------------------------------------------------ helpers
+    @staticmethod
+    def _stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def _run(self, name: str, *args) -> None:
+        code = getattr(self.lib, name)(*args)
+        if code != 0:
+            raise RuntimeError(f"{name}: {self.lib.egpt_error_string(code).decode()}")
+
+    @staticmethod
+    def _ptr(t: torch.Tensor | None):
+        return None if t is None else t.data_ptr()
+
+    @staticmethod
+    def _need(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise TypeError(f"{name} must be a tensor on the GPU")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+    @staticmethod
+    def _act(t: torch.Tensor, name: str) -> int:
+        if t.dtype not in _DT:
+            raise TypeError(f"{name} must be float32 or bfloat16, got {t.dtype}")
+        return _DT[t.dtype]
+
+    # ------------------------------------------------------------------ kernels
+    def embed(self, token_ids, table, out):
+        dt = self._act(table, "table")
+        v, h = table.shape
+        t = token_ids.shape[0]
+        self._need(token_ids, "token_ids", _I32, (t,))
+        self._need(table, "table")
+        self._need(out, "out", _F32, (t, h))
+        self._run("egpt_embed", token_ids.data_ptr(), table.data_ptr(), out.data_ptr(), t, h, v, dt, self._stream())
+
+    def add_rmsnorm(self, h, delta, weight, eps, out):
+        t, hid = h.shape
+        dt = self._act(out, "out")
+        self._need(h, "h", _F32)
+        self._need(weight, "weight", out.dtype, (hid,))
+        self._need(out, "out", None, (t, hid))
+        if delta is not None:
+            self._need(delta, "delta", out.dtype, (t, hid))
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), None, weight.data_ptr(), float(eps),
+                  out.data_ptr(), t, hid, dt, self._stream())
+
+    def rows_add_rmsnorm(self, h, delta, rows, weight, eps, out):
+        t, hid = h.shape
+        r = rows.shape[0]
+        dt = self._act(out, "out")
+        self._need(h, "h", _F32)
+        self._need(rows, "rows", _I32, (r,))
+        self._need(weight, "weight", out.dtype, (hid,))
+        self._need(out, "out", None, (r, hid))
+        if delta is not None:
+            self._need(delta, "delta", out.dtype, (t, hid))
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), rows.data_ptr(), weight.data_ptr(), float(eps),
+                  out.data_ptr(), r, hid, dt, self._stream())
+
+    def linear(self, x, w, bias, out):
+        m, k = x.shape
+        n = w.shape[0]
+        dt = self._act(x, "x")
+        self._need(x, "x")
+        self._need(w, "w", x.dtype, (n, k))
+        if bias is not None:
+            self._need(bias, "bias", x.dtype, (n,))
+        if out.dtype not in (x.dtype, _F32):
+            raise TypeError(f"out must be {x.dtype} or float32, got {out.dtype}")
+        self._need(out, "out", None, (m, n))
+        self._run("egpt_linear", x.data_ptr(), w.data_ptr(), self._ptr(bias), out.data_ptr(), m, n, k, dt,
+                  1 if out.dtype == _F32 else 0, self._stream())
+
+    def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
+                       page_size):
+        t = qkv.shape[0]
+        width = (nq + 2 * nkv) * hd
+        dt = self._act(qkv, "qkv")
+        self._need(qkv, "qkv", None, (t, width))
+        self._need(positions, "positions", _I32, (t,))
+        if bias is not None:
+            self._need(bias, "bias", qkv.dtype, (width,))
+        if rotary_dim:
+            if rotary_dim % 2 or rotary_dim > hd:
+                raise ValueError(f"rotary_dim {rotary_dim} must be even and <= head size {hd}")
+            self._need(inv_freq, "inv_freq", _F32, (rotary_dim // 2,))
+        if slots is not None:
+            self._need(slots, "slots", _I32, (t,))
+            for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+                self._need(c, name, qkv.dtype)
+                if c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, hd):
+                    raise ValueError(f"{name} must be [pages, {nkv}, {page_size}, {hd}], got {tuple(c.shape)}")
+        self._run("egpt_qkv_rope_store", qkv.data_ptr(), self._ptr(bias), positions.data_ptr(),
+                  self._ptr(inv_freq) if rotary_dim else None, int(rotary_dim), self._ptr(slots),
+                  self._ptr(k_cache), self._ptr(v_cache), t, nq, nkv, hd, page_size, dt, self._stream())
+
+    def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd, page_size,
+                        scale, window, max_q_len, max_kv_len):
+        t = qkv.shape[0]
+        b, width = block_table.shape
+        dt = self._act(qkv, "qkv")
+        self._need(qkv, "qkv", None, (t, (nq + 2 * nkv) * hd))
+        self._need(out, "out", qkv.dtype, (t, nq * hd))
+        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            self._need(c, name, qkv.dtype)
+            if c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, hd):
+                raise ValueError(f"{name} must be [pages, {nkv}, {page_size}, {hd}], got {tuple(c.shape)}")
+        self._need(block_table, "block_table", _I32)
+        for name, v in (("q_start", q_start), ("q_len", q_len), ("kv_len", kv_len)):
+            self._need(v, name, _I32, (b,))
+        if max_kv_len > width * page_size:
+            raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
+        if hd > 256:
+            raise ValueError(f"head size {hd} is not supported by the attention kernels (at most 256)")
+        self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                  block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
+                  nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())
+
+    def swiglu(self, gate_up, out):
+        t, inter = out.shape
+        dt = self._act(out, "out")
+        self._need(gate_up, "gate_up", out.dtype, (t, 2 * inter))
+        self._need(out, "out")
+        self._run("egpt_swiglu", gate_up.data_ptr(), out.data_ptr(), t, inter, dt, self._stream())
+
+    def argmax(self, logits, out):
+        r, v = logits.shape
+        self._need(logits, "logits", _F32)
+        self._need(out, "out", _I32, (r,))
+        self._run("egpt_argmax", logits.data_ptr(), out.data_ptr(), r, v, self._stream())
+
+    def sample(self, logits, temperature, top_k, top_p, uniform, out):
+        r, v = logits.shape
+        self._need(logits, "logits", _F32)
+        self._need(temperature, "temperature", _F32, (r,))
+        self._need(top_k, "top_k", _I32, (r,))
+        self._need(top_p, "top_p", _F32, (r,))
+        self._need(uniform, "uniform", _F32, (r,))
+        self._need(out, "out", _I32, (r,))
+        self._run("egpt_sample", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+                  uniform.data_ptr(), out.data_ptr(), r, v, self._stream())
