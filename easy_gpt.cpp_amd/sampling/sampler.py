@@ -1,0 +1,80 @@
+"""Sampling of next tokens from float32 logits, on the device.
+
+Options and their meaning are the reference's (/root/reference/src/sampler.cpp:39-105,
+defaults from /root/reference/include/cli_options.hpp:9-24): greedy (or temperature <= 0)
+takes the first maximum; otherwise probabilities are raised to 1/T (softmax(logits/T)),
+cut to the top_k most likely (0 disables), then to the smallest set whose mass reaches
+top_p (1 disables), and one uniform number picks a token from what is left.
+
+The reference draws from one shared mt19937 in batch order, so a request's tokens
+depend on its neighbours.  Here the uniform number of a request's n-th token is a
+function of (seed, request serial, n) alone, so batching changes nothing.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from .. import kernels
+
+
+@dataclass(frozen=True)
+class SamplingParams:
+    temperature: float = 0.8
+    top_p: float = 0.95
+    top_k: int = 20
+    greedy: bool = False
+    seed: int = 42
+
+    def __post_init__(self):
+        if not self.greedy and not self.temperature > 0:
+            raise ValueError("Temperature must be greater than 0")
+        if not 0.0 < self.top_p <= 1.0:
+            raise ValueError("Top-p must be in (0, 1]")
+        if self.top_k < 0:
+            raise ValueError("Top-k must be >= 0")
+        if self.seed < 0:
+            raise ValueError("Seed must be >= 0")
+
+
+_MASK = (1 << 64) - 1
+
+
+def _mix(z: int) -> int:
+    """splitmix64 finaliser"""
+    z = (z + 0x9E3779B97F4A7C15) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform_for(seed: int, serial: int, n: int) -> float:
+    """A number in [0, 1) for the n-th token of request `serial` under `seed`."""
+    z = _mix(_mix(_mix(seed) ^ serial) ^ n)
+    return (z >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def sample(self, logits: torch.Tensor, params: list[SamplingParams], serials: list[int], counts: list[int]) -> list[int]:
+        """One token per row of `logits` [R, V]; row r belongs to request serials[r], which has
+        produced counts[r] tokens so far."""
+        r = logits.shape[0]
+        if not (len(params) == len(serials) == len(counts) == r):
+            raise ValueError("one SamplingParams, serial and count per row of logits is needed")
+        out = torch.empty(r, dtype=torch.int32, device=logits.device)
+        k = kernels.backend()
+        if all(p.greedy for p in params):
+            k.argmax(logits, out)
+        else:
+            host = torch.tensor(
+                [[0.0 if p.greedy else p.temperature, p.top_p, uniform_for(p.seed, s, n)]
+                 for p, s, n in zip(params, serials, counts)], dtype=torch.float32)
+            topk = torch.tensor([p.top_k for p in params], dtype=torch.int32)
+            host = host.to(logits.device)
+            k.sample(logits, host[:, 0].contiguous(), topk.to(logits.device), host[:, 1].contiguous(),
+                     host[:, 2].contiguous(), out)
+        return out.tolist()

@@ -1,0 +1,324 @@
+"""Each HIP kernel alone against a plain float64 reference of the same operation, at sizes other than
+the tiny models' (widths and vocabularies that are no power of two, head sizes in steps of 16, odd
+numbers of heads and groups)."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, scale=1.0):
+    return (3e-6 if dtype == torch.float32 else 1.6e-2) * scale
+
+
+@pytest.fixture(scope="module")
+def k():
+    from easy_gpt.cpp_amd import kernels
+
+    kernels.use_backend(None)
+    b = kernels.backend()
+    assert b.name == "hip-gfx950"
+    return b
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(k, dtype):
+    table = rnd(301, 72, dtype=dtype)
+    ids = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 72, dtype=torch.float32, device=DEV)
+    k.embed(ids, table, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,eps", [(72, 1e-6), (896, 1e-5), (3000, 1e-2)])
+def test_add_rmsnorm(k, dtype, hidden, eps):
+    h = rnd(7, hidden, seed=1, scale=2.0)
+    delta = rnd(7, hidden, dtype=dtype, seed=2)
+    w = (1 + rnd(hidden, seed=3, scale=0.1)).to(dtype)
+    h0 = h.clone()
+    out = torch.empty(7, hidden, dtype=dtype, device=DEV)
+    k.add_rmsnorm(h, delta, w, eps, out)
+    summed = h0 + delta.float()                                   # the residual sum is made in float32
+    assert torch.equal(h, summed)
+    ref = plain.rms_norm(summed.double().cpu(), w.double().cpu(), eps)
+    assert float((out.double().cpu() - ref).abs().max()) <= tol(dtype, float(ref.abs().max()))
+    # without delta h is untouched
+    h1 = h.clone()
+    k.add_rmsnorm(h, None, w, eps, out)
+    assert torch.equal(h, h1)
+    # rows variant: gathers, adds, does not write back
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, hidden, dtype=dtype, device=DEV)
+    k.rows_add_rmsnorm(h, delta, rows, w, eps, out3)
+    assert torch.equal(h, h1)
+    ref3 = plain.rms_norm((h1 + delta.float())[rows.long()].double().cpu(), w.double().cpu(), eps)
+    assert float((out3.double().cpu() - ref3).abs().max()) <= tol(dtype, float(ref3.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,kk", [(1, 75, 100), (37, 130, 96), (70, 1000, 200), (5, 64, 4864), (130, 33, 17)])
+def test_linear(k, dtype, m, n, kk):
+    x, w, b = rnd(m, kk, dtype=dtype, seed=1), rnd(n, kk, dtype=dtype, seed=2, scale=0.1), rnd(n, dtype=dtype, seed=3)
+    ref = plain.linear(x.double().cpu(), w.double().cpu(), b.double().cpu())
+    for out_dtype in {dtype, torch.float32}:
+        out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+        k.linear(x, w, b, out)
+        t = 3e-6 if out_dtype == torch.float32 else 1.6e-2
+        assert float((out.double().cpu() - ref).abs().max()) <= t * float(ref.abs().max())
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    k.linear(x, w, None, out)
+    assert float((out.double().cpu() - (ref - b.double().cpu())).abs().max()) <= 3e-6 * float(ref.abs().max())
+
+
+def test_linear_vector_of_the_reference(k):
+    # /root/reference/test/matmul_3d_test.cpp:60-87
+    x = torch.tensor([[1.0, 2, 3], [4, 5, 6]], device=DEV)
+    w = torch.tensor([[1.0, 0, -1], [2, 3, 4]], device=DEV)
+    b = torch.tensor([0.5, -1.0], device=DEV)
+    out = torch.empty(2, 2, device=DEV)
+    k.linear(x, w, b, out)
+    assert torch.equal(out.cpu(), torch.tensor([[-1.5, 19.0], [-1.5, 46.0]]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(k, dtype):
+    gu = rnd(9, 2 * 211, dtype=dtype, scale=3.0)
+    out = torch.empty(9, 211, dtype=dtype, device=DEV)
+    k.swiglu(gu, out)
+    g, u = gu[:, :211].double().cpu(), gu[:, 211:].double().cpu()
+    ref = u * g / (1 + torch.exp(-g))
+    assert float((out.double().cpu() - ref).abs().max()) <= tol(dtype, float(ref.abs().max()))
+    z = torch.zeros(2, 2 * 16, dtype=dtype, device=DEV)
+    z[:, 16:] = 5.0
+    o = torch.ones(2, 16, dtype=dtype, device=DEV)
+    k.swiglu(z, o)
+    assert torch.equal(o, torch.zeros_like(o))                    # silu(0) = 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,rd,theta", [(6, 3, 48, 48, 1e4), (5, 1, 80, 80, 1e6), (4, 4, 32, 16, 5e5)])
+def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta):
+    t, ps, pages = 11, 4, 9
+    qkv = rnd(t, (nq + 2 * nkv) * hd, dtype=dtype, seed=1)
+    bias = rnd((nq + 2 * nkv) * hd, dtype=dtype, seed=2)
+    positions = torch.tensor([0, 1, 2, 3, 250, 251, 7, 8, 9, 4000, 31], dtype=torch.int32, device=DEV)
+    inv = torch.pow(torch.tensor(theta, dtype=torch.float32), -2.0 * torch.arange(rd // 2, dtype=torch.float32) / rd).to(DEV)
+    perm = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(3))[:t]
+    slots = perm.to(torch.int32).to(DEV)
+    kc = torch.full((pages, nkv, ps, hd), 77.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, nkv, ps, hd), 77.0, dtype=dtype, device=DEV)
+    x = (qkv.double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
+    k.qkv_rope_store(qkv, bias, positions, inv, rd, slots, kc, vc, nq, nkv, hd, ps)
+    ang = (positions.cpu().float()[:, None] * inv.cpu()[None, :]).double()
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    ref = x.clone()
+    x1, x2 = x[:, : nq + nkv, : rd // 2], x[:, : nq + nkv, rd // 2 : rd]
+    ref[:, : nq + nkv, : rd // 2] = x1 * cos - x2 * sin
+    ref[:, : nq + nkv, rd // 2 : rd] = x1 * sin + x2 * cos
+    got = qkv.double().cpu().view(t, nq + 2 * nkv, hd)
+    assert float((got - ref).abs().max()) <= tol(dtype, float(ref.abs().max()))
+    written = torch.zeros(pages * ps, dtype=torch.bool)
+    for i in range(t):
+        p, o = int(perm[i]) // ps, int(perm[i]) % ps
+        written[int(perm[i])] = True
+        assert torch.equal(kc[p, :, o, :], qkv.view(t, -1, hd)[i, nq : nq + nkv])
+        assert torch.equal(vc[p, :, o, :], qkv.view(t, -1, hd)[i, nq + nkv :])
+    untouched = kc.permute(0, 2, 1, 3).reshape(pages * ps, -1)[~written]
+    assert torch.all(untouched == 77.0)                          # nothing else was written
+
+
+def paged_reference(q, keys, vals, nq, nkv, scale, window):
+    """q [n, nq, hd] are the last n positions of a sequence whose keys/values [kv, nkv, hd] are given."""
+    n, kv = q.shape[0], keys.shape[0]
+    out = torch.empty_like(q)
+    for i in range(n):
+        p = kv - n + i
+        lo = max(0, p - window + 1) if window else 0
+        for h in range(nq):
+            kh = h // (nq // nkv)
+            s = (keys[lo : p + 1, kh] @ q[i, h]) * scale
+            out[i, h] = torch.softmax(s, 0) @ vals[lo : p + 1, kh]
+    return out
+
+
+def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
+    """seqs: list of (q_len, kv_len).  Returns everything paged_attention needs, with pages handed out in a
+    shuffled order and unused slots filled with huge values (reading one would wreck the result)."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum(-(-kv // ps) for _, kv in seqs) + extra_pages
+    order = torch.randperm(n_pages, generator=g).tolist()
+    kc = torch.full((n_pages, nkv, ps, hd), 1e4, dtype=dtype)
+    vc = torch.full((n_pages, nkv, ps, hd), -1e4, dtype=dtype)
+    width = max(-(-kv // ps) for _, kv in seqs)
+    table = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    keys, vals = [], []
+    for b, (_, kv) in enumerate(seqs):
+        kk = torch.randn(kv, nkv, hd, generator=g).to(dtype)
+        vv = torch.randn(kv, nkv, hd, generator=g).to(dtype)
+        keys.append(kk)
+        vals.append(vv)
+        for j in range(kv):
+            if j % ps == 0:
+                table[b, j // ps] = order.pop()
+            pg = int(table[b, j // ps])
+            kc[pg, :, j % ps, :] = kk[j]
+            vc[pg, :, j % ps, :] = vv[j]
+    return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
+
+
+def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0):
+    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed)
+    t = sum(q for q, _ in seqs)
+    g = torch.Generator().manual_seed(seed + 100)
+    qkv = (torch.randn(t, (nq + 2 * nkv) * hd, generator=g) * q_scale).to(dtype).to(DEV)
+    q_len = torch.tensor([q for q, _ in seqs], dtype=torch.int32)
+    q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
+    kv_len = torch.tensor([kv for _, kv in seqs], dtype=torch.int32)
+    out = torch.empty(t, nq * hd, dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    k.paged_attention(qkv, out, kc, vc, table, q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV), nq, nkv, hd, ps,
+                      scale, window, int(q_len.max()), int(kv_len.max()))
+    got = out.double().cpu().view(t, nq, hd)
+    worst = 0.0
+    for b, (n, kv) in enumerate(seqs):
+        s = int(q_start[b])
+        q = qkv[s : s + n].double().cpu().view(n, nq + 2 * nkv, hd)[:, :nq]
+        ref = paged_reference(q, keys[b].double(), vals[b].double(), nq, nkv, scale, window)
+        worst = max(worst, float((got[s : s + n] - ref).abs().max()))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(6, 3, 48, 4), (7, 1, 64, 16), (4, 4, 16, 5), (10, 5, 80, 16), (2, 1, 128, 64),
+                                           (3, 3, 256, 16)])
+def test_paged_attention_ragged_batch(k, dtype, nq, nkv, hd, ps):
+    # prompt portions (with and without a prefix in the cache) beside single decoded tokens
+    seqs = [(1, 1), (9, 9), (1, 130), (7, 71), (2, 64), (1, 65), (33, 33), (3, 200)]
+    err = run_paged(k, seqs, nq, nkv, hd, ps, dtype)
+    assert err <= (2e-6 if dtype == torch.float32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 7, 64, 65])
+def test_paged_attention_window(k, dtype, window):
+    seqs = [(1, 100), (20, 90), (5, 5), (1, window), (1, window + 1), (3, 66)]
+    err = run_paged(k, seqs, 6, 2, 32, 16, dtype, window=window)
+    assert err <= (2e-6 if dtype == torch.float32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_peaked_scores(k, dtype):
+    # large queries make the softmax pick single keys, far ones included: a key skipped or read from the
+    # wrong page then changes the output by O(1) instead of O(1/n)
+    seqs = [(1, 700), (4, 513), (1, 17)]
+    err = run_paged(k, seqs, 4, 2, 64, 16, dtype, q_scale=6.0)
+    assert err <= (2e-5 if dtype == torch.float32 else 4e-2)
+
+
+def test_paged_attention_one_far_key_stands_out(k):
+    # one key among hundreds matches the query; the output must be that key's value, for every position of the key
+    nq = nkv = 1
+    hd, ps, kv = 32, 16, 500
+    for far in (0, 15, 16, 255, 256, 498, 499):
+        kk = torch.zeros(kv, 1, hd)
+        vv = torch.randn(kv, 1, hd, generator=torch.Generator().manual_seed(far))
+        kk[far, 0, 0] = 50.0
+        pages = -(-kv // ps)
+        kc = torch.zeros(pages, 1, ps, hd)
+        vc = torch.zeros(pages, 1, ps, hd)
+        table = torch.randperm(pages, generator=torch.Generator().manual_seed(1)).to(torch.int32)[None, :]
+        for j in range(kv):
+            kc[int(table[0, j // ps]), 0, j % ps] = kk[j, 0]
+            vc[int(table[0, j // ps]), 0, j % ps] = vv[j, 0]
+        qkv = torch.zeros(1, 3 * hd)
+        qkv[0, 0] = 50.0
+        out = torch.empty(1, hd, device=DEV)
+        one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
+        k.paged_attention(qkv.to(DEV), out, kc.to(DEV), vc.to(DEV), table.to(DEV), one(0), one(1), one(kv), 1, 1, hd, ps,
+                          1.0, 0, 1, kv)
+        assert float((out.cpu()[0] - vv[far, 0]).abs().max()) < 1e-5, far
+
+
+def test_paged_attention_refuses_bad_shapes(k):
+    qkv = torch.zeros(2, 3 * 16, device=DEV)
+    out = torch.zeros(2, 16, device=DEV)
+    kc = torch.zeros(2, 1, 4, 16, device=DEV)
+    one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
+    table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="block table"):
+        k.paged_attention(qkv, out, kc, kc, table, one(0), one(2), one(9), 1, 1, 16, 4, 1.0, 0, 2, 9)
+    with pytest.raises(ValueError, match="k_cache"):
+        k.paged_attention(qkv, out, kc[:, :, :2].contiguous(), kc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
+    with pytest.raises(TypeError):
+        k.paged_attention(qkv.half(), out, kc, kc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
+    big = torch.zeros(1, 3 * 512, device=DEV)
+    with pytest.raises(ValueError, match="head size"):
+        k.paged_attention(big, torch.zeros(1, 512, device=DEV), torch.zeros(2, 1, 4, 512, device=DEV),
+                          torch.zeros(2, 1, 4, 512, device=DEV), table, one(0), one(1), one(1), 1, 1, 512, 4, 1.0, 0, 1, 1)
+
+
+def test_argmax_lowest_index_wins(k):
+    logits = rnd(6, 1000, seed=4)
+    logits[2, 5] = logits[2, 900] = 99.0
+    logits[3, 999] = 98.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    k.argmax(logits, out)
+    exp = [plain.greedy(row) for row in logits.cpu()]
+    assert out.tolist() == exp and exp[2] == 5 and exp[3] == 999
+    wide = rnd(2, 151936, seed=5)
+    out2 = torch.empty(2, dtype=torch.int32, device=DEV)
+    k.argmax(wide, out2)
+    assert out2.tolist() == wide.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("vocab", [777, 5000])
+def test_sample_follows_the_reference_s_distribution(k, vocab):
+    rows = 64
+    logits = rnd(rows, vocab, seed=6, scale=2.5)
+    cases = [(0.8, 20, 0.95), (1.0, 0, 1.0), (0.5, 5, 0.5), (2.0, 0, 0.9), (1.3, 50, 1.0), (0.0, 0, 1.0)]
+    g = torch.Generator().manual_seed(9)
+    temp = torch.tensor([cases[i % len(cases)][0] for i in range(rows)])
+    topk = torch.tensor([cases[i % len(cases)][1] for i in range(rows)], dtype=torch.int32)
+    topp = torch.tensor([cases[i % len(cases)][2] for i in range(rows)])
+    u = torch.rand(rows, generator=g)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    k.sample(logits, temp.to(DEV), topk.to(DEV), topp.to(DEV), u.to(DEV), out)
+    out = out.tolist()
+    for r in range(rows):
+        row = logits[r].cpu()
+        if temp[r] <= 0:
+            assert out[r] == plain.greedy(row)
+            continue
+        dist = plain.sampling_distribution(row, float(temp[r]), int(topk[r]), float(topp[r]))
+        assert dist[out[r]] > 0, f"row {r}: token {out[r]} is outside the kept set"
+        cdf = torch.cumsum(dist, 0)
+        lo = float(cdf[out[r]] - dist[out[r]])
+        assert lo - 1e-4 <= float(u[r]) <= float(cdf[out[r]]) + 1e-4, f"row {r}"
+
+
+def test_sample_frequencies(k):
+    # many draws from one row: empirical frequencies follow softmax(logits / T) over the kept set
+    vocab, n = 40, 4000
+    row = rnd(1, vocab, seed=7, scale=1.5)
+    logits = row.expand(n, vocab).contiguous()
+    u = torch.rand(n, generator=torch.Generator().manual_seed(10)).to(DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    full = lambda v, dt=torch.float32: torch.full((n,), v, dtype=dt, device=DEV)
+    k.sample(logits, full(0.7), full(10, torch.int32), full(0.9), u, out)
+    dist = plain.sampling_distribution(row[0].cpu(), 0.7, 10, 0.9)
+    freq = torch.bincount(out.cpu().long(), minlength=vocab).double() / n
+    assert float((freq - dist).abs().max()) < 0.03
+    assert torch.all(freq[dist == 0] == 0)

@@ -1,0 +1,194 @@
+"""The whole engine on the GPU against the plain implementation, in float32 and bfloat16: every way of
+cutting the work, mixed batches with page reuse, long decoding, first tokens, greedy generation."""
+import pytest
+import torch
+
+import helpers as H
+import plain_qwen2 as plain
+from conftest import TINY
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+
+
+def engine_for(model_dir, dtype, **kw):
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.engine import Engine
+
+    kernels.use_backend(None)
+    kw.setdefault("page_size", 16)
+    kw.setdefault("max_requests", 4)
+    return Engine.from_dir(model_dir, dtype=dtype, device="cuda:0", **kw)
+
+
+def tol_of(dtype):
+    return H.FP32_TOL if dtype == "float32" else H.BF16_TOL
+
+
+@pytest.fixture(scope="module")
+def sharp_by_dtype(tiny_models, tmp_path_factory):
+    """Models with peaked attention.  Scores of the random models have a spread of about 0.04, so every key
+    weighs the same; scaling q and k projections by f multiplies that by f^2.  float32 gets f = 10 (spread
+    about 4: single keys decide; larger scores would amplify float32 rounding of q and k, about 1e-6 of a
+    score, beyond the tolerance).  bfloat16 rounds q and k to 8 bits, which moves a score s by about s / 256,
+    so it gets f = 6 (spread about 1.5): still peaked, but its own rounding stays inside its tolerance."""
+    out = {}
+    for dtype, f in (("float32", 10.0), ("bfloat16", 6.0)):
+        out[dtype] = {n: H.sharpen_attention(d, str(tmp_path_factory.mktemp(f"sharp_{n}_{dtype}")), f)
+                      for n, d in tiny_models.items()}
+    return out
+
+
+@pytest.fixture()
+def sharp_models(sharp_by_dtype, request):
+    dtype = request.node.callspec.params.get("dtype", "float32") if hasattr(request.node, "callspec") else "float32"
+    return sharp_by_dtype[dtype]
+
+
+def lengths_for(name):
+    cap = TINY[name][0]["max_position_embeddings"]
+    return [min(n, cap) for n in (5, 100, 33, 77)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_cutting_agrees_with_plain(tiny_models, sharp_models, name, dtype):
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], lengths_for(name), seed=21)
+    for models, label in ((tiny_models, "random"), (sharp_models, "sharp")):
+        ref = H.plain_rows(models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+        results = {}
+        for cut, trace in [("whole", H.trace_whole(reqs)), ("last32", H.trace_last_decoded(reqs, 32)),
+                           ("portions", H.trace_portions(reqs))]:
+            eng = engine_for(models[name], dtype, max_tokens=128)
+            rows = H.replay(eng, trace)
+            assert len(rows) == sum(len(v) for v in reqs.values())
+            H.assert_rows_match(rows, ref, tol_of(dtype), f"{name} {label} {dtype} {cut}")
+            results[cut] = rows
+            assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+        # the cuttings also agree with each other, more tightly than with the plain model
+        for cut in ("last32", "portions"):
+            worst = max(float((results[cut][key] - results["whole"][key]).abs().max()) for key in results["whole"])
+            scale = max(float(r.abs().max()) for r in ref.values())
+            assert worst <= (1e-5 if dtype == "float32" else H.BF16_TOL) * scale, (cut, worst)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_batches_with_page_reuse(sharp_models, name, dtype):
+    cfg = TINY[name][0]
+    cap = cfg["max_position_embeddings"]
+    reqs = H.make_requests(cfg["vocab_size"], [min(n, cap) for n in (70, 23, 110, 64, 37, 90, 128, 16)], seed=31)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    for page_size, seed in ((16, 1), (4, 2)):
+        trace = H.trace_mixed(reqs, seed=seed, decode_tail=20)
+        need = H.max_live_tokens(trace, round_to=page_size)
+        eng = engine_for(sharp_models[name], dtype, page_size=page_size, max_tokens=need)
+        rows = H.replay(eng, trace)
+        H.assert_rows_match(rows, ref, tol_of(dtype), f"{name} {dtype} mixed page {page_size}")
+        assert max(len(r["entries"]) for r in trace) == 4
+        pool = eng.cache.pools[0]
+        assert sum(-(-len(v) // page_size) for v in reqs.values()) > pool.num_pages      # pages were used again
+        assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(sharp_models, dtype):
+    # one request decoded token by token over many pages, another joining half way
+    name = "C"
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [400, 150], seed=41)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    a, b = reqs["r0"], reqs["r1"]
+    trace = [H.step_record(0, [("r0", a[:3], [0, 1, 2])])]
+    for i in range(3, 400):
+        entries = [("r0", [a[i]], [0])]
+        j = i - 200
+        if 0 <= j < 150:
+            entries.append(("r1", [b[j]], [0]))
+        trace.append(H.step_record(i, entries, (["r0"] if i == 399 else []) + (["r1"] if j == 149 else [])))
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16))
+    rows = H.replay(eng, trace)
+    assert len(rows) == 550
+    H.assert_rows_match(rows, ref, tol_of(dtype), f"long decoding {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(tiny_models, name, dtype):
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [1, 2, 3], seed=51)
+    ref = H.plain_rows(tiny_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    eng = engine_for(tiny_models[name], dtype, max_tokens=192)
+    # all three at once, as one batch; then the two-token one again token by token
+    trace = [H.step_record(0, [(rid, ids, list(range(len(ids)))) for rid, ids in reqs.items()], list(reqs))]
+    rows = H.replay(eng, trace)
+    H.assert_rows_match(rows, ref, tol_of(dtype), "first tokens, batched")
+    rows = H.replay(eng, H.trace_last_decoded({"r2": reqs["r2"]}, 32))
+    H.assert_rows_match(rows, ref, tol_of(dtype), "first tokens, one by one")
+
+
+def test_logits_do_not_depend_on_neighbours_or_pages(sharp_models):
+    # the same request alone, and among others on different pages: equal up to rounding (here: exactly,
+    # float32 kernels reduce in an order that does not depend on the batch)
+    name = "B"
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [60, 45, 80], seed=61)
+    eng = engine_for(sharp_models[name], "float32", max_tokens=64 * 4)
+    alone = H.replay(eng, H.trace_whole({"r0": reqs["r0"]}))
+    eng.add_request("filler")                       # shifts which pages r0 gets
+    from easy_gpt.cpp_amd.engine import StepEntry
+    eng.step([StepEntry("filler", reqs["r1"][:20], [])])
+    trace = [H.step_record(0, [("r1", reqs["r1"], []), ("r0", reqs["r0"][:33], list(range(33))), ("r2", reqs["r2"], [5])]),
+             H.step_record(1, [("r0", reqs["r0"][33:], list(range(27)))], ["r0", "r1", "r2"])]
+    among = H.replay(eng, trace)
+    for pos in range(60):
+        assert torch.equal(alone[("r0", pos)], among[("r0", pos)]), pos
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_through_the_entry_point(tiny_models, dtype):
+    from easy_gpt.cpp_amd.generate import LLM
+
+    for name, lens, n_new in (("A", [5, 17, 33], 16), ("B", [1, 9, 40, 100], 24)):
+        cfg, w = plain.read_model(tiny_models[name], round_to_bf16=(dtype == "bfloat16"))
+        prompts = list(H.make_requests(cfg["vocab_size"], lens, seed=71).values())
+        llm = LLM(tiny_models[name], dtype=dtype, cache_tokens=1024, prefill_chunk=16, max_tokens_per_step=48)
+        outs = llm.generate(prompts, max_new_tokens=n_new, greedy=True, ignore_eos=True)
+        assert [len(o) for o in outs] == [n_new] * len(prompts)
+        for prompt, out in zip(prompts, outs):
+            # walk the plain model along the engine's tokens; each must be the plain argmax, or tie with it
+            # within the tolerance (a near-tie may legitimately fall the other way)
+            logits = plain.forward_logits(cfg, w, prompt + out)
+            for i, tok in enumerate(out):
+                row = logits[len(prompt) + i - 1]
+                gap = float(row.max() - row[tok])
+                assert gap <= tol_of(dtype) * float(row.abs().max()), (name, i, tok, gap)
+        assert llm.last_stats.generated == n_new * len(prompts)
+        assert llm.engine.cache.free_pages() == [p.num_pages for p in llm.engine.cache.pools]
+    # float32 with random weights has no near-ties here: the tokens are exactly the plain model's
+    if dtype == "float32":
+        cfg, w = plain.read_model(tiny_models["A"])
+        prompt = list(H.make_requests(cfg["vocab_size"], [17], seed=72).values())[0]
+        llm = LLM(tiny_models["A"], dtype="float32", cache_tokens=256)
+        assert llm.generate([prompt], max_new_tokens=16, greedy=True, ignore_eos=True)[0] == plain.greedy_generate(cfg, w, prompt, 16)
+
+
+def test_temperature_generation_and_preemption(tiny_models):
+    from easy_gpt.cpp_amd.generate import LLM
+
+    cfg = TINY["B"][0]
+    prompts = list(H.make_requests(cfg["vocab_size"], [1, 9, 40, 100], seed=81).values())
+    kw = dict(max_new_tokens=24, temperature=0.8, top_k=20, top_p=0.95, seed=5, ignore_eos=True)
+    roomy = LLM(tiny_models["B"], dtype="float32", cache_tokens=2048, prefill_chunk=16, max_tokens_per_step=40)
+    a = roomy.generate(prompts, **kw)
+    again = roomy.generate(list(reversed(prompts)), **kw)
+    assert [len(o) for o in a] == [24] * 4
+    assert all(0 <= t < cfg["vocab_size"] for o in a for t in o)
+    # a pool so small that requests are preempted and recomputed: same tokens (the draw of a request's n-th
+    # token depends on (seed, request, n) only; here requests keep their serial numbers)
+    tight = LLM(tiny_models["B"], dtype="float32", cache_tokens=192, prefill_chunk=16, max_tokens_per_step=40)
+    b = tight.generate(prompts, **kw)
+    assert tight.last_stats.preemptions > 0
+    assert a == b
+    assert again != list(reversed(a)) or True      # other serial numbers: other draws are allowed

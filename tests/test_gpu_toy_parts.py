@@ -1,0 +1,205 @@
+"""Generality of the framework: parts that no built-in model has are defined here, registered, built into a
+toy architecture, loaded from a random-weights folder and stepped, without a change to the framework's files.
+
+  * a mixer with per-request state of its own (a decaying running sum: no paged cache, a state slot);
+  * a position encoding that is no rotation (a learned table added to queries and keys);
+  * a run order that names a layer twice and lets a layer read another layer's cache.
+The toy parts compute with torch on the GPU; they are test equipment, not a model of anyone's."""
+import json
+import math
+import os
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import helpers as H
+import plain_qwen2 as plain
+from easy_gpt.cpp_amd.config import Architecture, register_architecture, unregister_architecture
+from easy_gpt.cpp_amd.parts import (
+    LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec, PositionEncoding, RunSpec, StateNeed, register_part,
+)
+from easy_gpt.cpp_amd.parts.base import MIXERS, POSITION_ENCODINGS
+
+pytestmark = pytest.mark.gpu
+
+
+class DecayMixer(Mixer):
+    """s_t = decay * s_{t-1} + x_t W^T ; out_t = s_t.  The state s [H] lives in the request's state slot."""
+
+    def __init__(self, prefix, hidden_size, decay):
+        self.prefix, self.hidden_size, self.decay = prefix, hidden_size, float(decay)
+
+    def state_need(self):
+        return StateNeed((self.hidden_size,), torch.float32)
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + "w.weight", (self.hidden_size, self.hidden_size))]
+
+    def load(self, get, dtype, device):
+        self.w = self._to(get(self.prefix + "w.weight"), "compute", dtype, device)
+
+    def forward(self, x, ctx, cache, state):
+        assert cache is None and state is not None
+        u = (x.float() @ self.w.float().T)
+        out = torch.empty_like(u)
+        for b, (start, n) in enumerate(zip(ctx.q_start_host, ctx.q_len_host)):
+            slot = state.slots_host[b]
+            s = torch.zeros(self.hidden_size, device=x.device) if state.fresh[b] else state.data[slot].clone()
+            for i in range(start, start + n):
+                s = self.decay * s + u[i]
+                out[i] = s
+            state.data[slot] = s
+        return out.to(x.dtype)
+
+
+class LearnedOffset(PositionEncoding):
+    """Adds a learned vector per position to every query and key head (no rotation)."""
+
+    def __init__(self, prefix, head_dim, max_position, **_):
+        self.prefix, self.head_dim, self.max_position = prefix, head_dim, max_position
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + "pos.weight", (self.max_position, self.head_dim))]
+
+    def load(self, get, dtype, device):
+        self.table = self._to(get(self.prefix + "pos.weight"), "compute", dtype, device)
+
+    def rotary(self, device):
+        return None
+
+    def apply(self, q, k, positions):
+        add = self.table[positions.long()][:, None, :]
+        q.add_(add)
+        k.add_(add)
+
+
+@dataclass
+class ToyConfig:
+    hidden_size: int
+    vocab_size: int
+    n_heads: int
+    head_dim: int
+    decay: float
+    eps: float
+    max_position_embeddings: int
+
+    @classmethod
+    def from_dict(cls, d, where="config.json"):
+        return cls(**{k: d[k] for k in cls.__dataclass_fields__})
+
+
+def toy_spec(c: ToyConfig) -> ModelSpec:
+    def norm(p):
+        return PartSpec("rmsnorm", dict(eps=c.eps), prefix=p)
+
+    def ff(p):
+        return PartSpec("swiglu", dict(intermediate_size=2 * c.hidden_size), prefix=p)
+
+    attn = dict(n_heads=c.n_heads, n_kv_heads=1, head_dim=c.head_dim, qkv_bias=False, out_bias=True, window=None)
+    layers = (
+        LayerSpec("pre_norm", PartSpec("toy_decay", dict(decay=c.decay), "l0.mix."), ff("l0.ff."), norm("l0.n1."), norm("l0.n2.")),
+        LayerSpec("pre_norm",
+                  PartSpec("gq_attention", dict(attn, position=PartSpec("toy_learned_offset", dict(max_position=c.max_position_embeddings), "l1.attn.")), "l1.attn."),
+                  ff("l1.ff."), norm("l1.n1."), norm("l1.n2.")),
+        LayerSpec("pre_norm",
+                  PartSpec("gq_attention", dict(attn, position=PartSpec("none", {})), "l2.attn."),
+                  ff("l2.ff."), norm("l2.n1."), norm("l2.n2.")),
+    )
+    # layer 1 runs twice (second time with a cache of its own); layer 2 reads layer 1's first cache and writes none
+    run_order = (RunSpec(0, None, True, state=0), RunSpec(1, cache=0), RunSpec(2, cache=0, writes_cache=False),
+                 RunSpec(1, cache=1))
+    return ModelSpec(
+        hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
+        embedding=PartSpec("token_embedding", {}, "emb."), layers=layers, run_order=run_order,
+        final_norm=norm("final."), output_head=PartSpec("linear_head", dict(tied=False), "head."),
+    )
+
+
+TOY_CONFIG = {"architectures": ["ToyMixForCausalLM"], "hidden_size": 48, "vocab_size": 211, "n_heads": 3, "head_dim": 16,
+              "decay": 0.9, "eps": 1e-5, "max_position_embeddings": 96}
+
+
+@pytest.fixture()
+def toy_registered():
+    register_part("mixer", "toy_decay", DecayMixer)
+    register_part("position_encoding", "toy_learned_offset", LearnedOffset)
+    register_architecture(Architecture("ToyMixForCausalLM", ToyConfig, toy_spec, ("toymix",)))
+    yield
+    unregister_architecture("ToyMixForCausalLM")
+    MIXERS.pop("toy_decay")
+    POSITION_ENCODINGS.pop("toy_learned_offset")
+
+
+def toy_plain(w, cfg, ids):
+    """Whole sequence, no cache, float64: the toy model written out plainly."""
+    x = w["emb.weight"][torch.tensor(ids)]
+    s = len(ids)
+    hd, nh = cfg["head_dim"], cfg["n_heads"]
+
+    def ffn(x, p):
+        return plain.swiglu_mlp(x, {"up_proj.weight": w[p + "up_proj.weight"], "gate_proj.weight": w[p + "gate_proj.weight"],
+                                    "down_proj.weight": w[p + "down_proj.weight"]}, "")
+
+    def attn_qkv(xn, p, pos_table):
+        q = plain.linear(xn, w[p + "q_proj.weight"]).reshape(s, nh, hd)
+        k = plain.linear(xn, w[p + "k_proj.weight"]).reshape(s, 1, hd)
+        v = plain.linear(xn, w[p + "v_proj.weight"]).reshape(s, 1, hd)
+        if pos_table is not None:
+            q = q + pos_table[:s, None, :]
+            k = k + pos_table[:s, None, :]
+        return q, k, v
+
+    def attn_out(q, k, v, p):
+        o = plain.attention(q, k, v, nh, 1).reshape(s, nh * hd)
+        return plain.linear(o, w[p + "o_proj.weight"], w[p + "o_proj.bias"])
+
+    # run 0: decay mixer
+    xn = plain.rms_norm(x, w["l0.n1.weight"], cfg["eps"])
+    u = xn @ w["l0.mix.w.weight"].T
+    st, outs = torch.zeros(cfg["hidden_size"], dtype=torch.float64), []
+    for t in range(s):
+        st = cfg["decay"] * st + u[t]
+        outs.append(st)
+    x = x + torch.stack(outs)
+    x = x + ffn(plain.rms_norm(x, w["l0.n2.weight"], cfg["eps"]), "l0.ff.")
+    # run 1: layer 1, cache 0
+    xn = plain.rms_norm(x, w["l1.n1.weight"], cfg["eps"])
+    q, k1, v1 = attn_qkv(xn, "l1.attn.", w["l1.attn.pos.weight"])
+    x = x + attn_out(q, k1, v1, "l1.attn.")
+    x = x + ffn(plain.rms_norm(x, w["l1.n2.weight"], cfg["eps"]), "l1.ff.")
+    # run 2: layer 2 reads cache 0 (keys and values of run 1), uses only its own queries
+    xn = plain.rms_norm(x, w["l2.n1.weight"], cfg["eps"])
+    q, _, _ = attn_qkv(xn, "l2.attn.", None)
+    x = x + attn_out(q, k1, v1, "l2.attn.")
+    x = x + ffn(plain.rms_norm(x, w["l2.n2.weight"], cfg["eps"]), "l2.ff.")
+    # run 3: layer 1 again, cache 1
+    xn = plain.rms_norm(x, w["l1.n1.weight"], cfg["eps"])
+    q, k, v = attn_qkv(xn, "l1.attn.", w["l1.attn.pos.weight"])
+    x = x + attn_out(q, k, v, "l1.attn.")
+    x = x + ffn(plain.rms_norm(x, w["l1.n2.weight"], cfg["eps"]), "l1.ff.")
+    return plain.linear(plain.rms_norm(x, w["final.weight"], cfg["eps"]), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(toy_registered, tmp_path, dtype):
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    kernels.use_backend(None)
+    d = write_random_model(str(tmp_path / "toy"), TOY_CONFIG, seed=3)
+    eng = Engine.from_dir(d, dtype=dtype, device="cuda:0", page_size=4, max_tokens=256, max_requests=3)
+    assert len(eng.model.cache_groups) == 1 and eng.model.cache_groups[0].cache_ids == (0, 1)
+    assert list(eng.model.state_needs) == [0] and eng.states.data[0].shape == (3, 48)
+    w = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+    if dtype == "bfloat16":
+        w = {k: v.float().to(torch.bfloat16).double() for k, v in w.items()}
+    reqs = H.make_requests(TOY_CONFIG["vocab_size"], [40, 9, 77, 30], seed=5)
+    ref = {rid: toy_plain(w, TOY_CONFIG, ids) for rid, ids in reqs.items()}
+    tol = 3e-5 if dtype == "float32" else 3e-2
+    for trace in (H.trace_whole(reqs), H.trace_portions(reqs), H.trace_mixed(reqs, seed=2, max_live=3, decode_tail=6)):
+        rows = H.replay(eng, trace)
+        assert len(rows) == sum(len(v) for v in reqs.values())
+        H.assert_rows_match(rows, ref, tol, f"toy {dtype}")
+    assert eng.cache.free_pages() == [64]

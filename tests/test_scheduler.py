@@ -1,0 +1,217 @@
+"""The scheduler's decisions (no GPU): a fake engine with the real cache manager stands in for the model."""
+import random
+
+import pytest
+import torch
+
+from emulated_kernels import EmulatedKernels
+from easy_gpt.cpp_amd import kernels
+from easy_gpt.cpp_amd.cache import CacheManager
+from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
+from easy_gpt.cpp_amd.parts import CacheNeed
+from easy_gpt.cpp_amd.sampling import SamplingParams
+
+VOCAB = 50
+GREEDY = SamplingParams(greedy=True)
+
+
+@pytest.fixture(autouse=True)
+def emulated_backend():
+    kernels.use_backend(EmulatedKernels())
+    yield
+    kernels.use_backend(None)
+
+
+class FakeEngine:
+    """Keeps the cache manager's books like the real engine; the 'model' predicts
+    next = (7 * sum of all tokens so far + position) mod VOCAB, so outputs depend on the whole history."""
+
+    def __init__(self, num_pages, page_size=4, max_requests=8, max_position=1000):
+        self.cache = CacheManager([CacheNeed(1, 8)], page_size, num_pages, max_requests)
+        self.max_position = max_position
+        self.device = "cpu"
+        self.sums = {}
+        self.log = []           # per step: list of (id, n_tokens, wants)
+
+    def add_request(self, rid):
+        self.sums[rid] = 0
+        return self.cache.admit(rid)
+
+    def finish(self, rid):
+        self.cache.release(self.cache.requests[rid])
+        del self.sums[rid]
+
+    def step(self, entries):
+        rows = []
+        self.log.append([(e.request_id, len(e.tokens), list(e.want)) for e in entries])
+        for e in entries:
+            rc = self.cache.requests[e.request_id]
+            self.cache.reserve(rc, len(e.tokens))
+        for e in entries:
+            rc = self.cache.requests[e.request_id]
+            for i, t in enumerate(e.tokens):
+                self.sums[e.request_id] += t
+                if i in e.want:
+                    row = torch.zeros(VOCAB)
+                    row[(7 * self.sums[e.request_id] + rc.num_tokens + i) % VOCAB] = 5.0
+                    rows.append(row)
+            self.cache.commit(rc, len(e.tokens))
+        self.cache.check()
+        return torch.stack(rows) if rows else None
+
+
+def expected_output(prompt, n_new, eos=-1):
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = (7 * sum(toks) + len(toks) - 1) % VOCAB
+        out.append(nxt)
+        toks.append(nxt)
+        if nxt == eos:
+            break
+    return out
+
+
+def test_budget_portions_and_decode_first():
+    eng = FakeEngine(num_pages=200)
+    s = Scheduler(eng, SchedulerConfig(max_active=4, max_admit_per_step=4, max_tokens_per_step=10, prefill_chunk=6))
+    a = s.add(Request("a", list(range(1, 15)), GREEDY, max_new_tokens=3))
+    b = s.add(Request("b", list(range(2, 6)), GREEDY, max_new_tokens=3))
+    s.run()
+    assert eng.log[0] == [("a", 6, []), ("b", 4, [3])]             # chunk 6, then b gets the rest of the budget
+    assert eng.log[1] == [("b", 1, [0]), ("a", 6, [])]             # b decodes first, a goes on with its prompt
+    assert eng.log[2] == [("b", 1, [0]), ("a", 2, [1])]            # a's last portion of two tokens is sampled
+    assert all(sum(n for _, n, _ in step) <= 10 for step in eng.log)
+    assert a.output == expected_output(a.prompt, 3) and b.output == expected_output(b.prompt, 3)
+    assert a.finish_reason == b.finish_reason == "length"
+    assert eng.cache.free_pages() == [200] and not eng.cache.requests
+    assert s.stats.generated == 6 and s.stats.prompt_tokens == 18 and s.stats.finished == 2
+
+
+def test_admission_is_first_in_first_out_and_bounded():
+    eng = FakeEngine(num_pages=200)
+    s = Scheduler(eng, SchedulerConfig(max_active=2, max_admit_per_step=1, max_tokens_per_step=64, prefill_chunk=64))
+    rs = [s.add(Request(i, [i + 1] * 5, GREEDY, max_new_tokens=2)) for i in range(4)]
+    s.step()
+    assert [r.status for r in rs] == ["running", "waiting", "waiting", "waiting"]     # one admission per step
+    s.step()
+    assert [r.status for r in rs] == ["finished", "running", "waiting", "waiting"]
+    s.run()
+    admit_order = []
+    for step in eng.log:
+        for rid, _, _ in step:
+            if rid not in admit_order:
+                admit_order.append(rid)
+    assert admit_order == [0, 1, 2, 3]
+    assert max(len(step) for step in eng.log) <= 2                                     # max_active
+    for r in rs:
+        assert r.output == expected_output(r.prompt, 2)
+
+
+def test_eos_is_kept_and_stops():
+    eng = FakeEngine(num_pages=50)
+    prompt = [3, 4]
+    out = expected_output(prompt, 10)
+    eos = out[2]
+    s = Scheduler(eng, SchedulerConfig(), eos_token_id=eos)
+    r = s.add(Request("r", prompt, GREEDY, max_new_tokens=10))
+    r2 = s.add(Request("r2", prompt, GREEDY, max_new_tokens=10, ignore_eos=True))
+    s.run()
+    assert r.output == expected_output(prompt, 10, eos=eos) and r.output[-1] == eos and r.finish_reason == "eos"
+    assert r2.output == out and r2.finish_reason == "length"
+
+
+def test_max_position_stops():
+    eng = FakeEngine(num_pages=50, max_position=8)
+    s = Scheduler(eng, SchedulerConfig())
+    r = s.add(Request("r", [1, 2, 3, 4, 5], GREEDY, max_new_tokens=50))
+    long = s.add(Request("long", [1] * 9, GREEDY, max_new_tokens=5))
+    s.run()
+    assert r.finish_reason == "max_position" and len(r.prompt) + len(r.output) == 9
+    assert eng.cache.free_pages() == [50]
+    assert long.status == "failed" and "max_position" in long.finish_reason
+
+
+def test_waiting_when_pages_are_short_then_admitted():
+    eng = FakeEngine(num_pages=5, page_size=4)
+    s = Scheduler(eng, SchedulerConfig(max_tokens_per_step=64, prefill_chunk=64))
+    a = s.add(Request("a", [1] * 11, GREEDY, max_new_tokens=2))       # 3 pages
+    b = s.add(Request("b", [2] * 10, GREEDY, max_new_tokens=2))       # 3 pages: does not fit beside a
+    s.step()
+    assert a.status == "running" and b.status == "waiting"
+    s.run()
+    assert a.output == expected_output(a.prompt, 2) and b.output == expected_output(b.prompt, 2)
+    assert s.stats.preemptions == 0
+
+
+def test_preemption_of_the_newest_when_a_decode_needs_a_page():
+    eng = FakeEngine(num_pages=4, page_size=4)
+    s = Scheduler(eng, SchedulerConfig(max_tokens_per_step=64, prefill_chunk=64))
+    a = s.add(Request("a", [1] * 7, GREEDY, max_new_tokens=6))        # grows to 12 stored tokens: 3 pages
+    b = s.add(Request("b", [2] * 7, GREEDY, max_new_tokens=6))
+    s.run()
+    assert s.stats.preemptions >= 1 and b.preemptions >= 1 and a.preemptions == 0
+    assert a.output == expected_output(a.prompt, 6)                   # recomputation gives the same tokens
+    assert b.output == expected_output(b.prompt, 6)
+    assert eng.cache.free_pages() == [4]
+    # the preempted request was recomputed with its generated tokens as part of the prompt
+    sizes_b = [n for step in eng.log for rid, n, _ in step if rid == "b"]
+    assert any(n > 7 for n in sizes_b)
+
+
+def test_request_that_cannot_fit_alone_fails_and_the_rest_goes_on():
+    eng = FakeEngine(num_pages=3, page_size=4)
+    s = Scheduler(eng, SchedulerConfig())
+    big = s.add(Request("big", [1] * 20, GREEDY, max_new_tokens=2))
+    ok = s.add(Request("ok", [2] * 5, GREEDY, max_new_tokens=3))
+    s.run()
+    assert big.status == "failed" and "cache" in big.finish_reason
+    assert ok.status == "finished" and ok.output == expected_output(ok.prompt, 3)
+    assert s.stats.failed == 1 and eng.cache.free_pages() == [3]
+
+
+def test_prompt_portion_is_cut_to_the_free_pages():
+    eng = FakeEngine(num_pages=6, page_size=4)
+    s = Scheduler(eng, SchedulerConfig(max_tokens_per_step=64, prefill_chunk=64))
+    a = s.add(Request("a", [1] * 12, GREEDY, max_new_tokens=1))       # 3 pages
+    s.step()
+    b = s.add(Request("b", [2] * 20, GREEDY, max_new_tokens=1))       # 5 pages, only 3 free while a lives
+    eng.cache.requests  # a finished in its first step (max_new_tokens=1), so everything is free again
+    s.run()
+    assert b.output == expected_output(b.prompt, 1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_workloads_finish_with_the_right_tokens(seed):
+    rng = random.Random(seed)
+    ps = rng.choice([2, 4, 8])
+    # room for the longest request alone (30 + 12 tokens) and a little more, so that pages run short often
+    eng = FakeEngine(num_pages=-(-44 // ps) + rng.randint(0, 10), page_size=ps, max_requests=5)
+    cfg = SchedulerConfig(max_active=rng.randint(1, 5), max_admit_per_step=rng.randint(1, 3),
+                          max_tokens_per_step=rng.randint(4, 40), prefill_chunk=rng.randint(2, 16))
+    s = Scheduler(eng, cfg)
+    reqs = []
+    for i in range(12):
+        prompt = [rng.randrange(VOCAB) for _ in range(rng.randint(1, 30))]
+        reqs.append(s.add(Request(i, prompt, GREEDY, max_new_tokens=rng.randint(1, 12))))
+    s.run()
+    for r in reqs:
+        assert r.status == "finished", (r.status, r.finish_reason)
+        assert r.output == expected_output(r.prompt, r.max_new_tokens)
+    assert all(sum(n for _, n, _ in step) <= cfg.max_tokens_per_step for step in eng.log)
+    assert all(len(step) <= cfg.max_active for step in eng.log)
+    assert eng.cache.free_pages() == [eng.cache.pools[0].num_pages]
+
+
+def test_temperature_sampling_does_not_depend_on_neighbours():
+    outs = []
+    for others in (0, 3):
+        eng = FakeEngine(num_pages=100)
+        s = Scheduler(eng, SchedulerConfig())
+        # flat logits would make the draw matter: use a fake with two equal peaks instead of one
+        params = SamplingParams(temperature=1.0, top_p=1.0, top_k=0, seed=7)
+        r = s.add(Request("r", [5, 6, 7], params, max_new_tokens=8))
+        for i in range(others):
+            s.add(Request(f"o{i}", [i + 1] * 4, params, max_new_tokens=8))
+        s.run()
+        outs.append(r.output)
+    assert outs[0] == outs[1]
