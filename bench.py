@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Benchmark of the serving step on one MI355X: decode tokens/s at batch 8 (value), batch 1 and 64 (points),
+and a 2,048-token prefill, for the Qwen2.5-0.5B layer sizes with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch: the engine's step function on one token per request, greedy
+sampling on the device, and the sampled tokens brought to the host (a server needs them there to detect the
+end of a request).  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBPS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+# Qwen2.5-0.5B layer sizes (the third configuration of the baseline record)
+QWEN25_05B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 24, "hidden_size": 896,
+    "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,
+    "use_sliding_window": False, "hidden_act": "silu", "torch_dtype": "bfloat16",
+}
+FULL_LAYERS = 24
+PREFIX = 2048
+NEW_TOKENS = 128
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=NEW_TOKENS - 16)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
+        return 2
+    if args.warmup + args.steps > CONTEXT - PREFIX:
+        print(f"--warmup + --steps must stay within the context of {CONTEXT} after a prefix of {PREFIX}")
+        return 2
+
+    import torch
+
+    from easy_gpt.cpp_amd.engine import Engine, StepEntry
+    from easy_gpt.cpp_amd.sampling import Sampler, SamplingParams
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    cfg = dict(QWEN25_05B, num_hidden_layers=args.layers)
+    dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    elem = 2 if args.dtype == "bfloat16" else 4
+    h, nq, nkv, inter, vocab = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
+                                cfg["intermediate_size"], cfg["vocab_size"])
+    hd = h // nq
+    layers = args.layers
+    page_size = 16
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    max_batch = max(batches)
+
+    t_setup = time.time()
+    tmp = tempfile.mkdtemp(prefix="egpt_bench_")
+    write_random_model(tmp, cfg, seed=0, dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
+    tokens_per_request = -(-(PREFIX + NEW_TOKENS) // page_size) * page_size
+    engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
+                             max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1)
+    for f in os.listdir(tmp):
+        os.remove(os.path.join(tmp, f))
+    os.rmdir(tmp)
+    sampler = Sampler(engine.device)
+    greedy = SamplingParams(greedy=True)
+    g = torch.Generator().manual_seed(0)
+    print(f"[bench] model ready in {time.time() - t_setup:.1f} s", file=sys.stderr, flush=True)
+
+    # per-step work of the model, for the rooflines
+    layer_weights = (h * (nq + 2 * nkv) * hd + (nq + 2 * nkv) * hd + nq * hd * h + 3 * h * inter + 2 * h) * elem
+    weight_bytes = layers * layer_weights + vocab * h * elem + h * elem          # output matrix read once, tied or not
+    kv_bytes_per_token = layers * 2 * nkv * hd * elem
+
+    def prefill_flops(t: int) -> float:
+        linear = 2.0 * t * (h * (nq + 2 * nkv) * hd + nq * hd * h + 3 * h * inter)
+        attention = 2.0 * t * (t + 1) * hd * nq                                  # QK^T and PV over the causal half
+        return layers * (linear + attention) + 2.0 * vocab * h                   # logits at the last place only
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---------------------------------------------------------------- prefill of 2,048 tokens, one request, one step
+    prefill = None
+    if not args.no_points:
+        ids = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
+        times = []
+        for rep in range(5):
+            engine.add_request("prefill")
+            sync()
+            t0 = time.perf_counter()
+            engine.step([StepEntry("prefill", ids, [PREFILL_TOKENS - 1])])
+            sync()
+            times.append(time.perf_counter() - t0)
+            engine.finish("prefill")
+        sec = sorted(times[1:])[len(times[1:]) // 2]
+        prefill = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
+                   "frac": round(prefill_flops(PREFILL_TOKENS) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
+        print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+
+    # ---------------------------------------------------------------- decoding at each batch size
+    def decode_run(batch: int, warmup: int, steps: int):
+        rids = [f"d{i}" for i in range(batch)]
+        prompts = [torch.randint(0, vocab, (PREFIX,), generator=g).tolist() for _ in rids]
+        last = []
+        for rid, p in zip(rids, prompts):                      # untimed: fill the cache with the prefixes
+            engine.add_request(rid)
+            out = engine.step([StepEntry(rid, p, [PREFIX - 1])])
+            last.append(sampler.sample(out, [greedy], [0], [0])[0])
+        params, serials = [greedy] * batch, list(range(batch))
+
+        def one_step(tokens, n):
+            logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(rids, tokens)])
+            return sampler.sample(logits, params, serials, [n] * batch)      # ends with the tokens on the host
+
+        for i in range(warmup):
+            last = one_step(last, i)
+        sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            last = one_step(last, warmup + i)
+        sync()
+        sec = time.perf_counter() - t0
+        for rid in rids:
+            engine.finish(rid)
+        mean_ctx = PREFIX + warmup + (steps + 1) / 2.0
+        step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
+        return sec, step_bytes
+
+    results = {}
+    for b in batches:
+        sec, step_bytes = decode_run(b, args.warmup, args.steps)
+        results[b] = (sec, step_bytes)
+        print(f"[bench] decode batch {b}: {b * args.steps / sec:.1f} tok/s, {sec / args.steps * 1e3:.3f} ms/step, "
+              f"{step_bytes / (sec / args.steps) / 1e9:.1f} GB/s", file=sys.stderr, flush=True)
+
+    sec, step_bytes = results[args.batch]
+    achieved = step_bytes / (sec / args.steps) / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8 (Qwen2.5-0.5B, prefix 2048)" if args.batch == 8
+        else f"decode tok/s at batch {args.batch} (Qwen2.5-0.5B, prefix 2048)",
+        "value": round(args.batch * args.steps / sec, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype_key,
+        "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
+        "config": {
+            "model": "Qwen2.5-0.5B layer sizes", "layers": layers, "layers_of_model": FULL_LAYERS, "hidden": h,
+            "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": True,
+            "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": NEW_TOKENS,
+            "page_size": page_size, "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
+            "sampling": "greedy", "parallelism": "single GPU",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 5)},
+    }
+    if prefill is not None:
+        line["prefill"] = prefill
+    points = {f"decode_b{b}": round(b * args.steps / results[b][0], 1) for b in batches if b != args.batch}
+    if points:
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
