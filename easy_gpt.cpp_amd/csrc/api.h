@@ -15,12 +15,18 @@ int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, 
                void* stream);
 // h += delta (delta may be null); out = rmsnorm(h) * weight.  rows == null: every row, h written back.
 // rows != null: only the listed rows, gathered into out[n_rows], h untouched.
-int egpt_add_rmsnorm(float* h, const void* delta, const int32_t* rows, const void* weight, float eps, void* out,
-                     int n_rows, int hidden, int dtype, void* stream);
-int egpt_swiglu(const void* gate_up, void* out, int n_tokens, int inter, int dtype, void* stream);
-int egpt_qkv_rope_store(void* qkv, const void* bias, const int32_t* positions, const float* inv_freq, int rotary_dim,
-                        const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv, int hd,
-                        int page_size, int dtype, void* stream);
+// A product may arrive as float32 partial sums of a split-k product, [n_splits][rows][cols]: then the
+// *_splits argument is > 0 and the consumer adds the splits up; 0 means one tensor of the activation type.
+int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
+                     const void* weight, float eps, void* out, int n_rows, int hidden, int dtype, void* stream);
+int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype, void* stream);
+// qkv_out [n_tokens, (nq + 2 nkv) hd] of the activation type; may be qkv_in itself when n_splits == 0.
+int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_out, const void* bias, const int32_t* positions,
+                        const float* inv_freq, int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache,
+                        int n_tokens, int nq, int nkv, int hd, int page_size, int dtype, void* stream);
+// bfloat16 product for m <= 64 rows on the matrix cores, optionally split over k (see gemm_skinny.hip).
+int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m, int n,
+                     int k, int n_splits, void* stream);
 // out = x w^T + bias; x [m,k], w [n,k], out [m,n]; out_f32 != 0 writes float32 whatever dtype is.
 int egpt_linear(const void* x, const void* w, const void* bias, void* out, int m, int n, int k, int dtype,
                 int out_f32, void* stream);

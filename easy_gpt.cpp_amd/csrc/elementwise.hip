@@ -5,6 +5,23 @@
 
 namespace egpt {
 
+// The output of a product arrives either as one tensor of the activation type, or as float32 partial
+// sums [n_splits][rows][cols] of a split-k product, which are added here in split order.
+template <typename T>
+struct ProductView {
+    const T* whole;          // used when n_splits == 0
+    const float* partial;    // used when n_splits > 0
+    int n_splits;
+    size_t split_stride;     // rows * cols
+    __device__ __forceinline__ bool present() const { return whole != nullptr || partial != nullptr; }
+    __device__ __forceinline__ float at(size_t idx) const {
+        if (n_splits == 0) return to_float(whole[idx]);
+        float v = partial[idx];
+        for (int s = 1; s < n_splits; ++s) v += partial[s * split_stride + idx];
+        return v;
+    }
+};
+
 // ----------------------------------------------------------------------------- embedding
 // x[t, :] = E[id_t, :]   (/root/reference/src/models/embedding.cpp:54-76); output float32.
 template <typename T>
@@ -23,19 +40,20 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restric
 // (/root/reference/src/models/norm.cpp:47-59, /root/reference/src/cuda/ops/self_attn_detail.cuh:385-418).
 // The residual addition h += delta happens here too, in float32.
 template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
                                    const int32_t* __restrict__ rows, const T* __restrict__ weight, float eps,
                                    T* __restrict__ out, int hidden) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
     float* hrow = h + src * hidden;
-    const T* drow = delta ? delta + src * hidden : nullptr;
-    const bool write_back = (rows == nullptr) && (delta != nullptr);
+    const bool has_delta = delta.present();
+    const size_t dbase = src * hidden;
+    const bool write_back = (rows == nullptr) && has_delta;
     float ss = 0.f;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = hrow[j];
-        if (drow) v += to_float(drow[j]);
+        if (has_delta) v += delta.at(dbase + j);
         if (write_back) hrow[j] = v;
         ss += v * v;
     }
@@ -44,7 +62,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
     T* orow = out + static_cast<size_t>(r) * hidden;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = hrow[j];                       // already updated when written back
-        if (drow && !write_back) v += to_float(drow[j]);
+        if (has_delta && !write_back) v += delta.at(dbase + j);
         orow[j] = from_float<T>(v * inv * to_float(weight[j]));
     }
 }
@@ -52,13 +70,13 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
 // ----------------------------------------------------------------------------- SwiGLU
 // out = up * gate / (1 + exp(-gate))   (/root/reference/src/cuda/ops/mlp.cu:152-162); [gate | up] per row.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int n_tokens, int inter) {
+__global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n_tokens, int inter) {
     const size_t total = static_cast<size_t>(n_tokens) * inter;
     for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
          i += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const size_t t = i / inter, j = i % inter;
-        const float g = to_float(gate_up[t * 2 * inter + j]);
-        const float u = to_float(gate_up[t * 2 * inter + inter + j]);
+        const float g = gate_up.at(t * 2 * inter + j);
+        const float u = gate_up.at(t * 2 * inter + inter + j);
         out[i] = from_float<T>(u * (g / (1.0f + expf(-g))));
     }
 }
@@ -70,13 +88,14 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
 // write the result back in place and store keys and values at their slot of the paged cache
 // [page][kv head][offset][hd].
 template <typename T>
-__global__ void qkv_rope_store_kernel(T* __restrict__ qkv, const T* __restrict__ bias,
+__global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv_out, const T* __restrict__ bias,
                                       const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
                                       int rotary_dim, const int32_t* __restrict__ slots, T* __restrict__ k_cache,
                                       T* __restrict__ v_cache, int nq, int nkv, int hd, int page_size) {
     const int t = blockIdx.x;
     const int n_heads = nq + 2 * nkv;
-    T* row = qkv + static_cast<size_t>(t) * n_heads * hd;
+    const size_t base = static_cast<size_t>(t) * n_heads * hd;
+    T* row = qkv_out + base;
     const float pos = static_cast<float>(positions[t]);
     const int half = rotary_dim / 2;
     long slot = slots ? slots[t] : -1;
@@ -85,10 +104,10 @@ __global__ void qkv_rope_store_kernel(T* __restrict__ qkv, const T* __restrict__
         const int head = item / hd, d = item % hd;
         const bool rotated = head < nq + nkv && d < rotary_dim;
         if (rotated && d >= half) continue;  // done by its partner
-        float a = to_float(row[item]) + (bias ? to_float(bias[item]) : 0.f);
+        float a = qkv_in.at(base + item) + (bias ? to_float(bias[item]) : 0.f);
         float b = 0.f;
         if (rotated) {
-            b = to_float(row[item + half]) + (bias ? to_float(bias[item + half]) : 0.f);
+            b = qkv_in.at(base + item + half) + (bias ? to_float(bias[item + half]) : 0.f);
             float s, c;
             sincosf(pos * inv_freq[d], &s, &c);
             const float ra = a * c - b * s, rb = a * s + b * c;
@@ -127,18 +146,31 @@ extern "C" int egpt_embed(const int32_t* ids, const void* table, float* out, int
     return EGPT_OK;
 }
 
-extern "C" int egpt_add_rmsnorm(float* h, const void* delta, const int32_t* rows, const void* weight, float eps,
-                                void* out, int n_rows, int hidden, int dtype, void* stream) {
-    if (!h || !weight || !out || n_rows < 0 || hidden <= 0) return EGPT_BAD_ARGUMENT;
+template <typename T>
+static ProductView<T> make_view(const void* p, int n_splits, size_t split_stride) {
+    ProductView<T> v;
+    v.whole = n_splits == 0 ? static_cast<const T*>(p) : nullptr;
+    v.partial = n_splits > 0 ? static_cast<const float*>(p) : nullptr;
+    v.n_splits = n_splits;
+    v.split_stride = split_stride;
+    return v;
+}
+
+extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
+                                const void* weight, float eps, void* out, int n_rows, int hidden, int dtype,
+                                void* stream) {
+    if (!h || !weight || !out || n_rows < 0 || hidden <= 0 || delta_splits < 0) return EGPT_BAD_ARGUMENT;
+    if (delta && delta_rows <= 0) return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int threads = hidden >= 2048 ? 512 : 256;
+    const size_t stride = static_cast<size_t>(delta_rows) * hidden;
     if (dtype == 0)
-        add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, static_cast<const float*>(delta), rows,
+        add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, make_view<float>(delta, delta_splits, stride), rows,
                                                              static_cast<const float*>(weight), eps,
                                                              static_cast<float*>(out), hidden);
     else if (dtype == 1)
-        add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(h, static_cast<const bf16_t*>(delta), rows,
+        add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(h, make_view<bf16_t>(delta, delta_splits, stride), rows,
                                                               static_cast<const bf16_t*>(weight), eps,
                                                               static_cast<bf16_t*>(out), hidden);
     else
@@ -147,42 +179,49 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, const int32_t* rows
     return EGPT_OK;
 }
 
-extern "C" int egpt_swiglu(const void* gate_up, void* out, int n_tokens, int inter, int dtype, void* stream) {
-    if (!gate_up || !out || n_tokens < 0 || inter <= 0) return EGPT_BAD_ARGUMENT;
+extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype,
+                           void* stream) {
+    if (!gate_up || !out || n_tokens < 0 || inter <= 0 || n_splits < 0) return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t total = static_cast<size_t>(n_tokens) * inter;
     const int blocks = static_cast<int>(total / 256 + 1 > 8192 ? 8192 : total / 256 + 1);
+    const size_t stride = total * 2;
     if (dtype == 0)
-        swiglu_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out),
-                                                    n_tokens, inter);
+        swiglu_kernel<float><<<blocks, 256, 0, s>>>(make_view<float>(gate_up, n_splits, stride),
+                                                    static_cast<float*>(out), n_tokens, inter);
     else if (dtype == 1)
-        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
-                                                     n_tokens, inter);
+        swiglu_kernel<bf16_t><<<blocks, 256, 0, s>>>(make_view<bf16_t>(gate_up, n_splits, stride),
+                                                     static_cast<bf16_t*>(out), n_tokens, inter);
     else
         return EGPT_BAD_ARGUMENT;
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
 
-extern "C" int egpt_qkv_rope_store(void* qkv, const void* bias, const int32_t* positions, const float* inv_freq,
-                                   int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens,
-                                   int nq, int nkv, int hd, int page_size, int dtype, void* stream) {
-    if (!qkv || !positions || n_tokens < 0 || nq <= 0 || nkv <= 0 || hd <= 0 || page_size <= 0)
+extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_out, const void* bias,
+                                   const int32_t* positions, const float* inv_freq, int rotary_dim,
+                                   const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv,
+                                   int hd, int page_size, int dtype, void* stream) {
+    if (!qkv_in || !qkv_out || !positions || n_tokens < 0 || nq <= 0 || nkv <= 0 || hd <= 0 || page_size <= 0 ||
+        n_splits < 0)
         return EGPT_BAD_ARGUMENT;
     if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim % 2) != 0 || (rotary_dim > 0 && !inv_freq))
         return EGPT_BAD_ARGUMENT;
     if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
     if (dtype == 0)
         qkv_rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(
-            static_cast<float*>(qkv), static_cast<const float*>(bias), positions, inv_freq, rotary_dim, slots,
-            static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq, nkv, hd, page_size);
+            make_view<float>(qkv_in, n_splits, stride), static_cast<float*>(qkv_out), static_cast<const float*>(bias),
+            positions, inv_freq, rotary_dim, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq,
+            nkv, hd, page_size);
     else if (dtype == 1)
         qkv_rope_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(
-            static_cast<bf16_t*>(qkv), static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots,
-            static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
+            make_view<bf16_t>(qkv_in, n_splits, stride), static_cast<bf16_t*>(qkv_out),
+            static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots, static_cast<bf16_t*>(k_cache),
+            static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
     else
         return EGPT_BAD_ARGUMENT;
     EGPT_CHECK_LAUNCH();
@@ -199,4 +238,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 1; }
+extern "C" int egpt_abi_version(void) { return 2; }

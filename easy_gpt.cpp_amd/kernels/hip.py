@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 1:
+    if lib.egpt_abi_version() != 2:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -44,10 +44,11 @@ class HipKernels:
         lib.egpt_error_string.argtypes = [i]
         sigs = {
             "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
-            "egpt_add_rmsnorm": [vp, vp, vp, vp, f, vp, i, i, i, vp],
-            "egpt_swiglu": [vp, vp, i, i, i, vp],
-            "egpt_qkv_rope_store": [vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
+            "egpt_swiglu": [vp, i, vp, i, i, i, vp],
+            "egpt_qkv_rope_store": [vp, i, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_argmax": [vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
@@ -88,6 +89,14 @@ class HipKernels:
             raise TypeError(f"{name} must be float32 or bfloat16, got {t.dtype}")
         return _DT[t.dtype]
 
+    def _product(self, t: torch.Tensor, name: str, act_dtype, rows: int, cols: int) -> int:
+        """A product operand: act [rows, cols] (returns 0) or float32 partial sums [splits, rows, cols] (returns splits)."""
+        if t.dim() == 3:
+            self._need(t, name, _F32, (t.shape[0], rows, cols))
+            return int(t.shape[0])
+        self._need(t, name, act_dtype, (rows, cols))
+        return 0
+
     # ------------------------------------------------------------------ kernels
     def embed(self, token_ids, table, out):
         dt = self._act(table, "table")
@@ -104,9 +113,8 @@ class HipKernels:
         self._need(h, "h", _F32)
         self._need(weight, "weight", out.dtype, (hid,))
         self._need(out, "out", None, (t, hid))
-        if delta is not None:
-            self._need(delta, "delta", out.dtype, (t, hid))
-        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), None, weight.data_ptr(), float(eps),
+        splits = self._product(delta, "delta", out.dtype, t, hid) if delta is not None else 0
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), splits, t, None, weight.data_ptr(), float(eps),
                   out.data_ptr(), t, hid, dt, self._stream())
 
     def rows_add_rmsnorm(self, h, delta, rows, weight, eps, out):
@@ -117,10 +125,9 @@ class HipKernels:
         self._need(rows, "rows", _I32, (r,))
         self._need(weight, "weight", out.dtype, (hid,))
         self._need(out, "out", None, (r, hid))
-        if delta is not None:
-            self._need(delta, "delta", out.dtype, (t, hid))
-        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), rows.data_ptr(), weight.data_ptr(), float(eps),
-                  out.data_ptr(), r, hid, dt, self._stream())
+        splits = self._product(delta, "delta", out.dtype, t, hid) if delta is not None else 0
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), splits, t, rows.data_ptr(), weight.data_ptr(),
+                  float(eps), out.data_ptr(), r, hid, dt, self._stream())
 
     def linear(self, x, w, bias, out):
         m, k = x.shape
@@ -133,18 +140,71 @@ class HipKernels:
         if out.dtype not in (x.dtype, _F32):
             raise TypeError(f"out must be {x.dtype} or float32, got {out.dtype}")
         self._need(out, "out", None, (m, n))
+        if m == 0:
+            return out
+        if x.dtype == _BF16 and k % 8 == 0:
+            to_f32 = out.dtype == _F32
+            if m <= 64 or to_f32:
+                # weight-streaming MFMA kernel; more than 64 rows with float32 output (logits at many places)
+                # go through it 64 rows at a time
+                for r0 in range(0, m, 64):
+                    r1 = min(m, r0 + 64)
+                    xo, oo = x[r0:r1], out[r0:r1]
+                    self._run("egpt_gemm_skinny", xo.data_ptr(), w.data_ptr(), self._ptr(bias),
+                              oo.data_ptr() if to_f32 else None, None if to_f32 else oo.data_ptr(), r1 - r0, n, k, 1,
+                              self._stream())
+                return out
+            # many rows: the library's matrix product (the reference uses cuBLAS for every linear layer)
+            if bias is None:
+                torch.mm(x, w.t(), out=out)
+            else:
+                torch.addmm(bias, x, w.t(), out=out)
+            return out
         self._run("egpt_linear", x.data_ptr(), w.data_ptr(), self._ptr(bias), out.data_ptr(), m, n, k, dt,
                   1 if out.dtype == _F32 else 0, self._stream())
+        return out
+
+    @staticmethod
+    def _n_splits(m: int, n: int, k: int) -> int:
+        """How many workgroups share the k range of a skinny product: enough to fill the GPU when n is small,
+        bounded so that the partial sums stay smaller than the weights they came from."""
+        steps = -(-k // 128)
+        n_blocks = -(-n // 64)
+        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)))
+        per = -(-steps // s)
+        return -(-steps // per)
+
+    def product(self, x, w):
+        """x w^T for a consumer that takes partial sums: returns act [m, n], or float32 [splits, m, n] whose sum
+        over splits is the product (few rows in bfloat16: the k range is split over workgroups)."""
+        m, k = x.shape
+        n = w.shape[0]
+        if x.dtype == _BF16 and 0 < m <= 64 and k % 8 == 0:
+            self._need(x, "x")
+            self._need(w, "w", x.dtype, (n, k))
+            s = self._n_splits(m, n, k)
+            out = torch.empty((s, m, n), dtype=_F32, device=x.device)
+            self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s,
+                      self._stream())
+            return out
+        out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+        return self.linear(x, w, None, out)
 
     def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
-                       page_size):
-        t = qkv.shape[0]
+                       page_size, out=None):
+        """qkv: act [T, W] or float32 partial sums [S, T, W]; out: act [T, W] (default: qkv itself, in place)."""
         width = (nq + 2 * nkv) * hd
-        dt = self._act(qkv, "qkv")
-        self._need(qkv, "qkv", None, (t, width))
+        t = qkv.shape[-2]
+        if out is None:
+            if qkv.dim() == 3:
+                raise ValueError("partial sums need an output tensor")
+            out = qkv
+        dt = self._act(out, "out")
+        self._need(out, "out", None, (t, width))
+        splits = self._product(qkv, "qkv", out.dtype, t, width)
         self._need(positions, "positions", _I32, (t,))
         if bias is not None:
-            self._need(bias, "bias", qkv.dtype, (width,))
+            self._need(bias, "bias", out.dtype, (width,))
         if rotary_dim:
             if rotary_dim % 2 or rotary_dim > hd:
                 raise ValueError(f"rotary_dim {rotary_dim} must be even and <= head size {hd}")
@@ -152,12 +212,13 @@ class HipKernels:
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
-                self._need(c, name, qkv.dtype)
+                self._need(c, name, out.dtype)
                 if c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, hd):
                     raise ValueError(f"{name} must be [pages, {nkv}, {page_size}, {hd}], got {tuple(c.shape)}")
-        self._run("egpt_qkv_rope_store", qkv.data_ptr(), self._ptr(bias), positions.data_ptr(),
+        self._run("egpt_qkv_rope_store", qkv.data_ptr(), splits, out.data_ptr(), self._ptr(bias), positions.data_ptr(),
                   self._ptr(inv_freq) if rotary_dim else None, int(rotary_dim), self._ptr(slots),
                   self._ptr(k_cache), self._ptr(v_cache), t, nq, nkv, hd, page_size, dt, self._stream())
+        return out
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd, page_size,
                         scale, window, max_q_len, max_kv_len):
@@ -184,9 +245,9 @@ class HipKernels:
     def swiglu(self, gate_up, out):
         t, inter = out.shape
         dt = self._act(out, "out")
-        self._need(gate_up, "gate_up", out.dtype, (t, 2 * inter))
+        splits = self._product(gate_up, "gate_up", out.dtype, t, 2 * inter)
         self._need(out, "out")
-        self._run("egpt_swiglu", gate_up.data_ptr(), out.data_ptr(), t, inter, dt, self._stream())
+        self._run("egpt_swiglu", gate_up.data_ptr(), splits, out.data_ptr(), t, inter, dt, self._stream())
 
     def argmax(self, logits, out):
         r, v = logits.shape

@@ -91,8 +91,9 @@ class GQAttention(Mixer):
     def forward(self, x, ctx, cache, state=None):
         k = kernels.backend()
         t = x.shape[0]
-        qkv = torch.empty((t, self.q_size + 2 * self.kv_size), dtype=x.dtype, device=x.device)
-        k.linear(x, self.w_qkv, None, qkv)
+        width = self.q_size + 2 * self.kv_size
+        prod = k.product(x, self.w_qkv)                 # act [T, W], or float32 partial sums [S, T, W]
+        qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=x.dtype, device=x.device)
         slots = cache.slots if cache.writes else None
         rot = self.position.rotary(x.device)
         common = dict(
@@ -101,22 +102,24 @@ class GQAttention(Mixer):
         )
         if rot is not None:
             inv_freq, rotary_dim = rot
-            k.qkv_rope_store(qkv, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, **common)
+            k.qkv_rope_store(prod, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, out=qkv, **common)
         else:
             # bias, then the position encoding's own transform, then the store
-            if self.b_qkv is not None:
-                k.qkv_rope_store(qkv, self.b_qkv, ctx.positions, None, 0, None, **common)
+            if self.b_qkv is not None or prod.dim() == 3:
+                k.qkv_rope_store(prod, self.b_qkv, ctx.positions, None, 0, None, out=qkv, **common)
             q_view = qkv[:, : self.q_size].view(t, self.n_heads, self.head_dim)
             k_view = qkv[:, self.q_size : self.q_size + self.kv_size].view(t, self.n_kv_heads, self.head_dim)
             self.position.apply(q_view, k_view, ctx.positions)
             if slots is not None:
-                k.qkv_rope_store(qkv, None, ctx.positions, None, 0, slots, **common)
+                k.qkv_rope_store(qkv, None, ctx.positions, None, 0, slots, out=qkv, **common)
         attn = torch.empty((t, self.q_size), dtype=x.dtype, device=x.device)
         k.paged_attention(
             qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
             nq=self.n_heads, nkv=self.n_kv_heads, hd=self.head_dim, page_size=cache.page_size,
             scale=self.scale, window=self.window or 0, max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len,
         )
+        if self.b_o is None:
+            return k.product(attn, self.w_o)            # the residual add that follows sums partial sums up
         out = torch.empty((t, self.hidden_size), dtype=x.dtype, device=x.device)
         k.linear(attn, self.w_o, self.b_o, out)
         return out

@@ -41,13 +41,10 @@ class SwiGLU(FeedForward):
     def forward(self, x, ctx=None):
         k = kernels.backend()
         t = x.shape[0]
-        gate_up = torch.empty((t, 2 * self.intermediate_size), dtype=x.dtype, device=x.device)
-        k.linear(x, self.w_gate_up, None, gate_up)
+        gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]
         act = torch.empty((t, self.intermediate_size), dtype=x.dtype, device=x.device)
         k.swiglu(gate_up, act)
-        out = torch.empty((t, self.hidden_size), dtype=x.dtype, device=x.device)
-        k.linear(act, self.w_down, None, out)
-        return out
+        return k.product(act, self.w_down)               # added to the residual stream by the next norm
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -14,13 +14,24 @@ import torch
 F64 = torch.float64
 
 
+def _whole(t):
+    """A product operand: a tensor, or float32 partial sums [splits, rows, cols] to be added up."""
+    return t.sum(0) if t is not None and t.dim() == 3 else t
+
+
 class EmulatedKernels:
     name = "emulated"
+
+    def product(self, x, w):
+        out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype)
+        self.linear(x, w, None, out)
+        return out
 
     def embed(self, token_ids, table, out):
         out.copy_(table[token_ids.long()].to(out.dtype))
 
     def add_rmsnorm(self, h, delta, weight, eps, out):
+        delta = _whole(delta)
         if delta is not None:
             h.add_(delta.to(h.dtype))
         x = h.to(F64)
@@ -28,6 +39,7 @@ class EmulatedKernels:
         out.copy_((x * inv * weight.to(F64)).to(out.dtype))
 
     def rows_add_rmsnorm(self, h, delta, rows, weight, eps, out):
+        delta = _whole(delta)
         x = h[rows.long()].to(F64)
         if delta is not None:
             x = (h[rows.long()] + delta[rows.long()].to(h.dtype)).to(F64)
@@ -41,9 +53,11 @@ class EmulatedKernels:
         out.copy_(y.to(out.dtype))
 
     def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
-                       page_size):
+                       page_size, out=None):
+        src = _whole(qkv)
+        qkv = src if out is None else out
         t = qkv.shape[0]
-        x = qkv.to(F64)
+        x = src.to(F64)
         if bias is not None:
             x = x + bias.to(F64)
         heads = x.view(t, nq + 2 * nkv, hd).clone()
@@ -64,6 +78,7 @@ class EmulatedKernels:
             for i in range(t):
                 k_cache[page[i], :, off[i], :] = k_new[i]
                 v_cache[page[i], :, off[i], :] = v_new[i]
+        return qkv
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd,
                         page_size, scale, window, max_q_len, max_kv_len):
@@ -87,6 +102,7 @@ class EmulatedKernels:
                     out[s + i, h * hd : (h + 1) * hd] = (pr @ vals).to(out.dtype)
 
     def swiglu(self, gate_up, out):
+        gate_up = _whole(gate_up)
         i = out.shape[1]
         g, u = gate_up[:, :i].to(F64), gate_up[:, i:].to(F64)
         out.copy_((u * g / (1.0 + torch.exp(-g))).to(out.dtype))

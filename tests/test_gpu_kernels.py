@@ -83,6 +83,75 @@ def test_linear(k, dtype, m, n, kk):
     assert float((out.double().cpu() - (ref - b.double().cpu())).abs().max()) <= 3e-6 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("m,n,kk", [(1, 75, 104), (8, 1152, 896), (16, 896, 4864), (17, 130, 96), (33, 1000, 200),
+                                    (64, 9728, 896), (5, 777, 120), (48, 64, 4864), (8, 151936, 896)])
+def test_skinny_product_and_partial_sums(k, m, n, kk):
+    # the bfloat16 product for few rows: direct (float32 and bfloat16 output, with bias) and split over k
+    dtype = torch.bfloat16
+    x, w, b = rnd(m, kk, dtype=dtype, seed=1), rnd(n, kk, dtype=dtype, seed=2, scale=0.1), rnd(n, dtype=dtype, seed=3)
+    ref = plain.linear(x.double().cpu(), w.double().cpu())
+    scale = float(ref.abs().max())
+    prod = k.product(x, w)
+    assert prod.dtype == torch.float32 and prod.dim() == 3 and prod.shape[1:] == (m, n)
+    assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale
+    for s in sorted({1, 2, min(3, -(-kk // 128)), -(-kk // 128)}):
+        steps = -(-kk // 128)
+        if s > steps or (s - 1) * -(-steps // s) >= steps:
+            continue
+        out = torch.full((s, m, n), 7.0, dtype=torch.float32, device=DEV)
+        k._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, kk, s, k._stream())
+        assert float((out.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale, s
+    out32 = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    k.linear(x, w, b, out32)
+    assert float((out32.double().cpu() - ref - b.double().cpu()).abs().max()) <= 3e-6 * scale
+    out16 = torch.empty(m, n, dtype=dtype, device=DEV)
+    k.linear(x, w, b, out16)
+    assert float((out16.double().cpu() - ref - b.double().cpu()).abs().max()) <= 1e-2 * scale
+
+
+def test_consumers_add_partial_sums_up(k):
+    # residual add + norm, SwiGLU and the QKV epilogue take float32 partial sums [splits, rows, cols]
+    dtype = torch.bfloat16
+    t, hid = 5, 200
+    parts = rnd(3, t, hid, seed=1)
+    h = rnd(t, hid, seed=2)
+    h0 = h.clone()
+    w = (1 + rnd(hid, seed=3, scale=0.1)).to(dtype)
+    out = torch.empty(t, hid, dtype=dtype, device=DEV)
+    k.add_rmsnorm(h, parts, w, 1e-6, out)
+    summed = h0 + (parts[0] + parts[1] + parts[2])
+    assert torch.equal(h, summed)
+    ref = plain.rms_norm(summed.double().cpu(), w.double().cpu(), 1e-6)
+    assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    rows = torch.tensor([4, 0], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(2, hid, dtype=dtype, device=DEV)
+    k.rows_add_rmsnorm(h0.clone(), parts, rows, w, 1e-6, out2)
+    assert float((out2.double().cpu() - ref[[4, 0]]).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    gu = rnd(2, t, 2 * 96, seed=4, scale=2.0)
+    act = torch.empty(t, 96, dtype=dtype, device=DEV)
+    k.swiglu(gu, act)
+    g, u = (gu[0] + gu[1])[:, :96].double().cpu(), (gu[0] + gu[1])[:, 96:].double().cpu()
+    refa = u * g / (1 + torch.exp(-g))
+    assert float((act.double().cpu() - refa).abs().max()) <= 1.6e-2 * float(refa.abs().max())
+    nq, nkv, hd, ps = 3, 1, 32, 4
+    width = (nq + 2 * nkv) * hd
+    qp = rnd(2, t, width, seed=5)
+    bias = rnd(width, dtype=dtype, seed=6)
+    positions = torch.arange(10, 10 + t, dtype=torch.int32, device=DEV)
+    inv = torch.pow(torch.tensor(1e4), -2.0 * torch.arange(hd // 2, dtype=torch.float32) / hd).to(DEV)
+    slots = torch.tensor([3, 9, 0, 14, 7], dtype=torch.int32, device=DEV)
+    kc = torch.zeros(4, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    got = torch.empty(t, width, dtype=dtype, device=DEV)
+    k.qkv_rope_store(qp, bias, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=got)
+    x = ((qp[0] + qp[1]).double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
+    refq = x.clone()
+    refq[:, : nq + nkv] = plain.rope(x[:, : nq + nkv], positions.cpu(), 1e4)
+    assert float((got.double().cpu().view(t, -1, hd) - refq).abs().max()) <= 1.6e-2 * float(refq.abs().max())
+    assert torch.equal(kc[0, :, 3, :], got.view(t, -1, hd)[0, nq : nq + nkv])
+    assert torch.equal(vc[3, :, 2, :], got.view(t, -1, hd)[3, nq + nkv :])
+
+
 def test_linear_vector_of_the_reference(k):
     # /root/reference/test/matmul_3d_test.cpp:60-87
     x = torch.tensor([[1.0, 2, 3], [4, 5, 6]], device=DEV)

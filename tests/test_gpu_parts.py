@@ -17,6 +17,11 @@ def tol(dtype):
     return 5e-6 if dtype == torch.float32 else 2e-2
 
 
+def whole(t):
+    """A part may hand back float32 partial sums [splits, T, H] of its last product; their sum is the output."""
+    return t.double().sum(0) if t.dim() == 3 else t.double()
+
+
 def weights_for(part, dtype, seed=0, scale=0.05):
     g = torch.Generator().manual_seed(seed)
     w = {}
@@ -58,8 +63,8 @@ def test_swiglu_part(dtype):
     w = weights_for(ff, dtype, scale=0.2)
     x = torch.randn(9, 72, generator=torch.Generator().manual_seed(3)).to(dtype)
     ref = plain.swiglu_mlp(x.double(), w, "m.")
-    out = ff.forward(x.to(DEV))
-    assert float((out.double().cpu() - ref).abs().max()) <= tol(dtype) * float(ref.abs().max())
+    out = whole(ff.forward(x.to(DEV)))
+    assert float((out.cpu() - ref).abs().max()) <= tol(dtype) * float(ref.abs().max())
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -114,14 +119,14 @@ def test_attention_part_whole_and_cut(dtype, nq, nkv, hd, hidden, window, bias, 
         ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(n), kv_len=one(pos + n), max_q_len=n,
                               max_kv_len=pos + n)
         cache = CacheView(kc, vc, ps, table, slots, window, True)
-        outs.append(att.forward(x[pos : pos + n].to(DEV), ctx, cache, None))
+        outs.append(whole(att.forward(x[pos : pos + n].to(DEV), ctx, cache, None)))
         pos += n
-    out = torch.cat(outs).double().cpu()
+    out = torch.cat(outs).cpu()
     assert float((out - ref).abs().max()) <= tol(dtype) * float(ref.abs().max())
     # a reader of the same cache that does not write (another layer's cache): same result for the last portion
     cache_ro = CacheView(kc, vc, ps, table, slots, window, False)
     kc_before = kc.clone()
-    again = att.forward(x[pos - n : pos].to(DEV), ctx, cache_ro, None)
+    again = whole(att.forward(x[pos - n : pos].to(DEV), ctx, cache_ro, None))
     assert torch.equal(kc, kc_before) and torch.equal(again, outs[-1])
 
 
@@ -155,6 +160,6 @@ def test_pre_norm_block(dtype):
     ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(s), kv_len=one(s), max_q_len=s, max_kv_len=s)
     h = x.to(DEV).clone()
     delta = block.forward(h, None, ctx, CacheView(kc, vc, ps, table, slots, None, True), None)
-    got = h.double().cpu() + delta.double().cpu()
+    got = h.double().cpu() + whole(delta).cpu()
     assert float((h.double().cpu() - a).abs().max()) <= tol(dtype) * float(a.abs().max())
     assert float((got - y).abs().max()) <= tol(dtype) * float(y.abs().max())
