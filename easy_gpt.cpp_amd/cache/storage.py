@@ -7,20 +7,24 @@ from ..parts.base import CacheNeed, StateNeed
 
 
 class KVStorage:
-    """For each group, keys and values as [slabs, num_pages, n_kv_heads, page_size, head_dim].
+    """For each group, keys as [slabs, num_pages, n_kv_heads, page_size, head_dim] and values
+    transposed within a page, [slabs, num_pages, n_kv_heads, head_dim, page_size].
 
-    Within a page one head's tokens are contiguous (page_size * head_dim elements), which
-    is what the attention kernels stream.  Pages are never cleared: a kernel reads only
-    positions below a request's length."""
+    One head's part of a page is contiguous in both.  A key's features are contiguous (the
+    score product sums over features); a feature's values over the page's tokens are
+    contiguous (the output product sums over tokens): each is the order in which the matrix
+    cores take their operands, so the attention kernels load them as they lie.  Pages are
+    never cleared: a kernel reads only positions below a request's length."""
 
     def __init__(self, groups, slabs_per_group, num_pages, page_size: int, dtype: torch.dtype, device):
         self.page_size = page_size
         self.k: list[torch.Tensor] = []
         self.v: list[torch.Tensor] = []
         for need, n_slabs, pages in zip(groups, slabs_per_group, num_pages):
-            shape = (n_slabs, pages, need.n_kv_heads, page_size, need.head_dim)
-            self.k.append(torch.zeros(shape, dtype=dtype, device=device))
-            self.v.append(torch.zeros(shape, dtype=dtype, device=device))
+            k_shape = (n_slabs, pages, need.n_kv_heads, page_size, need.head_dim)
+            v_shape = (n_slabs, pages, need.n_kv_heads, need.head_dim, page_size)
+            self.k.append(torch.zeros(k_shape, dtype=dtype, device=device))
+            self.v.append(torch.zeros(v_shape, dtype=dtype, device=device))
 
     def slab(self, group: int, index: int):
         return self.k[group][index], self.v[group][index]

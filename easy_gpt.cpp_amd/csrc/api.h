@@ -34,6 +34,14 @@ int egpt_paged_attention(const void* qkv, void* out, const void* k_cache, const 
                          const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int hd, int page_size,
                          float scale, int window, int dtype, void* stream);
+// The same on the matrix cores: bfloat16, head size 64 or 128, page size a multiple of 16.  With n_splits > 1
+// the key range of every request is split and part_o [n_splits][n_tokens][nq][hd], part_ml
+// [n_splits][n_tokens][nq][2] (float32) hold the partial results that a second kernel combines.
+int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                              const void* v_cache, const int32_t* block_table, int table_width,
+                              const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
+                              int n_tokens, int nq, int nkv, int hd, int page_size, float scale, int window,
+                              int n_splits, int rows_per_wave, void* stream);
 int egpt_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                 const float* uniform, int32_t* out, int n_rows, int vocab, void* stream);

@@ -5,7 +5,8 @@
 // (causal key limit as /root/reference/src/cuda/ops/self_attn_detail.cuh:695-751), and j > p - window
 // when a window is set.  score = (q . k) * scale, online softmax with float32 running maximum, sum and
 // accumulator (/root/reference/src/cuda/ops/self_attn_detail.cuh:299-383); query head h reads kv head
-// h / (nq / nkv) (:669).  Keys and values lie in pages [page][kv head][offset][hd] and are found
+// h / (nq / nkv) (:669).  Keys lie in pages [page][kv head][offset][hd], values in pages
+// [page][kv head][hd][offset], and are found
 // through the request's block table; nothing beyond kv_len is ever read, so pages need no clearing.
 #include "api.h"
 #include "common.h"
@@ -55,8 +56,9 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
         long off = 0;
         if (j < hi) {
             const long page = table[j / page_size];
-            off = ((page * nkv + kvh) * page_size + (j % page_size)) * hd;
-            const T* kr = k_cache + off;
+            const long head_base = (page * nkv + kvh) * page_size * hd;   // same for keys and values
+            off = head_base + (j % page_size);                          // values: [feature][offset]
+            const T* kr = k_cache + head_base + (j % page_size) * hd;     // keys: [offset][feature]
             float dot = 0.f;
             for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float(kr[d]), dot);
             s = dot * scale;
@@ -75,7 +77,8 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
             const int d = lane + r * kWave;
             if (d < hd) {
                 float a = acc[r] * alpha;
-                for (int jj = 0; jj < n_valid; ++jj) a = fmaf(p_s[jj], to_float(v_cache[v_off_s[jj] + d]), a);
+                for (int jj = 0; jj < n_valid; ++jj)
+                    a = fmaf(p_s[jj], to_float(v_cache[v_off_s[jj] + static_cast<long>(d) * page_size]), a);
                 acc[r] = a;
             }
         }

@@ -1,0 +1,285 @@
+// Paged attention on the matrix cores (bfloat16), for prompt portions and decoded tokens alike.
+//
+// A wavefront owns QT tiles of 16 query rows of one request and one key/value head.  A row is a
+// (token, query head) pair of the head's group, token-major, so the 7 heads of a decoded token share one
+// tile (and every load of its keys), and the rows of a prompt tile have nearly the same causal limit.
+// Keys are walked 32 at a time.  The scores are computed transposed,
+//     S^T[key, row] = K[key, :] . Q[row, :]        v_mfma_f32_16x16x32_bf16, A = K, B = Q
+// so that a lane ends up with the scores of ONE row (its column) for four keys per tile: the row's
+// running maximum and sum are per-lane scalars, and the probabilities are, as they lie in registers,
+// the B operand of the second product
+//     O^T[feature, row] += V^T[feature, key] . P^T[key, row]     A = V^T, B = P^T
+// whose A operand is what a page of values looks like in memory (values are stored transposed within
+// a page).  No operand passes through LDS.  Softmax statistics and the accumulator are float32
+// (as /root/reference/src/cuda/ops/self_attn_detail.cuh:299-383); P is rounded to bfloat16 for the
+// second product.  With n_splits > 1 each split of the key range writes an unnormalised partial result
+// and its (maximum, sum), which attention_reduce_kernel combines.
+#include "api.h"
+#include "common.h"
+
+namespace egpt {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <int HD, int QT>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int n_tokens, int nq, int nkv,
+    int page_size, float scale, int window, int n_splits) {
+    constexpr int KD = HD / 32;  // score MFMAs per key tile (32 features each)
+    constexpr int DT = HD / 16;  // output feature tiles
+    const int lane = threadIdx.x, lj = lane % 16, lg = lane / 16;
+    const int kh = blockIdx.y, split = blockIdx.z;
+    const int group_size = nq / nkv;
+
+    // which request, and which group of 16*QT rows of it
+    int b = 0, grp = blockIdx.x;
+    for (; b < n_seqs; ++b) {
+        const int groups = (q_len[b] * group_size + 16 * QT - 1) / (16 * QT);
+        if (grp < groups) break;
+        grp -= groups;
+    }
+    if (b >= n_seqs) return;
+    const int n = q_len[b], kv = kv_len[b], qs = q_start[b];
+    const int rows = n * group_size;
+    const int row_base = grp * 16 * QT;
+    const int width = (nq + 2 * nkv) * HD;
+    const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+
+    // this lane's row in each tile
+    bool valid[QT];
+    int tok[QT], head[QT], p_row[QT], lo_row[QT];
+    bf16x8 q[QT][KD];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        const int r = row_base + t * 16 + lj;
+        valid[t] = r < rows;
+        const int i = valid[t] ? r / group_size : 0;
+        tok[t] = qs + i;
+        head[t] = kh * group_size + (valid[t] ? r % group_size : 0);
+        p_row[t] = valid[t] ? kv - n + i : -1;
+        lo_row[t] = (window > 0 && valid[t]) ? max(0, p_row[t] - window + 1) : 0;
+        const bf16_t* qp = qkv + static_cast<size_t>(tok[t]) * width + head[t] * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            uint4 v = valid[t] ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+            q[t][kd] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    // key blocks (32 keys) this wave needs, and this split's share of them
+    const int last_row = min(rows, row_base + 16 * QT) - 1;
+    const int p_hi = kv - n + last_row / group_size;
+    const int first_pos = kv - n + row_base / group_size;
+    const int lo_first = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int kb_begin = lo_first / 32, kb_end = p_hi / 32 + 1;
+    const int per_split = (kb_end - kb_begin + n_splits - 1) / n_splits;
+    const int my_begin = kb_begin + split * per_split;
+    const int my_end = min(kb_end, my_begin + per_split);
+
+    f32x4 o[QT][DT];
+    float m_run[QT], l_run[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        m_run[t] = -INFINITY;
+        l_run[t] = 0.f;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) o[t][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    uint4 k_cur[2][KD], k_nxt[2][KD];
+    uint2 v_cur[2][DT], v_nxt[2][DT];
+    auto load_block = [&](uint4 (*kk)[KD], uint2 (*vv)[DT], int kb) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int key0 = kb * 32 + kt * 16;
+            // a tile is read only if some row of this wave can see one of its keys: then it lies in a page the
+            // request still holds (p_hi < kv; pages wholly behind the window may have been given back)
+            bool live = key0 <= p_hi && key0 + 15 >= lo_first;
+            long page = 0;
+            int off = 0;
+            if (live) {
+                page = table[key0 / page_size];
+                off = key0 % page_size;
+                live = page >= 0;
+                page = live ? page : 0;
+            }
+            const bf16_t* kp = k_cache + ((page * nkv + kh) * page_size + off + lj) * HD + lg * 8;
+            const bf16_t* vp = v_cache + ((page * nkv + kh) * HD + lj) * static_cast<long>(page_size) + off + lg * 4;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd)
+                kk[kt][kd] = live ? *reinterpret_cast<const uint4*>(kp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+                vv[kt][d] = live ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
+                                 : uint2{0u, 0u};
+        }
+    };
+
+    if (my_begin < my_end) load_block(k_cur, v_cur, my_begin);
+    for (int kb = my_begin; kb < my_end; ++kb) {
+        if (kb + 1 < my_end) load_block(k_nxt, v_nxt, kb + 1);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+            float s[2][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k_cur[kt][kd]), q[t][kd],
+                                                                  acc, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = kb * 32 + kt * 16 + lg * 4 + v;
+                    const bool vis = key <= p_row[t] && key >= lo_row[t];
+                    s[kt][v] = vis ? acc[v] * scale : -INFINITY;
+                    mx = fmaxf(mx, s[kt][v]);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+            const float m_new = fmaxf(m_run[t], mx);
+            const bool none = m_new == -INFINITY;             // no visible key yet for this row
+            const float alpha = none ? 1.f : __expf(m_run[t] - m_new);
+            float sum = 0.f;
+            bf16x8 pb;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float pv = none ? 0.f : __expf(s[kt][v] - m_new);
+                    sum += pv;
+                    pb[kt * 4 + v] = static_cast<__bf16>(pv);
+                }
+            l_run[t] = l_run[t] * alpha + sum;
+            m_run[t] = m_new;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                const uint4 a = uint4{v_cur[0][d].x, v_cur[0][d].y, v_cur[1][d].x, v_cur[1][d].y};
+                f32x4 acc = o[t][d];
+                acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+                o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb, acc, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) k_cur[kt][kd] = k_nxt[kt][kd];
+#pragma unroll
+            for (int d = 0; d < DT; ++d) v_cur[kt][d] = v_nxt[kt][d];
+        }
+    }
+
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        float l = l_run[t];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        if (!valid[t]) continue;
+        const size_t row = static_cast<size_t>(tok[t]) * nq + head[t];
+        if (n_splits == 1) {
+            const float inv = 1.0f / l;
+            bf16_t* op = out + row * HD + lg * 4;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                uint2 packed;
+                packed.x = f32_to_bf16_bits(o[t][d][0] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[t][d][1] * inv)) << 16);
+                packed.y = f32_to_bf16_bits(o[t][d][2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[t][d][3] * inv)) << 16);
+                *reinterpret_cast<uint2*>(op + d * 16) = packed;
+            }
+        } else {
+            const size_t prow = static_cast<size_t>(split) * n_tokens * nq + row;
+            float* pp = part_o + prow * HD + lg * 4;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) *reinterpret_cast<f32x4*>(pp + d * 16) = o[t][d];
+            if (lg == 0) {
+                part_ml[prow * 2] = m_run[t];
+                part_ml[prow * 2 + 1] = l;
+            }
+        }
+    }
+}
+
+// out[row, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits; one wavefront per row.
+__global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __restrict__ part_o,
+                                                              const float* __restrict__ part_ml,
+                                                              bf16_t* __restrict__ out, int n_rows, int hd, int n_splits) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    float m_max = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, part_ml[(static_cast<size_t>(s) * n_rows + row) * 2]);
+    float denom = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < n_splits; ++s) {
+        const size_t pr = static_cast<size_t>(s) * n_rows + row;
+        const float m = part_ml[pr * 2];
+        if (m == -INFINITY) continue;              // a split without visible keys
+        const float wgt = __expf(m - m_max);
+        denom += wgt * part_ml[pr * 2 + 1];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int d = lane + r * kWave;
+            if (d < hd) acc[r] += wgt * part_o[pr * hd + d];
+        }
+    }
+    const float inv = 1.0f / denom;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int d = lane + r * kWave;
+        if (d < hd) out[static_cast<size_t>(row) * hd + d] = from_float<bf16_t>(acc[r] * inv);
+    }
+}
+
+template <int HD, int QT>
+static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                       const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
+                       const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
+                       int page_size, float scale, int window, int n_splits, hipStream_t s) {
+    const int group = nq / nkv;
+    const long groups = (static_cast<long>(n_tokens) * group) / (16 * QT) + n_seqs;   // upper bound
+    dim3 grid(static_cast<unsigned>(groups), nkv, n_splits);
+    attention_mfma_kernel<HD, QT><<<grid, 64, 0, s>>>(
+        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
+        static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
+        q_len, kv_len, n_seqs, n_tokens, nq, nkv, page_size, scale, window, n_splits);
+    EGPT_CHECK_LAUNCH();
+    if (n_splits > 1) {
+        attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
+                                                             HD, n_splits);
+        EGPT_CHECK_LAUNCH();
+    }
+    return EGPT_OK;
+}
+
+}  // namespace egpt
+
+using namespace egpt;
+
+// bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.
+// part_o [n_splits][n_tokens][nq][hd] and part_ml [n_splits][n_tokens][nq][2] float32 are needed when n_splits > 1.
+extern "C" int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                                         const void* v_cache, const int32_t* block_table, int table_width,
+                                         const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len,
+                                         int n_seqs, int n_tokens, int nq, int nkv, int hd, int page_size, float scale,
+                                         int window, int n_splits, int rows_per_wave, void* stream) {
+    if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
+        return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 ||
+        n_splits < 1 || (n_splits > 1 && (!part_o || !part_ml)))
+        return EGPT_BAD_ARGUMENT;
+    if ((hd != 64 && hd != 128) || page_size % 16 != 0 || nkv > 65535 || n_splits > 65535 ||
+        (rows_per_wave != 16 && rows_per_wave != 32))
+        return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define EGPT_ATTN_ARGS                                                                                              \
+    qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len, n_seqs, n_tokens, \
+        nq, nkv, page_size, scale, window, n_splits, s
+    if (hd == 64) return rows_per_wave == 16 ? launch_mfma<64, 1>(EGPT_ATTN_ARGS) : launch_mfma<64, 2>(EGPT_ATTN_ARGS);
+    return rows_per_wave == 16 ? launch_mfma<128, 1>(EGPT_ATTN_ARGS) : launch_mfma<128, 2>(EGPT_ATTN_ARGS);
+#undef EGPT_ATTN_ARGS
+}

@@ -86,7 +86,7 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
 // (i, i + rotary_dim/2), angle = float(position) * inv_freq[i], cos/sin in float32
 // (/root/reference/src/ops.cpp:404-420, /root/reference/src/cuda/ops/self_attn_detail.cuh:512-541);
 // write the result back in place and store keys and values at their slot of the paged cache
-// [page][kv head][offset][hd].
+// (keys [page][kv head][offset][hd], values [page][kv head][hd][offset]).
 template <typename T>
 __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv_out, const T* __restrict__ bias,
                                       const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
@@ -120,9 +120,13 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv
         if (slot >= 0 && head >= nq) {
             const bool is_k = head < nq + nkv;
             const int kvh = is_k ? head - nq : head - nq - nkv;
-            T* dst = (is_k ? k_cache : v_cache) + ((page * nkv + kvh) * page_size + off) * hd;
-            dst[d] = ta;
-            if (rotated) dst[d + half] = tb;
+            if (is_k) {   // keys: [page][kv head][offset][feature]
+                T* dst = k_cache + ((page * nkv + kvh) * page_size + off) * hd;
+                dst[d] = ta;
+                if (rotated) dst[d + half] = tb;
+            } else {      // values: [page][kv head][feature][offset]
+                v_cache[((page * nkv + kvh) * hd + d) * page_size + off] = ta;
+            }
         }
     }
 }

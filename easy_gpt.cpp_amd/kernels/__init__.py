@@ -19,7 +19,8 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
                  rotary_dim, slots i32[T]|None, k_cache, v_cache, nq, nkv, hd, page_size)
         adds bias, rotates the first rotary_dim features of every query and key head
         (pairs (i, i + rotary_dim/2), angle = position * inv_freq[i]) in place, and stores
-        keys and values at `slots` (page * page_size + offset) of caches [P,nkv,page_size,hd]
+        keys and values at `slots` (page * page_size + offset) of the caches, keys [P,nkv,page_size,hd],
+        values [P,nkv,hd,page_size]
   paged_attention(qkv, out act[T,nq*hd], k_cache, v_cache, block_table i32[B,W], q_start i32[B],
                   q_len i32[B], kv_len i32[B], nq, nkv, hd, page_size, scale, window,
                   max_q_len, max_kv_len)

@@ -50,6 +50,7 @@ class HipKernels:
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
+            "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp],
             "egpt_argmax": [vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
         }
@@ -88,6 +89,16 @@ class HipKernels:
         if t.dtype not in _DT:
             raise TypeError(f"{name} must be float32 or bfloat16, got {t.dtype}")
         return _DT[t.dtype]
+
+    def _caches(self, k_cache, v_cache, dtype, nkv: int, page_size: int, hd: int) -> None:
+        self._need(k_cache, "k_cache", dtype)
+        self._need(v_cache, "v_cache", dtype)
+        if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, hd):
+            raise ValueError(f"k_cache must be [pages, {nkv}, {page_size}, {hd}], got {tuple(k_cache.shape)}")
+        if v_cache.dim() != 4 or tuple(v_cache.shape[1:]) != (nkv, hd, page_size):
+            raise ValueError(f"v_cache must be [pages, {nkv}, {hd}, {page_size}], got {tuple(v_cache.shape)}")
+        if v_cache.shape[0] != k_cache.shape[0]:
+            raise ValueError("k_cache and v_cache must have the same number of pages")
 
     def _product(self, t: torch.Tensor, name: str, act_dtype, rows: int, cols: int) -> int:
         """A product operand: act [rows, cols] (returns 0) or float32 partial sums [splits, rows, cols] (returns splits)."""
@@ -211,10 +222,7 @@ class HipKernels:
             self._need(inv_freq, "inv_freq", _F32, (rotary_dim // 2,))
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
-            for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
-                self._need(c, name, out.dtype)
-                if c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, hd):
-                    raise ValueError(f"{name} must be [pages, {nkv}, {page_size}, {hd}], got {tuple(c.shape)}")
+            self._caches(k_cache, v_cache, out.dtype, nkv, page_size, hd)
         self._run("egpt_qkv_rope_store", qkv.data_ptr(), splits, out.data_ptr(), self._ptr(bias), positions.data_ptr(),
                   self._ptr(inv_freq) if rotary_dim else None, int(rotary_dim), self._ptr(slots),
                   self._ptr(k_cache), self._ptr(v_cache), t, nq, nkv, hd, page_size, dt, self._stream())
@@ -227,10 +235,7 @@ class HipKernels:
         dt = self._act(qkv, "qkv")
         self._need(qkv, "qkv", None, (t, (nq + 2 * nkv) * hd))
         self._need(out, "out", qkv.dtype, (t, nq * hd))
-        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
-            self._need(c, name, qkv.dtype)
-            if c.dim() != 4 or tuple(c.shape[1:]) != (nkv, page_size, hd):
-                raise ValueError(f"{name} must be [pages, {nkv}, {page_size}, {hd}], got {tuple(c.shape)}")
+        self._caches(k_cache, v_cache, qkv.dtype, nkv, page_size, hd)
         self._need(block_table, "block_table", _I32)
         for name, v in (("q_start", q_start), ("q_len", q_len), ("kv_len", kv_len)):
             self._need(v, name, _I32, (b,))
@@ -238,6 +243,21 @@ class HipKernels:
             raise ValueError(f"block table of width {width} cannot hold {max_kv_len} tokens at page size {page_size}")
         if hd > 256:
             raise ValueError(f"head size {hd} is not supported by the attention kernels (at most 256)")
+        if qkv.dtype == _BF16 and hd in (64, 128) and page_size % 16 == 0:
+            # matrix-core kernel; the key range is split when there are too few (request, kv head) pairs to fill
+            # the GPU, which is the case when only decoded tokens are in the batch
+            n_splits = 1
+            if max_q_len == 1:
+                n_splits = max(1, min(2048 // (b * nkv), -(-max_kv_len // 64), 64))
+            part_o = part_ml = None
+            if n_splits > 1:
+                part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)
+                part_ml = torch.empty((n_splits, t, nq, 2), dtype=_F32, device=qkv.device)
+            self._run("egpt_paged_attention_mfma", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
+                      self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
+                      q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, hd, page_size,
+                      float(scale), int(window), n_splits, 16 if max_q_len == 1 else 32, self._stream())
+            return
         self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
                   nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())

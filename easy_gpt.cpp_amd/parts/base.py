@@ -45,7 +45,8 @@ class StateNeed:
 class CacheView:
     """One cache slab as a mixer sees it during a step.
 
-    k, v         [num_pages, n_kv_heads, page_size, head_dim], act
+    k            [num_pages, n_kv_heads, page_size, head_dim], act
+    v            [num_pages, n_kv_heads, head_dim, page_size], act (transposed within a page)
     block_table  int32 [B, W]: page ids of each request in order (-1 where a page was given back)
     slots        int32 [T]: page * page_size + offset where each token of the step is stored
     """

@@ -38,7 +38,17 @@ TINY_C = {
     "use_sliding_window": True, "sliding_window": 24, "max_window_layers": 1,
     "bos_token_id": 3, "eos_token_id": 4, "torch_dtype": "float32",
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# A fourth one with the head size of the benchmark models (64), for which bfloat16 attention runs on the
+# matrix cores; query width 6 * 64 differs from the model width.
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 192, "num_attention_heads": 6, "num_key_value_heads": 2,
+    "head_dim": 64, "intermediate_size": 328, "vocab_size": 650, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 640, "hidden_act": "silu",
+    "use_sliding_window": True, "sliding_window": 40, "max_window_layers": 1,
+    "bos_token_id": 5, "eos_token_id": 6, "torch_dtype": "bfloat16",
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 @pytest.fixture(scope="session")

@@ -77,7 +77,7 @@ class EmulatedKernels:
             v_new = qkv.view(t, nq + 2 * nkv, hd)[:, nq + nkv :]
             for i in range(t):
                 k_cache[page[i], :, off[i], :] = k_new[i]
-                v_cache[page[i], :, off[i], :] = v_new[i]
+                v_cache[page[i], :, :, off[i]] = v_new[i]
         return qkv
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd,
@@ -96,7 +96,7 @@ class EmulatedKernels:
                 for h in range(nq):
                     kh = h // group
                     keys = k_cache[pages, kh, offs, :].to(F64)
-                    vals = v_cache[pages, kh, offs, :].to(F64)
+                    vals = v_cache[pages, kh, :, offs].to(F64)
                     sc = (keys @ q_all[s + i, h]) * scale
                     pr = torch.softmax(sc, dim=0)
                     out[s + i, h * hd : (h + 1) * hd] = (pr @ vals).to(out.dtype)

@@ -141,7 +141,7 @@ def test_consumers_add_partial_sums_up(k):
     inv = torch.pow(torch.tensor(1e4), -2.0 * torch.arange(hd // 2, dtype=torch.float32) / hd).to(DEV)
     slots = torch.tensor([3, 9, 0, 14, 7], dtype=torch.int32, device=DEV)
     kc = torch.zeros(4, nkv, ps, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(4, nkv, hd, ps, dtype=dtype, device=DEV)
     got = torch.empty(t, width, dtype=dtype, device=DEV)
     k.qkv_rope_store(qp, bias, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=got)
     x = ((qp[0] + qp[1]).double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
@@ -149,7 +149,7 @@ def test_consumers_add_partial_sums_up(k):
     refq[:, : nq + nkv] = plain.rope(x[:, : nq + nkv], positions.cpu(), 1e4)
     assert float((got.double().cpu().view(t, -1, hd) - refq).abs().max()) <= 1.6e-2 * float(refq.abs().max())
     assert torch.equal(kc[0, :, 3, :], got.view(t, -1, hd)[0, nq : nq + nkv])
-    assert torch.equal(vc[3, :, 2, :], got.view(t, -1, hd)[3, nq + nkv :])
+    assert torch.equal(vc[3, :, :, 2], got.view(t, -1, hd)[3, nq + nkv :])
 
 
 def test_linear_vector_of_the_reference(k):
@@ -188,7 +188,7 @@ def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta):
     perm = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(3))[:t]
     slots = perm.to(torch.int32).to(DEV)
     kc = torch.full((pages, nkv, ps, hd), 77.0, dtype=dtype, device=DEV)
-    vc = torch.full((pages, nkv, ps, hd), 77.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, nkv, hd, ps), 77.0, dtype=dtype, device=DEV)
     x = (qkv.double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
     k.qkv_rope_store(qkv, bias, positions, inv, rd, slots, kc, vc, nq, nkv, hd, ps)
     ang = (positions.cpu().float()[:, None] * inv.cpu()[None, :]).double()
@@ -204,7 +204,7 @@ def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta):
         p, o = int(perm[i]) // ps, int(perm[i]) % ps
         written[int(perm[i])] = True
         assert torch.equal(kc[p, :, o, :], qkv.view(t, -1, hd)[i, nq : nq + nkv])
-        assert torch.equal(vc[p, :, o, :], qkv.view(t, -1, hd)[i, nq + nkv :])
+        assert torch.equal(vc[p, :, :, o], qkv.view(t, -1, hd)[i, nq + nkv :])
     untouched = kc.permute(0, 2, 1, 3).reshape(pages * ps, -1)[~written]
     assert torch.all(untouched == 77.0)                          # nothing else was written
 
@@ -230,7 +230,7 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
     n_pages = sum(-(-kv // ps) for _, kv in seqs) + extra_pages
     order = torch.randperm(n_pages, generator=g).tolist()
     kc = torch.full((n_pages, nkv, ps, hd), 1e4, dtype=dtype)
-    vc = torch.full((n_pages, nkv, ps, hd), -1e4, dtype=dtype)
+    vc = torch.full((n_pages, nkv, hd, ps), -1e4, dtype=dtype)
     width = max(-(-kv // ps) for _, kv in seqs)
     table = torch.full((len(seqs), width), -1, dtype=torch.int32)
     keys, vals = [], []
@@ -244,7 +244,7 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
                 table[b, j // ps] = order.pop()
             pg = int(table[b, j // ps])
             kc[pg, :, j % ps, :] = kk[j]
-            vc[pg, :, j % ps, :] = vv[j]
+            vc[pg, :, :, j % ps] = vv[j]
     return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
 
 
@@ -272,7 +272,8 @@ def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(6, 3, 48, 4), (7, 1, 64, 16), (4, 4, 16, 5), (10, 5, 80, 16), (2, 1, 128, 64),
-                                           (3, 3, 256, 16)])
+                                           (3, 3, 256, 16), (14, 2, 64, 16), (12, 2, 128, 16), (5, 5, 64, 32),
+                                           (6, 2, 64, 4)])
 def test_paged_attention_ragged_batch(k, dtype, nq, nkv, hd, ps):
     # prompt portions (with and without a prefix in the cache) beside single decoded tokens
     seqs = [(1, 1), (9, 9), (1, 130), (7, 71), (2, 64), (1, 65), (33, 33), (3, 200)]
@@ -281,11 +282,22 @@ def test_paged_attention_ragged_batch(k, dtype, nq, nkv, hd, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd", [32, 64])
 @pytest.mark.parametrize("window", [1, 7, 64, 65])
-def test_paged_attention_window(k, dtype, window):
-    seqs = [(1, 100), (20, 90), (5, 5), (1, window), (1, window + 1), (3, 66)]
-    err = run_paged(k, seqs, 6, 2, 32, 16, dtype, window=window)
+def test_paged_attention_window(k, dtype, window, hd):
+    seqs = [(1, 100), (20, 90), (5, 5), (1, window), (1, window + 1), (3, 66), (40, 300)]
+    err = run_paged(k, seqs, 6, 2, hd, 16, dtype, window=window)
     assert err <= (2e-6 if dtype == torch.float32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(14, 2, 64), (12, 2, 128), (3, 1, 64)])
+@pytest.mark.parametrize("batch,ctx", [(1, 2113), (8, 700), (64, 130), (3, 33)])
+def test_paged_attention_decode_batches_split_the_key_range(k, nq, nkv, hd, batch, ctx):
+    # only decoded tokens, different lengths: the matrix-core kernel splits the keys and combines the parts
+    seqs = [(1, max(1, ctx - 37 * i % ctx)) for i in range(batch)]
+    err = run_paged(k, seqs, nq, nkv, hd, 16, torch.bfloat16)
+    assert err <= 1.2e-2
+    assert run_paged(k, seqs, nq, nkv, hd, 16, torch.bfloat16, q_scale=6.0) <= 4e-2
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -302,41 +314,51 @@ def test_paged_attention_one_far_key_stands_out(k):
     nq = nkv = 1
     hd, ps, kv = 32, 16, 500
     for far in (0, 15, 16, 255, 256, 498, 499):
+        for dtype, hd in ((torch.float32, 32), (torch.bfloat16, 64)):
+            _one_far_key(k, far, dtype, hd)
+
+
+def _one_far_key(k, far, dtype, hd):
+    nq = nkv = 1
+    ps, kv = 16, 500
+    if True:
         kk = torch.zeros(kv, 1, hd)
         vv = torch.randn(kv, 1, hd, generator=torch.Generator().manual_seed(far))
         kk[far, 0, 0] = 50.0
         pages = -(-kv // ps)
         kc = torch.zeros(pages, 1, ps, hd)
-        vc = torch.zeros(pages, 1, ps, hd)
+        vc = torch.zeros(pages, 1, hd, ps)
         table = torch.randperm(pages, generator=torch.Generator().manual_seed(1)).to(torch.int32)[None, :]
         for j in range(kv):
             kc[int(table[0, j // ps]), 0, j % ps] = kk[j, 0]
-            vc[int(table[0, j // ps]), 0, j % ps] = vv[j, 0]
+            vc[int(table[0, j // ps]), 0, :, j % ps] = vv[j, 0]
         qkv = torch.zeros(1, 3 * hd)
         qkv[0, 0] = 50.0
-        out = torch.empty(1, hd, device=DEV)
+        out = torch.empty(1, hd, device=DEV, dtype=dtype)
         one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
-        k.paged_attention(qkv.to(DEV), out, kc.to(DEV), vc.to(DEV), table.to(DEV), one(0), one(1), one(kv), 1, 1, hd, ps,
-                          1.0, 0, 1, kv)
-        assert float((out.cpu()[0] - vv[far, 0]).abs().max()) < 1e-5, far
+        vv = vv.to(dtype)
+        k.paged_attention(qkv.to(dtype).to(DEV), out, kc.to(dtype).to(DEV), vc.to(dtype).to(DEV), table.to(DEV), one(0),
+                          one(1), one(kv), 1, 1, hd, ps, 1.0, 0, 1, kv)
+        assert float((out.cpu()[0].float() - vv[far, 0].float()).abs().max()) < 1e-5, far
 
 
 def test_paged_attention_refuses_bad_shapes(k):
     qkv = torch.zeros(2, 3 * 16, device=DEV)
     out = torch.zeros(2, 16, device=DEV)
     kc = torch.zeros(2, 1, 4, 16, device=DEV)
+    vc = torch.zeros(2, 1, 16, 4, device=DEV)
     one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
     table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
     with pytest.raises(ValueError, match="block table"):
-        k.paged_attention(qkv, out, kc, kc, table, one(0), one(2), one(9), 1, 1, 16, 4, 1.0, 0, 2, 9)
+        k.paged_attention(qkv, out, kc, vc, table, one(0), one(2), one(9), 1, 1, 16, 4, 1.0, 0, 2, 9)
     with pytest.raises(ValueError, match="k_cache"):
-        k.paged_attention(qkv, out, kc[:, :, :2].contiguous(), kc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
+        k.paged_attention(qkv, out, kc[:, :, :2].contiguous(), vc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
     with pytest.raises(TypeError):
-        k.paged_attention(qkv.half(), out, kc, kc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
+        k.paged_attention(qkv.half(), out, kc, vc, table, one(0), one(2), one(8), 1, 1, 16, 4, 1.0, 0, 2, 8)
     big = torch.zeros(1, 3 * 512, device=DEV)
     with pytest.raises(ValueError, match="head size"):
         k.paged_attention(big, torch.zeros(1, 512, device=DEV), torch.zeros(2, 1, 4, 512, device=DEV),
-                          torch.zeros(2, 1, 4, 512, device=DEV), table, one(0), one(1), one(1), 1, 1, 512, 4, 1.0, 0, 1, 1)
+                          torch.zeros(2, 1, 512, 4, device=DEV), table, one(0), one(1), one(1), 1, 1, 512, 4, 1.0, 0, 1, 1)
 
 
 def test_argmax_lowest_index_wins(k):

@@ -109,7 +109,7 @@ def test_attention_part_whole_and_cut(dtype, nq, nkv, hd, hidden, window, bias, 
     ref = plain.self_attention_block(x.double(), w, "a.", cfg, torch.arange(s), window)
     n_pages = 16
     kc = torch.zeros(n_pages, nkv, ps, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(n_pages, nkv, hd, ps, dtype=dtype, device=DEV)
     table = torch.randperm(n_pages, generator=torch.Generator().manual_seed(8)).to(torch.int32)[None, :12].contiguous().to(DEV)
     outs, pos = [], 0
     for n in (20, 1, 2, 22):                      # a prompt portion, a decoded token, two more portions
@@ -152,7 +152,7 @@ def test_pre_norm_block(dtype):
     a = xd + plain.self_attention_block(plain.rms_norm(xd, w["n1.weight"], eps), w, "a.", cfg, torch.arange(s))
     y = a + plain.swiglu_mlp(plain.rms_norm(a, w["n2.weight"], eps), w, "m.")
     kc = torch.zeros(3, nkv, ps, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(3, nkv, hd, ps, dtype=dtype, device=DEV)
     table = torch.tensor([[2, 0, 1]], dtype=torch.int32, device=DEV)
     positions = torch.arange(s, dtype=torch.int32, device=DEV)
     slots = (table[0, (positions // ps).long()] * ps + positions % ps).to(torch.int32)
