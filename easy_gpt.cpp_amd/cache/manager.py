@@ -33,6 +33,7 @@ class RequestCache:
     num_tokens: int = 0                      # tokens whose keys and values are in the cache
     tables: list[list[int]] = field(default_factory=list)   # per group: page ids, -1 = given back
     live: bool = True
+    version: int = 0                         # changes whenever a table changes
 
 
 def _ceil_div(a: int, b: int) -> int:
@@ -86,7 +87,9 @@ class CacheManager:
                     f"{pool.free_count} of {pool.num_pages} are free"
                 )
         for n, pool, table in zip(need, self.pools, rc.tables):
-            table.extend(pool.take(n))
+            if n:
+                table.extend(pool.take(n))
+                rc.version += 1
 
     def commit(self, rc: RequestCache, n_new: int) -> None:
         rc.num_tokens += n_new
@@ -103,6 +106,7 @@ class CacheManager:
                 pool.give_back(gone)
                 for i in range(dead_pages):
                     table[i] = -1
+                rc.version += 1
 
     def release(self, rc: RequestCache) -> None:
         if not rc.live:
@@ -112,6 +116,7 @@ class CacheManager:
             table.clear()
         self.slots.give_back(rc.slot)
         rc.live = False
+        rc.version += 1
         del self.requests[rc.request_id]
 
     # ------------------------------------------------------------------ queries

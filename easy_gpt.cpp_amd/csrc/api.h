@@ -42,7 +42,8 @@ int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* 
                               const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
                               int n_tokens, int nq, int nkv, int hd, int page_size, float scale, int window,
                               int n_splits, int rows_per_wave, void* stream);
-int egpt_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
+// scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
+int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                 const float* uniform, int32_t* out, int n_rows, int vocab, void* stream);
 

@@ -206,27 +206,41 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 }
 
 // out[row, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits; one wavefront per row.
+// Lane s first takes split s's (maximum, sum) so that the weights of up to 64 splits are known after one
+// round of loads; the partial outputs are then read eight splits at a time.
 __global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __restrict__ part_o,
                                                               const float* __restrict__ part_ml,
                                                               bf16_t* __restrict__ out, int n_rows, int hd, int n_splits) {
     const int row = blockIdx.x, lane = threadIdx.x;
-    float m_max = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) m_max = fmaxf(m_max, part_ml[(static_cast<size_t>(s) * n_rows + row) * 2]);
-    float denom = 0.f;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < n_splits; ++s) {
-        const size_t pr = static_cast<size_t>(s) * n_rows + row;
-        const float m = part_ml[pr * 2];
-        if (m == -INFINITY) continue;              // a split without visible keys
-        const float wgt = __expf(m - m_max);
-        denom += wgt * part_ml[pr * 2 + 1];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int d = lane + r * kWave;
-            if (d < hd) acc[r] += wgt * part_o[pr * hd + d];
-        }
+    float m = -INFINITY, l = 0.f;
+    if (lane < n_splits) {
+        const size_t pr = static_cast<size_t>(lane) * n_rows + row;
+        m = part_ml[pr * 2];
+        l = part_ml[pr * 2 + 1];
     }
-    const float inv = 1.0f / denom;
+    const float m_max = wave_max(m);
+    const float wgt = m == -INFINITY ? 0.f : __expf(m - m_max);    // a split without visible keys weighs nothing
+    const float inv = 1.0f / wave_sum(wgt * l);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+        float v[8][4], w8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int s = s0 + i;
+            w8[i] = __shfl(wgt, s < n_splits ? s : 0, kWave);
+            if (s >= n_splits) w8[i] = 0.f;
+            const size_t pr = static_cast<size_t>(s < n_splits ? s : 0) * n_rows + row;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int d = lane + r * kWave;
+                v[i][r] = (d < hd && w8[i] != 0.f) ? part_o[pr * hd + d] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] += w8[i] * v[i][r];
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int d = lane + r * kWave;
@@ -271,7 +285,7 @@ extern "C" int egpt_paged_attention_mfma(const void* qkv, void* out, float* part
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 ||
         n_splits < 1 || (n_splits > 1 && (!part_o || !part_ml)))
         return EGPT_BAD_ARGUMENT;
-    if ((hd != 64 && hd != 128) || page_size % 16 != 0 || nkv > 65535 || n_splits > 65535 ||
+    if ((hd != 64 && hd != 128) || page_size % 16 != 0 || nkv > 65535 || n_splits > 64 ||
         (rows_per_wave != 16 && rows_per_wave != 32))
         return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;

@@ -16,8 +16,17 @@ struct ProductView {
     __device__ __forceinline__ bool present() const { return whole != nullptr || partial != nullptr; }
     __device__ __forceinline__ float at(size_t idx) const {
         if (n_splits == 0) return to_float(whole[idx]);
-        float v = partial[idx];
-        for (int s = 1; s < n_splits; ++s) v += partial[s * split_stride + idx];
+        // eight loads in flight at a time; the order of the additions is fixed
+        float v = 0.f;
+        int s = 0;
+        for (; s + 8 <= n_splits; s += 8) {
+            float t[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) t[i] = partial[(s + i) * split_stride + idx];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v += t[i];
+        }
+        for (; s < n_splits; ++s) v += partial[s * split_stride + idx];
         return v;
     }
 };
@@ -87,6 +96,8 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
 // (/root/reference/src/ops.cpp:404-420, /root/reference/src/cuda/ops/self_attn_detail.cuh:512-541);
 // write the result back in place and store keys and values at their slot of the paged cache
 // (keys [page][kv head][offset][hd], values [page][kv head][hd][offset]).
+constexpr int kHeadsPerBlock = 2;   // heads of one token that a workgroup of the QKV epilogue handles
+
 template <typename T>
 __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv_out, const T* __restrict__ bias,
                                       const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
@@ -94,13 +105,15 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv
                                       T* __restrict__ v_cache, int nq, int nkv, int hd, int page_size) {
     const int t = blockIdx.x;
     const int n_heads = nq + 2 * nkv;
+    const int item_begin = blockIdx.y * kHeadsPerBlock * hd;
+    const int item_end = min(n_heads * hd, item_begin + kHeadsPerBlock * hd);
     const size_t base = static_cast<size_t>(t) * n_heads * hd;
     T* row = qkv_out + base;
     const float pos = static_cast<float>(positions[t]);
     const int half = rotary_dim / 2;
     long slot = slots ? slots[t] : -1;
     const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
-    for (int item = threadIdx.x; item < n_heads * hd; item += blockDim.x) {
+    for (int item = item_begin + threadIdx.x; item < item_end; item += blockDim.x) {
         const int head = item / hd, d = item % hd;
         const bool rotated = head < nq + nkv && d < rotary_dim;
         if (rotated && d >= half) continue;  // done by its partner
@@ -167,7 +180,8 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, i
     if (delta && delta_rows <= 0) return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int threads = hidden >= 2048 ? 512 : 256;
+    // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for
+    const int threads = (delta_splits > 1 || hidden >= 4096) ? 1024 : (hidden >= 2048 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
     if (dtype == 0)
         add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, make_view<float>(delta, delta_splits, stride), rows,
@@ -216,13 +230,15 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_o
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
+    const dim3 grid(n_tokens, (nq + 2 * nkv + kHeadsPerBlock - 1) / kHeadsPerBlock);
+    const int block = kHeadsPerBlock * hd >= 256 ? 256 : (kHeadsPerBlock * hd >= 128 ? 128 : 64);
     if (dtype == 0)
-        qkv_rope_store_kernel<float><<<n_tokens, 256, 0, s>>>(
+        qkv_rope_store_kernel<float><<<grid, block, 0, s>>>(
             make_view<float>(qkv_in, n_splits, stride), static_cast<float*>(qkv_out), static_cast<const float*>(bias),
             positions, inv_freq, rotary_dim, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq,
             nkv, hd, page_size);
     else if (dtype == 1)
-        qkv_rope_store_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(
+        qkv_rope_store_kernel<bf16_t><<<grid, block, 0, s>>>(
             make_view<bf16_t>(qkv_in, n_splits, stride), static_cast<bf16_t*>(qkv_out),
             static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots, static_cast<bf16_t*>(k_cache),
             static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
@@ -242,4 +258,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 2; }
+extern "C" int egpt_abi_version(void) { return 3; }

@@ -59,6 +59,46 @@ __global__ __launch_bounds__(kSampleThreads) void argmax_kernel(const float* __r
     if (threadIdx.x == 0) out[r] = best;
 }
 
+// Two stages for wide vocabularies: workgroup (row, c) finds the maximum of its piece of the row, then one
+// workgroup per row picks among the pieces (lowest index among equal maxima in both stages).
+constexpr int kArgmaxPieces = 32;
+
+__global__ __launch_bounds__(256) void argmax_pieces_kernel(const float* __restrict__ logits,
+                                                            float* __restrict__ piece_val,
+                                                            int32_t* __restrict__ piece_idx, int vocab) {
+    __shared__ float s_val[16];
+    __shared__ int s_idx[16];
+    const int r = blockIdx.x, c = blockIdx.y;
+    const int piece = (vocab + kArgmaxPieces - 1) / kArgmaxPieces;
+    const int begin = min(vocab, c * piece), n = min(vocab, begin + piece) - begin;
+    int best = 0;
+    float val = -INFINITY;
+    if (n > 0) {
+        const float* row = logits + static_cast<size_t>(r) * vocab + begin;
+        best = block_argmax(row, n, s_val, s_idx);
+        val = row[best];
+    }
+    if (threadIdx.x == 0) {
+        piece_val[r * kArgmaxPieces + c] = val;
+        piece_idx[r * kArgmaxPieces + c] = begin + best;
+    }
+}
+
+__global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict__ piece_val,
+                                                         const int32_t* __restrict__ piece_idx,
+                                                         int32_t* __restrict__ out) {
+    const int r = blockIdx.x, lane = threadIdx.x;
+    float v = lane < kArgmaxPieces ? piece_val[r * kArgmaxPieces + lane] : -INFINITY;
+    int i = lane < kArgmaxPieces ? piece_idx[r * kArgmaxPieces + lane] : 0x7fffffff;
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, kWave);
+        const int oi = __shfl_xor(i, o, kWave);
+        argmax_combine(v, i, ov, oi);
+    }
+    if (lane == 0) out[r] = i;
+}
+
 // weight of token j: exp((x_j - max) / T), in (0, 1]
 __device__ __forceinline__ float weight_of(float x, float mx, float inv_t) { return expf((x - mx) * inv_t); }
 
@@ -166,10 +206,20 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 using namespace egpt;
 
-extern "C" int egpt_argmax(const float* logits, int32_t* out, int n_rows, int vocab, void* stream) {
+// scratch: room for n_rows * 32 floats and n_rows * 32 int32 (used for wide vocabularies), or null.
+extern "C" int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream) {
     if (!logits || !out || n_rows < 0 || vocab <= 0) return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
-    argmax_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, out, vocab);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (scratch && vocab >= 8192) {
+        float* pv = static_cast<float*>(scratch);
+        int32_t* pi = reinterpret_cast<int32_t*>(pv + static_cast<size_t>(n_rows) * kArgmaxPieces);
+        argmax_pieces_kernel<<<dim3(n_rows, kArgmaxPieces), 256, 0, s>>>(logits, pv, pi, vocab);
+        EGPT_CHECK_LAUNCH();
+        argmax_pick_kernel<<<n_rows, kWave, 0, s>>>(pv, pi, out);
+    } else {
+        argmax_kernel<<<n_rows, kSampleThreads, 0, s>>>(logits, out, vocab);
+    }
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

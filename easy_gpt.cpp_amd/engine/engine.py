@@ -65,6 +65,7 @@ class Engine:
         max_tokens: int | None = None,
         num_pages: int | None = None,
         max_requests: int = 64,
+        use_graphs: bool = True,
     ):
         """max_tokens: the most tokens live requests hold at any time (each request's count
         rounded up to a page); the pools are made for that many.  num_pages sets the page
@@ -87,6 +88,10 @@ class Engine:
         self.states = StateStorage(model.state_needs, max_requests, self.device)
         self.vocab_size = model.spec.vocab_size
         self.max_position = model.spec.max_position
+        # steps that hold one token per request are replayed from captured device graphs
+        self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe
+        self._decode_plans: dict = {}
+        self._graph_pool = None
 
     @classmethod
     def from_dir(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
@@ -108,10 +113,13 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
         of each entry's `want`, or None if nothing is wanted.  Raises OutOfPages (with the cache
-        unchanged) if the tokens do not fit."""
+        unchanged) if the tokens do not fit.  The returned tensor may be overwritten by the next
+        call of `step`: use it (or copy it) before stepping again."""
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
             return None
+        if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
+            return self._step_decode(entries)
         rcs = self._check(entries)
         self._reserve_all(rcs, entries)
         ctx = self._build_context(rcs, entries)
@@ -213,3 +221,122 @@ class Engine:
             groups=groups, page_size=ps, kv_storage=self.kv, state_storage=self.states,
             cache_location=self.model.cache_location, group_windows=[n.window for n in self.cache.groups],
         )
+
+    # ------------------------------------------------------------------ one token per request, from a graph
+    def _step_decode(self, entries) -> torch.Tensor:
+        """The step for batches of single tokens that all want their logits: the same model code, captured
+        once per (batch size, block-table width) into a device graph and replayed with new metadata.  The
+        launch of some two hundred kernels costs more host time than they run on the device; the graph
+        removes that."""
+        rcs = self._check(entries)
+        self._reserve_all(rcs, entries)
+        ps = self.page_size
+        b = len(rcs)
+        n_groups = len(self.cache.groups)
+        widths = []
+        for g in range(n_groups):
+            need = max(len(rc.tables[g]) for rc in rcs)
+            w = 4
+            while w < need:
+                w *= 2
+            widths.append(w)
+        key = (b, tuple(widths))
+        plan = self._decode_plans.get(key)
+        if plan is None:
+            plan = self._decode_plans[key] = _DecodePlan(self, b, widths)
+        plan.fill(rcs, [e.tokens[0] for e in entries])
+        if plan.graph is None:
+            logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
+            plan.runs += 1
+            if plan.runs >= 2:                              # captured from the second visit on
+                plan.capture(self)
+        else:
+            plan.graph.replay()
+            logits = plan.logits
+        for rc in rcs:
+            self.cache.commit(rc, 1)
+        return logits
+
+
+class _DecodePlan:
+    """Static device buffers, a host mirror and the captured graph of one decode batch shape."""
+
+    def __init__(self, engine: Engine, batch: int, widths: list[int]):
+        self.batch, self.widths = batch, list(widths)
+        dev = engine.device
+        n_groups = len(widths)
+        b = batch
+        n_small = (7 + n_groups) * b
+        self.host_small = torch.empty(n_small, dtype=torch.int32, pin_memory=True)
+        self.dev_small = torch.empty(n_small, dtype=torch.int32, device=dev)
+        n_tab = sum(b * w for w in widths)
+        self.host_tab = torch.full((max(n_tab, 1),), -1, dtype=torch.int32).pin_memory()
+        self.dev_tab = torch.full((max(n_tab, 1),), -1, dtype=torch.int32, device=dev)
+        self.np_small = self.host_small.numpy()
+        self.np_tab = self.host_tab.numpy()
+        hs = self.np_small
+        hs[2 * b : 3 * b] = np.arange(b)          # q_start
+        hs[3 * b : 4 * b] = 1                     # q_len
+        hs[6 * b : 7 * b] = np.arange(b)          # wanted rows: all
+        v = lambda i: self.dev_small[i * b : (i + 1) * b]
+        groups, off = [], 0
+        self.tab_offsets = []
+        for g, w in enumerate(widths):
+            groups.append(GroupTables(self.dev_tab[off : off + b * w].view(b, w), v(7 + g)))
+            self.tab_offsets.append(off)
+            off += b * w
+        ps = engine.page_size
+        self.ctx = StepContext(
+            num_tokens=b, num_seqs=b, token_ids=v(0), positions=v(1), q_start=v(2), q_len=v(3), kv_len=v(4),
+            want_rows=v(6), max_q_len=1, max_kv_len=min(w * ps for w in widths) if widths else 1,
+            q_start_host=list(range(b)), q_len_host=[1] * b, kv_len_host=[0] * b,
+            state_slots=v(5), state_slots_host=[0] * b, groups=groups, page_size=ps, kv_storage=engine.kv,
+            state_storage=engine.states, cache_location=engine.model.cache_location,
+            group_windows=[n.window for n in engine.cache.groups],
+        )
+        self.row_owner: list = [None] * b
+        self.row_version = [-1] * b
+        self.copied = None           # event after the last host-to-device copy
+        self.graph = None
+        self.logits = None
+        self.runs = 0
+        self.ps = ps
+
+    def fill(self, rcs, tokens) -> None:
+        if self.copied is not None:
+            self.copied.synchronize()                       # the pinned mirror is free again
+        b, ps, hs = self.batch, self.ps, self.np_small
+        pos = [rc.num_tokens for rc in rcs]
+        hs[0:b] = tokens
+        hs[b : 2 * b] = pos
+        hs[4 * b : 5 * b] = [p + 1 for p in pos]
+        hs[5 * b : 6 * b] = [rc.slot for rc in rcs]
+        tables_changed = False
+        for g, w in enumerate(self.widths):
+            hs[(7 + g) * b : (8 + g) * b] = [rc.tables[g][p // ps] * ps + p % ps for rc, p in zip(rcs, pos)]
+        for i, rc in enumerate(rcs):
+            if self.row_owner[i] is not rc or self.row_version[i] != rc.version:
+                for g, w in enumerate(self.widths):
+                    o = self.tab_offsets[g] + i * w
+                    t = rc.tables[g]
+                    self.np_tab[o : o + len(t)] = t
+                    self.np_tab[o + len(t) : o + w] = -1
+                self.row_owner[i], self.row_version[i] = rc, rc.version
+                tables_changed = True
+        self.ctx.kv_len_host = [p + 1 for p in pos]
+        self.ctx.state_slots_host = [rc.slot for rc in rcs]
+        self.dev_small.copy_(self.host_small, non_blocking=True)
+        if tables_changed:
+            self.dev_tab.copy_(self.host_tab, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+
+    def capture(self, engine: Engine) -> None:
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        if engine._graph_pool is None:
+            engine._graph_pool = torch.cuda.graph_pool_handle()
+        with torch.cuda.graph(graph, pool=engine._graph_pool):
+            self.logits = engine.model.forward(self.ctx)
+        self.graph = graph

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 2:
+    if lib.egpt_abi_version() != 3:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -51,7 +51,7 @@ class HipKernels:
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp],
-            "egpt_argmax": [vp, vp, i, i, vp],
+            "egpt_argmax": [vp, vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
         }
         for name, argtypes in sigs.items():
@@ -181,7 +181,7 @@ class HipKernels:
         bounded so that the partial sums stay smaller than the weights they came from."""
         steps = -(-k // 128)
         n_blocks = -(-n // 64)
-        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)))
+        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)), 16)
         per = -(-steps // s)
         return -(-steps // per)
 
@@ -273,7 +273,8 @@ class HipKernels:
         r, v = logits.shape
         self._need(logits, "logits", _F32)
         self._need(out, "out", _I32, (r,))
-        self._run("egpt_argmax", logits.data_ptr(), out.data_ptr(), r, v, self._stream())
+        scratch = torch.empty(r * 64, dtype=_F32, device=logits.device) if v >= 8192 else None
+        self._run("egpt_argmax", logits.data_ptr(), out.data_ptr(), self._ptr(scratch), r, v, self._stream())
 
     def sample(self, logits, temperature, top_k, top_p, uniform, out):
         r, v = logits.shape

@@ -22,6 +22,8 @@ from .spec import ParamSpec, PartSpec
 
 
 class GQAttention(Mixer):
+    graph_safe = True
+
     def __init__(
         self,
         prefix: str,
@@ -47,6 +49,7 @@ class GQAttention(Mixer):
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = make_part("position_encoding", position, head_dim=self.head_dim)
+        self.graph_safe = bool(getattr(self.position, "graph_safe", False))
         self.q_size = self.n_heads * self.head_dim
         self.kv_size = self.n_kv_heads * self.head_dim
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None

@@ -77,7 +77,14 @@ class StateView:
 
 # --------------------------------------------------------------------------- part interfaces
 class Part:
-    """Common interface: parameters declared, loaded, then used."""
+    """Common interface: parameters declared, loaded, then used.
+
+    graph_safe: True if `forward` only launches device work whose arguments do not depend on host
+    values other than the step's shapes (no reads of device data on the host, no host loops over
+    requests).  Steps of models whose parts are all graph-safe can be captured into a device graph
+    and replayed."""
+
+    graph_safe = False
 
     def param_specs(self) -> list[ParamSpec]:
         return []

@@ -16,6 +16,8 @@ from .spec import ParamSpec
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int):
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
@@ -35,6 +37,8 @@ class TokenEmbedding(Part):
 
 
 class OutputHead(Part):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool):
         self.prefix = prefix
         self.hidden_size = int(hidden_size)

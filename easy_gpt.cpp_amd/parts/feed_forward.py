@@ -16,6 +16,8 @@ from .spec import ParamSpec
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
             raise ValueError(f"activation '{activation}' is not supported by the swiglu feed-forward")

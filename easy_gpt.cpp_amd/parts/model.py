@@ -43,6 +43,7 @@ class Model:
         self.dtype: torch.dtype | None = None
         self.device: torch.device | None = None
         self._plan_caches()
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.parts())
 
     # ------------------------------------------------------------------ cache and state plan
     def _plan_caches(self) -> None:

@@ -15,6 +15,8 @@ from .spec import ParamSpec
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden_size: int, eps: float):
         self.prefix = prefix
         self.hidden_size = int(hidden_size)

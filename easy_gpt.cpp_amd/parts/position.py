@@ -16,6 +16,8 @@ from .base import PositionEncoding, register_part
 class RotaryHalfSplit(PositionEncoding):
     """Rotation of the first `rotary_dim` features of each head (all of them by default)."""
 
+    graph_safe = True
+
     def __init__(self, prefix: str, head_dim: int, theta: float, rotary_dim: int | None = None, **_):
         self.head_dim = int(head_dim)
         self.theta = float(theta)
@@ -42,6 +44,8 @@ class RotaryHalfSplit(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """No position information enters the mixer."""
+
+    graph_safe = True
 
     def __init__(self, prefix: str = "", **_):
         pass
