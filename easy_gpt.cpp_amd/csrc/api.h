@@ -21,7 +21,9 @@ int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_ro
                      const void* weight, float eps, void* out, int n_rows, int hidden, int dtype, void* stream);
 int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype, void* stream);
 // qkv_out [n_tokens, (nq + 2 nkv) hd] of the activation type; may be qkv_in itself when n_splits == 0.
-int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_out, const void* bias, const int32_t* positions,
+// row_ss != null: the product still lacks each row's factor 1 / sqrt(sum_s row_ss[s][row] / hidden + eps).
+int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, int ss_splits, int hidden, float eps,
+                        void* qkv_out, const void* bias, const int32_t* positions,
                         const float* inv_freq, int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache,
                         int n_tokens, int nq, int nkv, int hd, int page_size, int dtype, void* stream);
 // bfloat16 product for m <= 64 rows on the matrix cores, optionally split over k (see gemm_skinny.hip).
@@ -41,7 +43,22 @@ int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* 
                               const void* v_cache, const int32_t* block_table, int table_width,
                               const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
                               int n_tokens, int nq, int nkv, int hd, int page_size, float scale, int window,
-                              int n_splits, int rows_per_wave, void* stream);
+                              int n_splits, int rows_per_wave, int combine, void* stream);
+// One decoded token per request: workgroups of n_waves wavefronts per (request, kv head, key split).
+int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                                const void* v_cache, const int32_t* block_table, int table_width,
+                                const int32_t* q_start, const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd,
+                                int page_size, float scale, int window, int n_splits, int n_waves, int combine,
+                                void* stream);
+int egpt_attention_combine(const float* part_o, const float* part_ml, void* out, int n_rows, int hd, int n_splits,
+                           void* stream);
+// Products for m <= 16 rows whose x operand is computed while it is staged (see gemm_skinny.hip).
+int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits, const void* norm_w,
+                          const void* w, float* out, float* ss_out, int m, int n, int k, int n_splits, void* stream);
+int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits, int hidden,
+                            float eps, const void* w, float* out, int m, int n, int k, int n_splits, void* stream);
+int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd, const void* w,
+                          float* out, int m, int n, int n_splits, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,

@@ -205,6 +205,171 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     }
 }
 
+// Decoded tokens only (one query token per request, its heads of one kv group in one 16-row tile): a
+// workgroup of NW wavefronts shares one (request, kv head, key split); each wavefront walks its share of
+// the keys, PF blocks of 32 keys per round with all of the round's loads in flight together (the kernel is
+// a chain of round trips to memory, not of arithmetic), and the wavefronts' results are combined through
+// LDS.  With n_splits > 1 the combined, still unnormalised result goes to part_o / part_ml.
+template <int HD, int PF>
+__global__ __launch_bounds__(512) void attention_decode_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ kv_len, int n_tokens, int nq, int nkv, int page_size, float scale, int window,
+    int n_splits) {
+    constexpr int KD = HD / 32, DT = HD / 16;
+    extern __shared__ float wave_state[];          // [n_waves][16][HD + 2]: O, then maximum, then sum
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
+    const int lj = lane % 16, lg = lane / 16;
+    const int b = blockIdx.x, kh = blockIdx.y, split = blockIdx.z;
+    const int group_size = nq / nkv;
+    const int kv = kv_len[b], tok = q_start[b];
+    const int p = kv - 1;
+    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    const bool valid = lj < group_size;
+    const int head = kh * group_size + (valid ? lj : 0);
+    const int width = (nq + 2 * nkv) * HD;
+    const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+
+    bf16x8 q[KD];
+    {
+        const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+            q[kd] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    const int kb_begin = lo / 32, kb_end = p / 32 + 1;
+    const int per_split = (kb_end - kb_begin + n_splits - 1) / n_splits;
+    const int s_begin = kb_begin + split * per_split, s_end = min(kb_end, s_begin + per_split);
+    const int per_wave = (max(s_end - s_begin, 0) + n_waves - 1) / n_waves;
+    const int w_begin = s_begin + wave * per_wave, w_end = min(s_end, w_begin + per_wave);
+
+    f32x4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    for (int kb0 = w_begin; kb0 < w_end; kb0 += PF) {
+        uint4 kk[PF][2][KD];
+        uint2 vv[PF][2][DT];
+        // first all page numbers of the round (one wait for all of them), then all key and value loads
+        int pages[PF][2];
+        bool live[PF][2];
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                const int key0 = (kb0 + i) * 32 + kt * 16;
+                live[i][kt] = kb0 + i < w_end && key0 <= p && key0 + 15 >= lo;
+                pages[i][kt] = table[live[i][kt] ? key0 / page_size : 0];
+            }
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                const int key0 = (kb0 + i) * 32 + kt * 16;
+                const bool ok = live[i][kt] && pages[i][kt] >= 0;
+                const long page = ok ? pages[i][kt] : 0;
+                const int off = ok ? key0 % page_size : 0;
+                const bf16_t* kp = k_cache + ((page * nkv + kh) * page_size + off + lj) * HD + lg * 8;
+                const bf16_t* vp = v_cache + ((page * nkv + kh) * HD + lj) * static_cast<long>(page_size) + off + lg * 4;
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd)
+                    kk[i][kt][kd] = ok ? *reinterpret_cast<const uint4*>(kp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int d = 0; d < DT; ++d)
+                    vv[i][kt][d] = ok ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
+                                      : uint2{0u, 0u};
+            }
+#pragma unroll
+        for (int i = 0; i < PF; ++i) {
+            if (kb0 + i >= w_end) break;
+            float s[2][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kk[i][kt][kd]), q[kd], acc,
+                                                                  0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = (kb0 + i) * 32 + kt * 16 + lg * 4 + v;
+                    const bool vis = valid && key <= p && key >= lo;
+                    s[kt][v] = vis ? acc[v] * scale : -INFINITY;
+                    mx = fmaxf(mx, s[kt][v]);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+            const float m_new = fmaxf(m_run, mx);
+            const bool none = m_new == -INFINITY;
+            const float alpha = none ? 1.f : __expf(m_run - m_new);
+            float sum = 0.f;
+            bf16x8 pb;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float pv = none ? 0.f : __expf(s[kt][v] - m_new);
+                    sum += pv;
+                    pb[kt * 4 + v] = static_cast<__bf16>(pv);
+                }
+            l_run = l_run * alpha + sum;
+            m_run = m_new;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                const uint4 av = uint4{vv[i][0][d].x, vv[i][0][d].y, vv[i][1][d].x, vv[i][1][d].y};
+                f32x4 acc = o[d];
+                acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+                o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb, acc, 0, 0, 0);
+            }
+        }
+    }
+    float l = l_run;
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+
+    // every wavefront leaves its state in LDS; then all threads combine
+    constexpr int kRow = HD + 2;
+    float* mine = wave_state + (wave * 16 + lj) * kRow;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) mine[d * 16 + lg * 4 + v] = o[d][v];
+    if (lg == 0) {
+        mine[HD] = m_run;
+        mine[HD + 1] = l;
+    }
+    __syncthreads();
+    const size_t row0 = static_cast<size_t>(tok) * nq + kh * group_size;
+    for (int idx = threadIdx.x; idx < group_size * HD; idx += blockDim.x) {
+        const int r = idx / HD, d = idx % HD;
+        float mx = -INFINITY;
+        for (int w = 0; w < n_waves; ++w) mx = fmaxf(mx, wave_state[(w * 16 + r) * kRow + HD]);
+        float num = 0.f, den = 0.f;
+        for (int w = 0; w < n_waves; ++w) {
+            const float* st = wave_state + (w * 16 + r) * kRow;
+            const float wgt = st[HD] == -INFINITY ? 0.f : __expf(st[HD] - mx);
+            num += wgt * st[d];
+            den += wgt * st[HD + 1];
+        }
+        if (n_splits == 1) {
+            out[(row0 + r) * HD + d] = from_float<bf16_t>(num / den);
+        } else {
+            const size_t prow = static_cast<size_t>(split) * n_tokens * nq + row0 + r;
+            part_o[prow * HD + d] = num;
+            if (d == 0) {
+                part_ml[prow * 2] = mx;
+                part_ml[prow * 2 + 1] = den;
+            }
+        }
+    }
+}
+
 // out[row, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits; one wavefront per row.
 // Lane s first takes split s's (maximum, sum) so that the weights of up to 64 splits are known after one
 // round of loads; the partial outputs are then read eight splits at a time.
@@ -252,7 +417,7 @@ template <int HD, int QT>
 static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                        const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                        const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
-                       int page_size, float scale, int window, int n_splits, hipStream_t s) {
+                       int page_size, float scale, int window, int n_splits, int combine, hipStream_t s) {
     const int group = nq / nkv;
     const long groups = (static_cast<long>(n_tokens) * group) / (16 * QT) + n_seqs;   // upper bound
     dim3 grid(static_cast<unsigned>(groups), nkv, n_splits);
@@ -261,7 +426,28 @@ static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml
         static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
         q_len, kv_len, n_seqs, n_tokens, nq, nkv, page_size, scale, window, n_splits);
     EGPT_CHECK_LAUNCH();
-    if (n_splits > 1) {
+    if (n_splits > 1 && combine) {
+        attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
+                                                             HD, n_splits);
+        EGPT_CHECK_LAUNCH();
+    }
+    return EGPT_OK;
+}
+
+template <int HD>
+static int launch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                         const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
+                         const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size, float scale,
+                         int window, int n_splits, int n_waves, int combine, hipStream_t s) {
+    constexpr int PF = HD == 64 ? 4 : 2;
+    dim3 grid(n_seqs, nkv, n_splits);
+    const size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
+    attention_decode_kernel<HD, PF><<<grid, n_waves * kWave, lds, s>>>(
+        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
+        static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
+        kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits);
+    EGPT_CHECK_LAUNCH();
+    if (n_splits > 1 && combine) {
         attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
                                                              HD, n_splits);
         EGPT_CHECK_LAUNCH();
@@ -273,13 +459,37 @@ static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml
 
 using namespace egpt;
 
+// One decoded token per request (n_tokens == n_seqs, q_len all 1), nq / nkv <= 16: workgroups of n_waves
+// wavefronts (1..8) per (request, kv head, key split).  Same operands and meaning as egpt_paged_attention_mfma.
+extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float* part_ml,
+                                           const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                           int table_width, const int32_t* q_start, const int32_t* kv_len, int n_seqs,
+                                           int nq, int nkv, int hd, int page_size, float scale, int window,
+                                           int n_splits, int n_waves, int combine, void* stream) {
+    if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !kv_len) return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 || n_splits < 1 ||
+        (n_splits > 1 && (!part_o || !part_ml)))
+        return EGPT_BAD_ARGUMENT;
+    if ((hd != 64 && hd != 128) || page_size % 16 != 0 || nq / nkv > 16 || nkv > 65535 || n_splits > 64 ||
+        n_waves < 1 || n_waves > 8)
+        return EGPT_UNSUPPORTED_SIZE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (hd == 64)
+        return launch_decode<64>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start,
+                                 kv_len, n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine,
+                                 s);
+    return launch_decode<128>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
+                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, s);
+}
+
 // bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.
-// part_o [n_splits][n_tokens][nq][hd] and part_ml [n_splits][n_tokens][nq][2] float32 are needed when n_splits > 1.
+// part_o [n_splits][n_tokens][nq][hd] and part_ml [n_splits][n_tokens][nq][2] float32 are needed when n_splits > 1;
+// with combine == 0 they are left for the caller to combine (the output projection does it while it stages x).
 extern "C" int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                                          const void* v_cache, const int32_t* block_table, int table_width,
                                          const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len,
                                          int n_seqs, int n_tokens, int nq, int nkv, int hd, int page_size, float scale,
-                                         int window, int n_splits, int rows_per_wave, void* stream) {
+                                         int window, int n_splits, int rows_per_wave, int combine, void* stream) {
     if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
         return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 ||
@@ -292,8 +502,21 @@ extern "C" int egpt_paged_attention_mfma(const void* qkv, void* out, float* part
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define EGPT_ATTN_ARGS                                                                                              \
     qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len, n_seqs, n_tokens, \
-        nq, nkv, page_size, scale, window, n_splits, s
+        nq, nkv, page_size, scale, window, n_splits, combine, s
     if (hd == 64) return rows_per_wave == 16 ? launch_mfma<64, 1>(EGPT_ATTN_ARGS) : launch_mfma<64, 2>(EGPT_ATTN_ARGS);
     return rows_per_wave == 16 ? launch_mfma<128, 1>(EGPT_ATTN_ARGS) : launch_mfma<128, 2>(EGPT_ATTN_ARGS);
 #undef EGPT_ATTN_ARGS
+}
+
+// Combines the parts that egpt_paged_attention_mfma left with combine == 0: out [n_rows][hd] bfloat16.
+extern "C" int egpt_attention_combine(const float* part_o, const float* part_ml, void* out, int n_rows, int hd,
+                                      int n_splits, void* stream) {
+    if (!part_o || !part_ml || !out || n_rows < 0 || hd <= 0 || n_splits < 1) return EGPT_BAD_ARGUMENT;
+    if (n_splits > 64 || hd > 256) return EGPT_UNSUPPORTED_SIZE;
+    if (n_rows == 0) return EGPT_OK;
+    attention_reduce_kernel<<<n_rows, 64, 0, static_cast<hipStream_t>(stream)>>>(part_o, part_ml,
+                                                                               static_cast<bf16_t*>(out), n_rows, hd,
+                                                                               n_splits);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
 }

@@ -16,17 +16,16 @@ struct ProductView {
     __device__ __forceinline__ bool present() const { return whole != nullptr || partial != nullptr; }
     __device__ __forceinline__ float at(size_t idx) const {
         if (n_splits == 0) return to_float(whole[idx]);
-        // eight loads in flight at a time; the order of the additions is fixed
+        // up to sixteen loads in flight at a time (a chain of dependent kernels pays for round trips, not
+        // bytes); the order of the additions is fixed
         float v = 0.f;
-        int s = 0;
-        for (; s + 8 <= n_splits; s += 8) {
-            float t[8];
+        for (int s0 = 0; s0 < n_splits; s0 += 16) {
+            float t[16];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) t[i] = partial[(s + i) * split_stride + idx];
+            for (int i = 0; i < 16; ++i) t[i] = s0 + i < n_splits ? partial[(s0 + i) * split_stride + idx] : 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v += t[i];
+            for (int i = 0; i < 16; ++i) v += t[i];
         }
-        for (; s < n_splits; ++s) v += partial[s * split_stride + idx];
         return v;
     }
 };
@@ -99,7 +98,8 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
 constexpr int kHeadsPerBlock = 2;   // heads of one token that a workgroup of the QKV epilogue handles
 
 template <typename T>
-__global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv_out, const T* __restrict__ bias,
+__global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __restrict__ row_ss, int ss_splits,
+                                      float inv_hidden, float eps, T* __restrict__ qkv_out, const T* __restrict__ bias,
                                       const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
                                       int rotary_dim, const int32_t* __restrict__ slots, T* __restrict__ k_cache,
                                       T* __restrict__ v_cache, int nq, int nkv, int hd, int page_size) {
@@ -111,16 +111,29 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, T* __restrict__ qkv
     T* row = qkv_out + base;
     const float pos = static_cast<float>(positions[t]);
     const int half = rotary_dim / 2;
+    // the product may still lack its row's 1/rms factor (sum of squares of the row in row_ss, by split)
+    float row_scale = 1.f;
+    if (row_ss) {
+        float ss = 0.f;
+        for (int s0 = 0; s0 < ss_splits; s0 += 16) {
+            float part[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) part[i] = s0 + i < ss_splits ? row_ss[(s0 + i) * gridDim.x + t] : 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ss += part[i];
+        }
+        row_scale = 1.0f / sqrtf(ss * inv_hidden + eps);
+    }
     long slot = slots ? slots[t] : -1;
     const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
     for (int item = item_begin + threadIdx.x; item < item_end; item += blockDim.x) {
         const int head = item / hd, d = item % hd;
         const bool rotated = head < nq + nkv && d < rotary_dim;
         if (rotated && d >= half) continue;  // done by its partner
-        float a = qkv_in.at(base + item) + (bias ? to_float(bias[item]) : 0.f);
+        float a = qkv_in.at(base + item) * row_scale + (bias ? to_float(bias[item]) : 0.f);
         float b = 0.f;
         if (rotated) {
-            b = qkv_in.at(base + item + half) + (bias ? to_float(bias[item + half]) : 0.f);
+            b = qkv_in.at(base + item + half) * row_scale + (bias ? to_float(bias[item + half]) : 0.f);
             float s, c;
             sincosf(pos * inv_freq[d], &s, &c);
             const float ra = a * c - b * s, rb = a * s + b * c;
@@ -217,7 +230,8 @@ extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_t
     return EGPT_OK;
 }
 
-extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_out, const void* bias,
+extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, int ss_splits, int hidden,
+                                   float eps, void* qkv_out, const void* bias,
                                    const int32_t* positions, const float* inv_freq, int rotary_dim,
                                    const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv,
                                    int hd, int page_size, int dtype, void* stream) {
@@ -227,20 +241,23 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, void* qkv_o
     if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim % 2) != 0 || (rotary_dim > 0 && !inv_freq))
         return EGPT_BAD_ARGUMENT;
     if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
+    if (row_ss && (ss_splits < 1 || hidden < 1)) return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const float inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
     const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
     const dim3 grid(n_tokens, (nq + 2 * nkv + kHeadsPerBlock - 1) / kHeadsPerBlock);
     const int block = kHeadsPerBlock * hd >= 256 ? 256 : (kHeadsPerBlock * hd >= 128 ? 128 : 64);
     if (dtype == 0)
         qkv_rope_store_kernel<float><<<grid, block, 0, s>>>(
-            make_view<float>(qkv_in, n_splits, stride), static_cast<float*>(qkv_out), static_cast<const float*>(bias),
+            make_view<float>(qkv_in, n_splits, stride), row_ss, ss_splits, inv_hidden, eps,
+            static_cast<float*>(qkv_out), static_cast<const float*>(bias),
             positions, inv_freq, rotary_dim, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq,
             nkv, hd, page_size);
     else if (dtype == 1)
         qkv_rope_store_kernel<bf16_t><<<grid, block, 0, s>>>(
-            make_view<bf16_t>(qkv_in, n_splits, stride), static_cast<bf16_t*>(qkv_out),
-            static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots, static_cast<bf16_t*>(k_cache),
+            make_view<bf16_t>(qkv_in, n_splits, stride), row_ss, ss_splits, inv_hidden, eps,
+            static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots, static_cast<bf16_t*>(k_cache),
             static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
     else
         return EGPT_BAD_ARGUMENT;
@@ -258,4 +275,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 3; }
+extern "C" int egpt_abi_version(void) { return 4; }

@@ -9,9 +9,18 @@
 // workgroup (four wavefronts = 64 rows of w share it) in exactly that order.
 //
 // To fill 256 CUs when n is small the k range is split over `n_splits` workgroups, each writing its
-// partial sums to out[split][m][n] in float32.  The kernels that consume the result (bias + rotary +
-// cache store, SwiGLU, residual add + RMSNorm) add the partial sums up, in a fixed order, so the result
-// does not depend on scheduling.
+// partial sums to out[split][m][n] in float32.  The kernels that consume the result add the partial sums
+// up, in a fixed order, so the result does not depend on scheduling.
+//
+// A decode step is a chain of small dependent kernels, and each link costs a few microseconds whatever it
+// computes.  So for m <= 16 the staging of x can also compute x from what the previous kernels left
+// ("prologues"), which removes the separate norm, SwiGLU and attention-combine kernels from the chain:
+//   NORM    x = (h + sum_s delta_s) * norm_weight, not yet divided by the row's RMS: that factor is the same
+//           for the whole row, so it is applied to the product afterwards by the consumer.  Workgroups of
+//           the first column also write h + delta (the new residual stream, into a second buffer) and the
+//           row's sum of squares of their k range.
+//   SWIGLU  x = silu(g) * u with [g | u] = inv_rms * sum_s gate_up_s (partial sums of a NORM product).
+//   ATTN    x = sum_s wgt_s * o_s: the combination of the partial attention results over key splits.
 #include "api.h"
 #include "common.h"
 
@@ -24,47 +33,249 @@ constexpr int kStep = 128;          // k elements per step
 constexpr int kRowsPerWave = 16;
 constexpr int kWavesPerBlock = 4;
 constexpr int kLdsRow = kStep + 8;  // bf16 elements per staged row of x (16 bytes of padding)
+constexpr int kMaxLocalHeads = 8;   // ATTN prologue: heads that one workgroup's k range may touch
+constexpr int kMaxAttnSplits = 64;
+
+enum Prologue { kPlain = 0, kNorm = 1, kSwiglu = 2, kAttn = 3 };
+
+struct SkinnyArgs {
+    const bf16_t* w;
+    const bf16_t* bias;
+    float* out_f32;
+    bf16_t* out_bf16;
+    int m, n, k, steps_per_split;
+    // kPlain
+    const bf16_t* x;
+    // kNorm
+    const float* h_in;
+    float* h_out;
+    const float* delta;        // [delta_splits][m][k] or null
+    int delta_splits;
+    const bf16_t* norm_w;      // [k]
+    float* ss_out;             // [n_splits][m]
+    // kSwiglu: x[m][k] from gate_up [gu_splits][m][2k]
+    const float* gu;
+    int gu_splits;
+    const float* ss_in;        // [ss_splits][m] or null
+    int ss_splits;
+    float inv_hidden, eps;
+    // kAttn: x[m][head*hd + d] from part_o [a_splits][m*nq][hd], part_ml [a_splits][m*nq][2]
+    const float* part_o;
+    const float* part_ml;
+    int a_splits, nq, hd;
+};
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p, bool ok) {
     return ok ? *reinterpret_cast<const uint4*>(p) : uint4{0u, 0u, 0u, 0u};
 }
 
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                          const bf16_t* __restrict__ bias, float* __restrict__ out_f32,
-                                                          bf16_t* __restrict__ out_bf16, int m, int n, int k,
-                                                          int steps_per_split) {
+__device__ __forceinline__ uint4 pack8(const float* v) {
+    uint4 r;
+    r.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+    r.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+    r.z = f32_to_bf16_bits(v[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5])) << 16);
+    r.w = f32_to_bf16_bits(v[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7])) << 16);
+    return r;
+}
+
+__device__ __forceinline__ void load8f(const float* p, float* v) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+    v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3];
+    v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
+}
+
+// v += sum over splits of p[s * stride .. + 8]; up to kInFlight splits' loads are in flight together (what a
+// dependent kernel chain pays for is round trips to L2, not bytes; more would cost registers and with them
+// the co-residency of all workgroups); additions in split order
+constexpr int kInFlight = 8;
+
+__device__ __forceinline__ void add_splits8(const float* p, int n_splits, size_t stride, float* v) {
+    for (int s0 = 0; s0 < n_splits; s0 += kInFlight) {
+        float t[kInFlight][8];
+#pragma unroll
+        for (int i = 0; i < kInFlight; ++i) {
+            if (s0 + i < n_splits) {
+                load8f(p + (s0 + i) * stride, t[i]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) t[i][j] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kInFlight; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] += t[i][j];
+    }
+}
+
+// sum over splits of p[s * stride], up to 16 loads in flight
+__device__ __forceinline__ float sum_splits(const float* p, int n_splits, size_t stride) {
+    float v = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 16) {
+        float t[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t[i] = s0 + i < n_splits ? p[(s0 + i) * stride] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v += t[i];
+    }
+    return v;
+}
+
+template <int MT, int PRO>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][kLdsRow];
+    __shared__ float row_scale[16];                                      // kSwiglu: 1 / rms of each row
+    __shared__ float head_wgt[PRO == kAttn ? 16 * kMaxLocalHeads * kMaxAttnSplits : 1];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int li = lane % 16, lg = lane / 16;
     const int split = blockIdx.y;
+    const int m = a.m, n = a.n, k = a.k;
     const int n0 = (blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
     const int total_steps = (k + kStep - 1) / kStep;
-    const int step_begin = split * steps_per_split;
-    const int step_end = min(total_steps, step_begin + steps_per_split);
+    const int step_begin = split * a.steps_per_split;
+    const int step_end = min(total_steps, step_begin + a.steps_per_split);
     const int w_row = min(n0 + li, n - 1);
-    const bf16_t* wp = w + static_cast<size_t>(w_row) * k + lg * 32;
+    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + lg * 32;
 
     f32x4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // ---- what the prologue needs once per workgroup
+    int head_begin = 0;
+    if constexpr (PRO == kSwiglu) {
+        if (tid < 16) {
+            float inv = 1.f;
+            if (a.ss_in && tid < m) {
+                const float ss = sum_splits(a.ss_in + tid, a.ss_splits, m);
+                inv = 1.0f / sqrtf(ss * a.inv_hidden + a.eps);
+            }
+            row_scale[tid] = inv;
+        }
+        __syncthreads();
+    }
+    if constexpr (PRO == kAttn) {
+        // weight of split s for (row r, head): exp(max_s - max) / sum_s exp(max_s - max) * l_s
+        head_begin = (step_begin * kStep) / a.hd;
+        const int head_end = min(a.nq, (min(k, step_end * kStep) + a.hd - 1) / a.hd);
+        const int n_local = head_end - head_begin;
+        const int rows = m * a.nq;
+        // 16 lanes per (row, head) pair, each lane four of the (at most 64) splits, so that all loads of a
+        // pair are in flight together
+        const int sub = tid % 16;
+        for (int pair = tid / 16; pair < 16 * kMaxLocalHeads; pair += 16) {
+            const int r = pair / kMaxLocalHeads, hl = pair % kMaxLocalHeads;
+            if (r >= m || hl >= n_local) continue;                 // the same for all 16 lanes of the pair
+            const size_t row = static_cast<size_t>(r) * a.nq + head_begin + hl;
+            float ms[4], ls[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int sp = sub + 16 * i;
+                const bool has = sp < a.a_splits;
+                const float* p = a.part_ml + (static_cast<size_t>(has ? sp : 0) * rows + row) * 2;
+                ms[i] = has ? p[0] : -INFINITY;
+                ls[i] = has ? p[1] : 0.f;
+            }
+            float mx = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
+            mx = fmaxf(mx, __shfl_xor(mx, 1, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 2, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 4, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 8, kWave));
+            float wg[4], denom = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                wg[i] = ms[i] == -INFINITY ? 0.f : __expf(ms[i] - mx);
+                denom += wg[i] * ls[i];
+            }
+            denom += __shfl_xor(denom, 1, kWave);
+            denom += __shfl_xor(denom, 2, kWave);
+            denom += __shfl_xor(denom, 4, kWave);
+            denom += __shfl_xor(denom, 8, kWave);
+            const float inv = 1.0f / denom;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) head_wgt[pair * kMaxAttnSplits + sub + 16 * i] = wg[i] * inv;
+        }
+        __syncthreads();
+    }
+
+    float ss_acc = 0.f;   // kNorm: this thread's share of its row's sum of squares
     // staging of x: MT*16 rows x 128 columns = MT*16*16 chunks of 16 bytes, 256 threads
     auto stage = [&](int buf, int step) {
         const int k0 = step * kStep;
 #pragma unroll
         for (int c = tid; c < MT * 16 * 16; c += 256) {
             const int r = c / 16, col = (c % 16) * 8;
-            const bool ok = r < m && k0 + col < k;
-            const uint4 v = load16(x + static_cast<size_t>(r) * k + k0 + col, ok);
+            const int kc = k0 + col;
+            const bool ok = r < m && kc < k;
+            uint4 v = uint4{0u, 0u, 0u, 0u};
+            if constexpr (PRO == kPlain) {
+                v = load16(a.x + static_cast<size_t>(r) * k + kc, ok);
+            } else if (ok) {
+                float f[8];
+                if constexpr (PRO == kNorm) {
+                    const size_t idx = static_cast<size_t>(r) * k + kc;
+                    load8f(a.h_in + idx, f);
+                    if (a.delta) add_splits8(a.delta + idx, a.delta_splits, static_cast<size_t>(m) * k, f);
+                    if (blockIdx.x == 0) {
+                        *reinterpret_cast<f32x4*>(a.h_out + idx) = f32x4{f[0], f[1], f[2], f[3]};
+                        *reinterpret_cast<f32x4*>(a.h_out + idx + 4) = f32x4{f[4], f[5], f[6], f[7]};
+                    }
+                    const uint4 wv = *reinterpret_cast<const uint4*>(a.norm_w + kc);
+                    const uint32_t wb[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        ss_acc += f[j] * f[j];
+                        const uint32_t bits = (j & 1) ? (wb[j / 2] & 0xffff0000u) : (wb[j / 2] << 16);
+                        f[j] *= __uint_as_float(bits);
+                    }
+                } else if constexpr (PRO == kSwiglu) {
+                    float g[8] = {}, u[8] = {};
+                    const size_t idx = static_cast<size_t>(r) * 2 * k + kc;
+                    const size_t stride = static_cast<size_t>(m) * 2 * k;
+                    add_splits8(a.gu + idx, a.gu_splits, stride, g);
+                    add_splits8(a.gu + idx + k, a.gu_splits, stride, u);
+                    const float inv = row_scale[r];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float gg = g[j] * inv;
+                        f[j] = (u[j] * inv) * (gg / (1.0f + __expf(-gg)));
+                    }
+                } else {  // kAttn
+                    const int head = kc / a.hd, d = kc % a.hd;
+                    const float* wl = head_wgt + (r * kMaxLocalHeads + head - head_begin) * kMaxAttnSplits;
+                    const size_t rows = static_cast<size_t>(m) * a.nq;
+                    const float* po = a.part_o + (static_cast<size_t>(r) * a.nq + head) * a.hd + d;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = 0.f;
+                    for (int s0 = 0; s0 < a.a_splits; s0 += kInFlight) {
+                        float t[kInFlight][8];
+#pragma unroll
+                        for (int i = 0; i < kInFlight; ++i) {
+                            if (s0 + i < a.a_splits) {
+                                load8f(po + (s0 + i) * rows * a.hd, t[i]);
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < 8; ++j) t[i][j] = 0.f;
+                            }
+                        }
+#pragma unroll
+                        for (int i = 0; i < kInFlight; ++i) {
+                            const float wt = s0 + i < a.a_splits ? wl[s0 + i] : 0.f;
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) f[j] += wt * t[i][j];
+                        }
+                    }
+                }
+                v = pack8(f);
+            }
             *reinterpret_cast<uint4*>(&xs[buf][r][col]) = v;
         }
     };
     uint4 a_cur[4], a_next[4];
-    auto load_w = [&](uint4* a, int step) {
+    auto load_w = [&](uint4* av, int step) {
         const int k0 = step * kStep + lg * 32;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) a[q] = load16(wp + static_cast<size_t>(step) * kStep + q * 8, k0 + q * 8 < k);
+        for (int q = 0; q < 4; ++q) av[q] = load16(wp + static_cast<size_t>(step) * kStep + q * 8, k0 + q * 8 < k);
     };
 
     if (step_begin < step_end) {
@@ -80,16 +291,28 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
         }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, a_cur[q]);
+            const bf16x8 av = __builtin_bit_cast(bf16x8, a_cur[q]);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const uint4 bv = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + li][lg * 32 + q * 8]);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
             }
         }
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < 4; ++q) a_cur[q] = a_next[q];
+    }
+    if constexpr (PRO == kNorm) {
+        // the 16 threads that staged a row sit side by side in one wavefront
+        if (blockIdx.x == 0) {
+            float ss = ss_acc;
+            ss += __shfl_xor(ss, 1, kWave);
+            ss += __shfl_xor(ss, 2, kWave);
+            ss += __shfl_xor(ss, 4, kWave);
+            ss += __shfl_xor(ss, 8, kWave);
+            const int r = tid / 16;
+            if (tid % 16 == 0 && r < m) a.ss_out[split * m + r] = ss;
+        }
     }
     // D layout: lane (li, lg) holds rows lg*4 + v of the 16 x 16 tile (an n index) at column li (an m index)
 #pragma unroll
@@ -101,15 +324,25 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
             const int nn = n0 + lg * 4 + v;
             if (nn >= n) continue;
             float val = acc[t][v];
-            if (out_bf16) {
-                if (bias) val += to_float(bias[nn]);
-                out_bf16[static_cast<size_t>(mm) * n + nn] = from_float<bf16_t>(val);
-            } else {
-                if (bias) val += to_float(bias[nn]);
-                out_f32[(static_cast<size_t>(split) * m + mm) * n + nn] = val;
-            }
+            if (a.bias) val += to_float(a.bias[nn]);
+            if (a.out_bf16)
+                a.out_bf16[static_cast<size_t>(mm) * n + nn] = from_float<bf16_t>(val);
+            else
+                a.out_f32[(static_cast<size_t>(split) * m + mm) * n + nn] = val;
         }
     }
+}
+
+static int check_splits(int k, int n_splits, int* steps_per_split) {
+    const int total_steps = (k + kStep - 1) / kStep;
+    if (n_splits < 1 || n_splits > total_steps) return EGPT_BAD_ARGUMENT;
+    *steps_per_split = (total_steps + n_splits - 1) / n_splits;
+    if ((n_splits - 1) * *steps_per_split >= total_steps) return EGPT_BAD_ARGUMENT;  // an empty split
+    return EGPT_OK;
+}
+
+static dim3 skinny_grid(int n, int n_splits) {
+    return dim3((n + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock), n_splits);
 }
 
 }  // namespace egpt
@@ -124,23 +357,85 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
         return EGPT_BAD_ARGUMENT;
     if (m > 64 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
     if (n_splits > 1 && (bias || out_bf16)) return EGPT_BAD_ARGUMENT;
-    const int total_steps = (k + kStep - 1) / kStep;
-    if (n_splits > total_steps) return EGPT_BAD_ARGUMENT;
-    const int steps_per_split = (total_steps + n_splits - 1) / n_splits;
-    if ((n_splits - 1) * steps_per_split >= total_steps) return EGPT_BAD_ARGUMENT;  // an empty split
-    dim3 grid((n + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock), n_splits);
+    SkinnyArgs a = {};
+    if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
+    a.x = static_cast<const bf16_t*>(x);
+    a.w = static_cast<const bf16_t*>(w);
+    a.bias = static_cast<const bf16_t*>(bias);
+    a.out_f32 = out_f32;
+    a.out_bf16 = static_cast<bf16_t*>(out_bf16);
+    a.m = m; a.n = n; a.k = k;
+    const dim3 grid = skinny_grid(n, n_splits);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bf16_t* xp = static_cast<const bf16_t*>(x);
-    const bf16_t* wp = static_cast<const bf16_t*>(w);
-    const bf16_t* bp = static_cast<const bf16_t*>(bias);
-    bf16_t* ob = static_cast<bf16_t*>(out_bf16);
-    const int mt = (m + 15) / 16;
-    switch (mt) {
-        case 1: gemm_skinny_kernel<1><<<grid, 256, 0, s>>>(xp, wp, bp, out_f32, ob, m, n, k, steps_per_split); break;
-        case 2: gemm_skinny_kernel<2><<<grid, 256, 0, s>>>(xp, wp, bp, out_f32, ob, m, n, k, steps_per_split); break;
-        case 3: gemm_skinny_kernel<3><<<grid, 256, 0, s>>>(xp, wp, bp, out_f32, ob, m, n, k, steps_per_split); break;
-        default: gemm_skinny_kernel<4><<<grid, 256, 0, s>>>(xp, wp, bp, out_f32, ob, m, n, k, steps_per_split); break;
+    switch ((m + 15) / 16) {
+        case 1: gemm_skinny_kernel<1, kPlain><<<grid, 256, 0, s>>>(a); break;
+        case 2: gemm_skinny_kernel<2, kPlain><<<grid, 256, 0, s>>>(a); break;
+        case 3: gemm_skinny_kernel<3, kPlain><<<grid, 256, 0, s>>>(a); break;
+        default: gemm_skinny_kernel<4, kPlain><<<grid, 256, 0, s>>>(a); break;
     }
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// out[split][m][n] = partial sums of ((h_in + sum delta) * norm_w) w^T; h_out = h_in + sum delta;
+// ss_out[split][m] = sums of squares of h_out over the split's k range.  m <= 16, k % 8 == 0.
+extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits,
+                                     const void* norm_w, const void* w, float* out, float* ss_out, int m, int n, int k,
+                                     int n_splits, void* stream) {
+    if (!h_in || !h_out || h_in == h_out || !norm_w || !w || !out || !ss_out || m <= 0 || n <= 0 || k <= 0 ||
+        delta_splits < 0 || (delta && delta_splits == 0))
+        return EGPT_BAD_ARGUMENT;
+    if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
+    SkinnyArgs a = {};
+    if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
+    a.w = static_cast<const bf16_t*>(w);
+    a.out_f32 = out;
+    a.m = m; a.n = n; a.k = k;
+    a.h_in = h_in; a.h_out = h_out; a.delta = delta; a.delta_splits = delta ? delta_splits : 0;
+    a.norm_w = static_cast<const bf16_t*>(norm_w);
+    a.ss_out = ss_out;
+    gemm_skinny_kernel<1, kNorm><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// out[split][m][n] = partial sums of swiglu(inv_rms * sum gate_up) w^T, gate_up [gu_splits][m][2k];
+// inv_rms[m] = 1 / sqrt(sum_s ss_in[s][m] / hidden + eps), or 1 if ss_in is null.
+extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits,
+                                       int hidden, float eps, const void* w, float* out, int m, int n, int k,
+                                       int n_splits, void* stream) {
+    if (!gate_up || gu_splits < 1 || !w || !out || m <= 0 || n <= 0 || k <= 0 || (ss_in && (ss_splits < 1 || hidden < 1)))
+        return EGPT_BAD_ARGUMENT;
+    if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
+    SkinnyArgs a = {};
+    if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
+    a.w = static_cast<const bf16_t*>(w);
+    a.out_f32 = out;
+    a.m = m; a.n = n; a.k = k;
+    a.gu = gate_up; a.gu_splits = gu_splits; a.ss_in = ss_in; a.ss_splits = ss_splits;
+    a.inv_hidden = ss_in ? 1.0f / static_cast<float>(hidden) : 0.f;
+    a.eps = eps;
+    gemm_skinny_kernel<1, kSwiglu><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// out[split][m][n] = partial sums of (combined attention output) w^T; part_o [a_splits][m*nq][hd] unnormalised
+// partial outputs, part_ml [a_splits][m*nq][2] their (maximum, sum); k = nq * hd.
+extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd,
+                                     const void* w, float* out, int m, int n, int n_splits, void* stream) {
+    if (!part_o || !part_ml || a_splits < 1 || nq < 1 || hd < 1 || !w || !out || m <= 0 || n <= 0)
+        return EGPT_BAD_ARGUMENT;
+    const int k = nq * hd;
+    if (m > 16 || (hd % 8) != 0 || a_splits > kMaxAttnSplits) return EGPT_UNSUPPORTED_SIZE;
+    SkinnyArgs a = {};
+    if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
+    if ((a.steps_per_split * kStep + hd - 1) / hd + 1 > kMaxLocalHeads) return EGPT_UNSUPPORTED_SIZE;
+    a.w = static_cast<const bf16_t*>(w);
+    a.out_f32 = out;
+    a.m = m; a.n = n; a.k = k;
+    a.part_o = part_o; a.part_ml = part_ml; a.a_splits = a_splits; a.nq = nq; a.hd = hd;
+    gemm_skinny_kernel<1, kAttn><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

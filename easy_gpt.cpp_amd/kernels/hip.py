@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 3:
+    if lib.egpt_abi_version() != 4:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -46,11 +46,16 @@ class HipKernels:
             "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
             "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
             "egpt_swiglu": [vp, i, vp, i, i, i, vp],
-            "egpt_qkv_rope_store": [vp, i, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp],
+            "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, vp],
+            "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, vp],
+            "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
+            "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
-            "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp],
+            "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
         }
@@ -185,6 +190,86 @@ class HipKernels:
         per = -(-steps // s)
         return -(-steps // per)
 
+    fused_rows = 16     # products with a computed x operand take at most this many rows
+
+    def product_normed(self, h, delta, norm_weight, w):
+        """((h + delta) * norm_weight) w^T without the rows' 1/rms factor, for few rows in bfloat16.
+        Returns (float32 partial sums [S, T, N], row sums of squares [S, T], h + delta as a new tensor),
+        or None if this case is not covered (the caller then runs the norm by itself)."""
+        t, k = h.shape
+        n = w.shape[0]
+        if w.dtype != _BF16 or not 0 < t <= self.fused_rows or k % 8 or not h.is_cuda:
+            return None
+        if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
+            return None
+        self._need(h, "h", _F32)
+        self._need(w, "w", _BF16, (n, k))
+        self._need(norm_weight, "norm_weight", _BF16, (k,))
+        d_splits = 0
+        if delta is not None:
+            d_splits = int(delta.shape[0])
+            self._need(delta, "delta", _F32, (d_splits, t, k))
+        s = self._n_splits(t, n, k)
+        out = torch.empty((s, t, n), dtype=_F32, device=h.device)
+        ss = torch.empty((s, t), dtype=_F32, device=h.device)
+        h_new = torch.empty_like(h)
+        self._run("egpt_gemm_skinny_norm", h.data_ptr(), h_new.data_ptr(), self._ptr(delta), d_splits,
+                  norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, self._stream())
+        return out, ss, h_new
+
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=16):
+        """swiglu(scale * sum gate_up) w^T for float32 partial sums gate_up [S, T, 2I]; scale is the rows' 1/rms
+        from row_ss [S2, T] (or 1).  Returns float32 partial sums [S3, T, N] or None if not covered."""
+        if gate_up.dim() != 3 or gate_up.dtype != _F32 or w.dtype != _BF16:
+            return None
+        g_splits, t, two_i = gate_up.shape
+        n, k = w.shape
+        if two_i != 2 * k or not 0 < t <= self.fused_rows or k % 8:
+            return None
+        self._need(gate_up, "gate_up", _F32)
+        self._need(w, "w", _BF16)
+        ss_splits = 0
+        if row_ss is not None:
+            ss_splits = int(row_ss.shape[0])
+            self._need(row_ss, "row_ss", _F32, (ss_splits, t))
+        s = min(self._n_splits(t, n, k), max_splits)
+        steps = -(-k // 128)
+        s = -(-steps // -(-steps // s))
+        out = torch.empty((s, t, n), dtype=_F32, device=w.device)
+        self._run("egpt_gemm_skinny_swiglu", gate_up.data_ptr(), int(g_splits), self._ptr(row_ss), ss_splits, int(hidden),
+                  float(eps), w.data_ptr(), out.data_ptr(), t, n, k, s, self._stream())
+        return out
+
+    def product_attention(self, part_o, part_ml, w, max_splits=4):
+        """(combined attention output) w^T from the parts of a split attention: part_o [S, T, nq, hd],
+        part_ml [S, T, nq, 2].  Returns float32 partial sums [S2, T, N] or None if not covered."""
+        a_splits, t, nq, hd = part_o.shape
+        n, k = w.shape
+        if w.dtype != _BF16 or k != nq * hd or not 0 < t <= self.fused_rows or hd % 8 or a_splits > 64:
+            return None
+        self._need(part_o, "part_o", _F32)
+        self._need(part_ml, "part_ml", _F32, (a_splits, t, nq, 2))
+        self._need(w, "w", _BF16)
+        s = min(self._n_splits(t, n, k), max_splits)
+        steps = -(-k // 128)
+        per = -(-steps // s)
+        s = -(-steps // per)
+        if -(-per * 128 // hd) + 1 > 8:
+            return None
+        out = torch.empty((s, t, n), dtype=_F32, device=w.device)
+        self._run("egpt_gemm_skinny_attn", part_o.data_ptr(), part_ml.data_ptr(), int(a_splits), int(nq), int(hd),
+                  w.data_ptr(), out.data_ptr(), t, n, s, self._stream())
+        return out
+
+    def combine_attention(self, part_o, part_ml, out):
+        """out act [T, nq*hd] from the parts of a split attention (what paged_attention does with combine=True)."""
+        a_splits, t, nq, hd = part_o.shape
+        self._need(part_o, "part_o", _F32)
+        self._need(part_ml, "part_ml", _F32, (a_splits, t, nq, 2))
+        self._need(out, "out", _BF16, (t, nq * hd))
+        self._run("egpt_attention_combine", part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), t * nq, hd,
+                  int(a_splits), self._stream())
+
     def product(self, x, w):
         """x w^T for a consumer that takes partial sums: returns act [m, n], or float32 [splits, m, n] whose sum
         over splits is the product (few rows in bfloat16: the k range is split over workgroups)."""
@@ -202,8 +287,9 @@ class HipKernels:
         return self.linear(x, w, None, out)
 
     def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
-                       page_size, out=None):
-        """qkv: act [T, W] or float32 partial sums [S, T, W]; out: act [T, W] (default: qkv itself, in place)."""
+                       page_size, out=None, row_ss=None, hidden=0, eps=0.0):
+        """qkv: act [T, W] or float32 partial sums [S, T, W]; out: act [T, W] (default: qkv itself, in place).
+        row_ss float32 [S2, T]: the product still lacks each row's factor 1/sqrt(sum_s row_ss[s] / hidden + eps)."""
         width = (nq + 2 * nkv) * hd
         t = qkv.shape[-2]
         if out is None:
@@ -223,13 +309,20 @@ class HipKernels:
         if slots is not None:
             self._need(slots, "slots", _I32, (t,))
             self._caches(k_cache, v_cache, out.dtype, nkv, page_size, hd)
-        self._run("egpt_qkv_rope_store", qkv.data_ptr(), splits, out.data_ptr(), self._ptr(bias), positions.data_ptr(),
+        ss_splits = 0
+        if row_ss is not None:
+            ss_splits = int(row_ss.shape[0])
+            self._need(row_ss, "row_ss", _F32, (ss_splits, t))
+        self._run("egpt_qkv_rope_store", qkv.data_ptr(), splits, self._ptr(row_ss), ss_splits, int(hidden), float(eps),
+                  out.data_ptr(), self._ptr(bias), positions.data_ptr(),
                   self._ptr(inv_freq) if rotary_dim else None, int(rotary_dim), self._ptr(slots),
                   self._ptr(k_cache), self._ptr(v_cache), t, nq, nkv, hd, page_size, dt, self._stream())
         return out
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd, page_size,
-                        scale, window, max_q_len, max_kv_len):
+                        scale, window, max_q_len, max_kv_len, combine=True):
+        """combine=False: when the kernel splits the key range, leave the parts to the caller and return
+        (part_o [S, T, nq, hd], part_ml [S, T, nq, 2]); `out` is then not written.  Returns None otherwise."""
         t = qkv.shape[0]
         b, width = block_table.shape
         dt = self._act(qkv, "qkv")
@@ -246,9 +339,28 @@ class HipKernels:
         if qkv.dtype == _BF16 and hd in (64, 128) and page_size % 16 == 0:
             # matrix-core kernel; the key range is split when there are too few (request, kv head) pairs to fill
             # the GPU, which is the case when only decoded tokens are in the batch
+            if max_q_len == 1 and t == b and nq // nkv <= 16:
+                # only decoded tokens: workgroups of four wavefronts per (request, kv head, key split); the key
+                # range is split over workgroups when the requests alone do not fill the GPU.  Parts that the
+                # output projection combines are read by every column of workgroups there, so they stay few.
+                # The kernel is a chain of round trips to memory: a wavefront takes one round per 4 (head size
+                # 64) or 2 key blocks of 32 keys, so the split aims at one round per wavefront.
+                key_blocks = -(-max_kv_len // 32)
+                per_round = 4 * (4 if hd == 64 else 2)
+                n_splits = max(1, min(-(-key_blocks // per_round), 8 if not combine else 16,
+                                      max(1, 2048 // (b * nkv))))
+                part_o = part_ml = None
+                if n_splits > 1:
+                    part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)
+                    part_ml = torch.empty((n_splits, t, nq, 2), dtype=_F32, device=qkv.device)
+                self._run("egpt_paged_attention_decode", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
+                          self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
+                          q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale), int(window),
+                          n_splits, 4, 1 if combine else 0, self._stream())
+                return (part_o, part_ml) if (n_splits > 1 and not combine) else None
             n_splits = 1
             if max_q_len == 1:
-                n_splits = max(1, min(2048 // (b * nkv), -(-max_kv_len // 64), 64))
+                n_splits = max(1, min(1024 // (b * nkv), -(-max_kv_len // 64), 64))
             part_o = part_ml = None
             if n_splits > 1:
                 part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)
@@ -256,8 +368,9 @@ class HipKernels:
             self._run("egpt_paged_attention_mfma", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
                       self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
                       q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, hd, page_size,
-                      float(scale), int(window), n_splits, 16 if max_q_len == 1 else 32, self._stream())
-            return
+                      float(scale), int(window), n_splits, 16 if max_q_len == 1 else 32, 1 if combine else 0,
+                      self._stream())
+            return (part_o, part_ml) if (n_splits > 1 and not combine) else None
         self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
                   nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())

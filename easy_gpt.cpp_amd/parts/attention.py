@@ -17,12 +17,13 @@ import math
 import torch
 
 from .. import kernels
-from .base import CacheNeed, Mixer, make_part, register_part
+from .base import CacheNeed, Mixer, PendingNorm, make_part, register_part
 from .spec import ParamSpec, PartSpec
 
 
 class GQAttention(Mixer):
     graph_safe = True
+    takes_pending_norm = True
 
     def __init__(
         self,
@@ -93,19 +94,36 @@ class GQAttention(Mixer):
     # ------------------------------------------------------------------ computation
     def forward(self, x, ctx, cache, state=None):
         k = kernels.backend()
-        t = x.shape[0]
         width = self.q_size + 2 * self.kv_size
-        prod = k.product(x, self.w_qkv)                 # act [T, W], or float32 partial sums [S, T, W]
-        qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=x.dtype, device=x.device)
+        rot = self.position.rotary(x.h.device if isinstance(x, PendingNorm) else x.device)
+        # ---- q, k, v.  With few tokens the residual addition and the norm before this layer fold into the
+        # product's staging of x; the rows' 1/rms factor is applied by the epilogue kernel below.
+        scale_args = {}
+        prod = None
+        if isinstance(x, PendingNorm):
+            fused = None
+            rms = x.rms()
+            if rms is not None and rot is not None and hasattr(k, "product_normed"):
+                fused = k.product_normed(x.h, x.delta, rms[0], self.w_qkv)
+            if fused is not None:
+                prod, row_ss, h_new = fused
+                x.applied(h_new)
+                scale_args = dict(row_ss=row_ss, hidden=self.hidden_size, eps=rms[1])
+                dtype, device, t = self.w_qkv.dtype, h_new.device, h_new.shape[0]
+            else:
+                x = x.materialize()
+        if prod is None:
+            prod = k.product(x, self.w_qkv)             # act [T, W], or float32 partial sums [S, T, W]
+            dtype, device, t = x.dtype, x.device, x.shape[0]
+        qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=dtype, device=device)
         slots = cache.slots if cache.writes else None
-        rot = self.position.rotary(x.device)
         common = dict(
             k_cache=cache.k, v_cache=cache.v, nq=self.n_heads, nkv=self.n_kv_heads,
             hd=self.head_dim, page_size=cache.page_size,
         )
         if rot is not None:
             inv_freq, rotary_dim = rot
-            k.qkv_rope_store(prod, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, out=qkv, **common)
+            k.qkv_rope_store(prod, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, out=qkv, **common, **scale_args)
         else:
             # bias, then the position encoding's own transform, then the store
             if self.b_qkv is not None or prod.dim() == 3:
@@ -115,15 +133,25 @@ class GQAttention(Mixer):
             self.position.apply(q_view, k_view, ctx.positions)
             if slots is not None:
                 k.qkv_rope_store(qkv, None, ctx.positions, None, 0, slots, out=qkv, **common)
-        attn = torch.empty((t, self.q_size), dtype=x.dtype, device=x.device)
-        k.paged_attention(
-            qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
+        # ---- attention over the cache.  If the kernel splits the keys, the output projection combines the parts.
+        attn = torch.empty((t, self.q_size), dtype=dtype, device=device)
+        want_parts = self.b_o is None and hasattr(k, "product_attention") and t <= getattr(k, "fused_rows", 0)
+        args = dict(
             nq=self.n_heads, nkv=self.n_kv_heads, hd=self.head_dim, page_size=cache.page_size,
             scale=self.scale, window=self.window or 0, max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len,
         )
+        if want_parts:
+            args["combine"] = False
+        parts = k.paged_attention(qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
+                                  **args)
+        if parts is not None:
+            out = k.product_attention(parts[0], parts[1], self.w_o)
+            if out is not None:
+                return out
+            k.combine_attention(parts[0], parts[1], attn)
         if self.b_o is None:
             return k.product(attn, self.w_o)            # the residual add that follows sums partial sums up
-        out = torch.empty((t, self.hidden_size), dtype=x.dtype, device=x.device)
+        out = torch.empty((t, self.hidden_size), dtype=dtype, device=device)
         k.linear(attn, self.w_o, self.b_o, out)
         return out
 

@@ -111,6 +111,32 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class PendingNorm:
+    """x = norm(h + delta), not computed yet.
+
+    A block hands this to a mixer or feed-forward that sets `takes_pending_norm`: such a part may fold the
+    addition and the norm into its own first kernel (`rms()` gives it the norm's weight and eps when the
+    norm is an RMSNorm) and must then call `applied(h_new)` with the updated residual stream; or it calls
+    `materialize()` to get x as a tensor, as any other part would have been given.
+    """
+
+    def __init__(self, h: torch.Tensor, delta: torch.Tensor | None, norm: "Norm"):
+        self.h, self.delta, self.norm = h, delta, norm
+        self.h_after: torch.Tensor | None = None
+
+    def rms(self):
+        """(weight, eps) if the norm is y = x / rms(x) * weight, else None."""
+        return self.norm.rms_params() if hasattr(self.norm, "rms_params") else None
+
+    def applied(self, h_new: torch.Tensor) -> None:
+        self.h_after = h_new
+
+    def materialize(self) -> torch.Tensor:
+        x = self.norm.forward(self.h, self.delta)      # adds delta into h in place
+        self.h_after = self.h
+        return x
+
+
 class PositionEncoding(Part):
     """How token positions enter a mixer.
 
@@ -134,6 +160,8 @@ class Mixer(Part):
     state a StateView if `state_need()` is not None.
     """
 
+    takes_pending_norm = False     # True: forward may be given a PendingNorm instead of x
+
     def cache_need(self) -> CacheNeed | None:
         return None
 
@@ -147,6 +175,8 @@ class Mixer(Part):
 class FeedForward(Part):
     """forward(x) -> act [T, H] for x act [T, H]; tokens are independent."""
 
+    takes_pending_norm = False
+
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         raise NotImplementedError
 
@@ -154,10 +184,11 @@ class FeedForward(Part):
 class Block:
     """Arrangement of one layer's parts around the residual stream.
 
-    forward(h, delta, ctx, cache, state) -> delta': `h` float32 [T, H] is updated in
-    place; `delta` is the not-yet-added output of the previous layer (None for the
-    first) and the return value the not-yet-added output of this one, so that the
-    addition fuses with the next norm.
+    forward(h, delta, ctx, cache, state) -> (h', delta'): `h` float32 [T, H] is the residual
+    stream and `delta` the not-yet-added output of the previous layer (None for the first);
+    h' is the residual stream after this layer's additions but one (it may be `h` updated in
+    place, or a new tensor) and delta' this layer's not-yet-added output, so that the
+    addition fuses with whatever norm comes next.
     """
 
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):

@@ -6,15 +6,19 @@ The additions are made in float32 inside the following norm's kernel.
 """
 from __future__ import annotations
 
-from .base import Block, register_part
+from .base import Block, PendingNorm, register_part
 
 
 class PreNormBlock(Block):
     def forward(self, h, delta, ctx, cache, state):
-        x = self.mixer_norm.forward(h, delta)          # h += delta; x = N1(h)
+        pending = PendingNorm(h, delta, self.mixer_norm)                      # x = N1(h + delta)
+        x = pending if self.mixer.takes_pending_norm else pending.materialize()
         a = self.mixer.forward(x, ctx, cache, state)
-        x = self.feed_forward_norm.forward(h, a)       # h += a;     x = N2(h)
-        return self.feed_forward.forward(x, ctx)       # added by whoever comes next
+        h = pending.h_after
+        pending = PendingNorm(h, a, self.feed_forward_norm)                   # x = N2(h + a)
+        x = pending if self.feed_forward.takes_pending_norm else pending.materialize()
+        m = self.feed_forward.forward(x, ctx)
+        return pending.h_after, m                                            # m is added by whoever comes next
 
 
 register_part("block", "pre_norm", PreNormBlock)

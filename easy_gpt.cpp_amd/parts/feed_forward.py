@@ -11,12 +11,13 @@ from __future__ import annotations
 import torch
 
 from .. import kernels
-from .base import FeedForward, register_part
+from .base import FeedForward, PendingNorm, register_part
 from .spec import ParamSpec
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    takes_pending_norm = True
 
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
@@ -42,8 +43,27 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx=None):
         k = kernels.backend()
+        # With few tokens: the norm folds into the first product's staging of x, and SwiGLU (with the rows'
+        # 1/rms factor) into the second's.
+        if isinstance(x, PendingNorm):
+            rms = x.rms()
+            fused = None
+            if rms is not None and hasattr(k, "product_normed") and self.intermediate_size % 8 == 0:
+                fused = k.product_normed(x.h, x.delta, rms[0], self.w_gate_up)
+            if fused is not None:
+                gate_up, row_ss, h_new = fused
+                x.applied(h_new)
+                out = k.product_swiglu(gate_up, row_ss, self.hidden_size, rms[1], self.w_down)
+                if out is None:
+                    raise RuntimeError("the fused SwiGLU product does not cover this size")
+                return out
+            x = x.materialize()
         t = x.shape[0]
         gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]
+        if gate_up.dim() == 3 and hasattr(k, "product_swiglu"):
+            out = k.product_swiglu(gate_up, None, self.hidden_size, 0.0, self.w_down)
+            if out is not None:
+                return out
         act = torch.empty((t, self.intermediate_size), dtype=x.dtype, device=x.device)
         k.swiglu(gate_up, act)
         return k.product(act, self.w_down)               # added to the residual stream by the next norm

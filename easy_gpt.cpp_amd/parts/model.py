@@ -122,7 +122,7 @@ class Model:
             block = self.layers[run.layer]
             cache = ctx.cache_view(run.cache, run.writes_cache) if run.cache is not None else None
             state = ctx.state_view(run.state) if run.state is not None else None
-            delta = block.forward(h, delta, ctx, cache, state)
+            h, delta = block.forward(h, delta, ctx, cache, state)
         if ctx.want_rows is None or ctx.want_rows.shape[0] == 0:
             return None
         x = self.final_norm.forward_rows(h, delta, ctx.want_rows)

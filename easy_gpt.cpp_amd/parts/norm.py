@@ -30,6 +30,9 @@ class RMSNorm(Norm):
     def load(self, get, dtype, device):
         self.weight = self._to(get(self.prefix + "weight").reshape(self.hidden_size), "compute", dtype, device)
 
+    def rms_params(self):
+        return self.weight, self.eps
+
     def forward(self, h, delta):
         out = torch.empty(h.shape, dtype=self.weight.dtype, device=h.device)
         kernels.backend().add_rmsnorm(h, delta, self.weight, self.eps, out)

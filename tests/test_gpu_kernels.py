@@ -152,6 +152,84 @@ def test_consumers_add_partial_sums_up(k):
     assert torch.equal(vc[3, :, :, 2], got.view(t, -1, hd)[3, nq + nkv :])
 
 
+@pytest.mark.parametrize("t,hid,n,d_splits", [(1, 896, 1152, 0), (8, 896, 9728, 4), (16, 200, 130, 3), (5, 1536, 2048, 13)])
+def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
+    # ((h + delta) * norm_weight) w^T with the rows' 1/rms applied afterwards equals rmsnorm(h + delta) w^T
+    dtype = torch.bfloat16
+    h = rnd(t, hid, seed=1, scale=2.0)
+    delta = rnd(d_splits, t, hid, seed=2) if d_splits else None
+    nw = (1 + rnd(hid, seed=3, scale=0.1)).to(dtype)
+    w = rnd(n, hid, dtype=dtype, seed=4, scale=0.05)
+    h0 = h.clone()
+    prod, ss, h_new = k.product_normed(h, delta, nw, w)
+    assert torch.equal(h, h0)                                           # the input stream is left alone
+    summed = h0.clone()
+    for s in range(d_splits):
+        summed += delta[s]
+    assert torch.equal(h_new, summed)
+    sd = summed.double().cpu()
+    assert torch.allclose(ss.double().sum(0).cpu(), (sd * sd).sum(-1), rtol=1e-5)
+    eps = 1e-6
+    inv = 1.0 / torch.sqrt(ss.double().sum(0).cpu() / hid + eps)
+    got = prod.double().sum(0).cpu() * inv[:, None]
+    ref = plain.linear(plain.rms_norm(sd, nw.double().cpu(), eps), w.double().cpu())
+    assert float((got - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+    # and the QKV epilogue applies that factor
+    if n == 1152:
+        nq, nkv, hd, ps = 14, 2, 64, 16
+        positions = torch.zeros(t, dtype=torch.int32, device=DEV)
+        out = torch.empty(t, n, dtype=dtype, device=DEV)
+        kc = torch.zeros(1, nkv, ps, hd, dtype=dtype, device=DEV)
+        vc = torch.zeros(1, nkv, hd, ps, dtype=dtype, device=DEV)
+        inv_freq = torch.ones(hd // 2, device=DEV)
+        k.qkv_rope_store(prod, None, positions, inv_freq, hd, None, kc, vc, nq, nkv, hd, ps, out=out, row_ss=ss, hidden=hid, eps=eps)
+        assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())   # position 0: no rotation
+
+
+@pytest.mark.parametrize("t,inter,n,g_splits", [(8, 4864, 896, 4), (3, 200, 120, 1), (16, 328, 192, 2)])
+def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
+    gu = rnd(g_splits, t, 2 * inter, seed=1, scale=1.5)
+    ss = torch.rand(3, t, generator=torch.Generator().manual_seed(2)).to(DEV) * 50 + 1
+    w = rnd(n, inter, dtype=torch.bfloat16, seed=3, scale=0.05)
+    hidden, eps = 77, 1e-5
+    for row_ss in (None, ss):
+        scale = 1.0 if row_ss is None else (1.0 / torch.sqrt(ss.double().sum(0).cpu() / hidden + eps))[:, None]
+        z = gu.double().sum(0).cpu() * scale
+        g, u = z[:, :inter], z[:, inter:]
+        ref = plain.linear(u * g / (1 + torch.exp(-g)), w.double().cpu())
+        prod = k.product_swiglu(gu, row_ss, hidden, eps, w)
+        assert prod is not None and prod.dim() == 3
+        assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("nq,nkv,hd,batch,ctx", [(14, 2, 64, 8, 700), (12, 2, 128, 3, 300), (14, 2, 64, 1, 2113), (3, 1, 64, 16, 90)])
+def test_output_projection_combines_attention_parts(k, nq, nkv, hd, batch, ctx):
+    # split attention left uncombined, then combined by the output projection: equals combine + plain product
+    dtype, ps = torch.bfloat16, 16
+    seqs = [(1, max(1, ctx - 37 * i % ctx)) for i in range(batch)]
+    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed=5)
+    t = batch
+    qkv = rnd(t, (nq + 2 * nkv) * hd, dtype=dtype, seed=6)
+    q_len = torch.ones(t, dtype=torch.int32)
+    q_start = torch.arange(t, dtype=torch.int32)
+    kv_len = torch.tensor([kv for _, kv in seqs], dtype=torch.int32)
+    args = (kc, vc, table, q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV), nq, nkv, hd, ps, 1.0 / math.sqrt(hd), 0, 1,
+            int(kv_len.max()))
+    out = torch.empty(t, nq * hd, dtype=dtype, device=DEV)
+    assert k.paged_attention(qkv, out, *args) is None
+    parts = k.paged_attention(qkv, torch.empty_like(out), *args, combine=False)
+    if parts is None:            # few requests with short contexts are not split
+        assert int(kv_len.max()) < 512
+        return
+    again = torch.empty_like(out)
+    k.combine_attention(parts[0], parts[1], again)
+    assert float((again.float() - out.float()).abs().max()) <= 2e-2      # other splits, other rounding
+    w = rnd(200, nq * hd, dtype=dtype, seed=7, scale=0.05)
+    prod = k.product_attention(parts[0], parts[1], w)
+    ref = plain.linear(again.double().cpu(), w.double().cpu())
+    assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+
+
 def test_linear_vector_of_the_reference(k):
     # /root/reference/test/matmul_3d_test.cpp:60-87
     x = torch.tensor([[1.0, 2, 3], [4, 5, 6]], device=DEV)

@@ -158,8 +158,7 @@ def test_pre_norm_block(dtype):
     slots = (table[0, (positions // ps).long()] * ps + positions % ps).to(torch.int32)
     one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
     ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(s), kv_len=one(s), max_q_len=s, max_kv_len=s)
-    h = x.to(DEV).clone()
-    delta = block.forward(h, None, ctx, CacheView(kc, vc, ps, table, slots, None, True), None)
+    h, delta = block.forward(x.to(DEV).clone(), None, ctx, CacheView(kc, vc, ps, table, slots, None, True), None)
     got = h.double().cpu() + whole(delta).cpu()
     assert float((h.double().cpu() - a).abs().max()) <= tol(dtype) * float(a.abs().max())
     assert float((got - y).abs().max()) <= tol(dtype) * float(y.abs().max())
