@@ -36,11 +36,15 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     const int kh = blockIdx.y, split = blockIdx.z;
     const int group_size = nq / nkv;
 
-    // which request, and which group of 16*QT rows of it
+    // which request, and which group of 16*QT rows of it; within a request the last rows come first: they
+    // have the most keys to walk, and the launch is over when the longest wavefront is
     int b = 0, grp = blockIdx.x;
     for (; b < n_seqs; ++b) {
         const int groups = (q_len[b] * group_size + 16 * QT - 1) / (16 * QT);
-        if (grp < groups) break;
+        if (grp < groups) {
+            grp = groups - 1 - grp;
+            break;
+        }
         grp -= groups;
     }
     if (b >= n_seqs) return;
@@ -90,89 +94,105 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
         for (int d = 0; d < DT; ++d) o[t][d] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    uint4 k_cur[2][KD], k_nxt[2][KD];
-    uint2 v_cur[2][DT], v_nxt[2][DT];
-    auto load_block = [&](uint4 (*kk)[KD], uint2 (*vv)[DT], int kb) {
+    // Keys are walked in rounds of kRound blocks of 32; the loads of the next round are in flight while this
+    // round computes (a wavefront is alone on its SIMD here, so nothing else hides the latency).
+    constexpr int kRound = 2;
+    uint4 k_cur[kRound][2][KD], k_nxt[kRound][2][KD];
+    uint2 v_cur[kRound][2][DT], v_nxt[kRound][2][DT];
+    auto load_round = [&](uint4 (*kk)[2][KD], uint2 (*vv)[2][DT], int kb0) {
+        int pages[kRound][2];
+        bool live[kRound][2];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            const int key0 = kb * 32 + kt * 16;
-            // a tile is read only if some row of this wave can see one of its keys: then it lies in a page the
-            // request still holds (p_hi < kv; pages wholly behind the window may have been given back)
-            bool live = key0 <= p_hi && key0 + 15 >= lo_first;
-            long page = 0;
-            int off = 0;
-            if (live) {
-                page = table[key0 / page_size];
-                off = key0 % page_size;
-                live = page >= 0;
-                page = live ? page : 0;
-            }
-            const bf16_t* kp = k_cache + ((page * nkv + kh) * page_size + off + lj) * HD + lg * 8;
-            const bf16_t* vp = v_cache + ((page * nkv + kh) * HD + lj) * static_cast<long>(page_size) + off + lg * 4;
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd)
-                kk[kt][kd] = live ? *reinterpret_cast<const uint4*>(kp + kd * 32) : uint4{0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int d = 0; d < DT; ++d)
-                vv[kt][d] = live ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
-                                 : uint2{0u, 0u};
-        }
-    };
-
-    if (my_begin < my_end) load_block(k_cur, v_cur, my_begin);
-    for (int kb = my_begin; kb < my_end; ++kb) {
-        if (kb + 1 < my_end) load_block(k_nxt, v_nxt, kb + 1);
-#pragma unroll
-        for (int t = 0; t < QT; ++t) {
-            float s[2][4];
-            float mx = -INFINITY;
+        for (int i = 0; i < kRound; ++i)
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
-                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+                const int key0 = (kb0 + i) * 32 + kt * 16;
+                // a tile is read only if some row of this wave can see one of its keys: then it lies in a page the
+                // request still holds (p_hi < kv; pages wholly behind the window may have been given back)
+                live[i][kt] = kb0 + i < my_end && key0 <= p_hi && key0 + 15 >= lo_first;
+                pages[i][kt] = table[live[i][kt] ? key0 / page_size : 0];
+            }
+#pragma unroll
+        for (int i = 0; i < kRound; ++i)
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                const int key0 = (kb0 + i) * 32 + kt * 16;
+                const bool ok = live[i][kt] && pages[i][kt] >= 0;
+                const long page = ok ? pages[i][kt] : 0;
+                const int off = ok ? key0 % page_size : 0;
+                const bf16_t* kp = k_cache + ((page * nkv + kh) * page_size + off + lj) * HD + lg * 8;
+                const bf16_t* vp = v_cache + ((page * nkv + kh) * HD + lj) * static_cast<long>(page_size) + off + lg * 4;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k_cur[kt][kd]), q[t][kd],
-                                                                  acc, 0, 0, 0);
+                    kk[i][kt][kd] = ok ? *reinterpret_cast<const uint4*>(kp + kd * 32) : uint4{0u, 0u, 0u, 0u};
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int key = kb * 32 + kt * 16 + lg * 4 + v;
-                    const bool vis = key <= p_row[t] && key >= lo_row[t];
-                    s[kt][v] = vis ? acc[v] * scale : -INFINITY;
-                    mx = fmaxf(mx, s[kt][v]);
-                }
+                for (int d = 0; d < DT; ++d)
+                    vv[i][kt][d] = ok ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
+                                      : uint2{0u, 0u};
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-            const float m_new = fmaxf(m_run[t], mx);
-            const bool none = m_new == -INFINITY;             // no visible key yet for this row
-            const float alpha = none ? 1.f : __expf(m_run[t] - m_new);
-            float sum = 0.f;
-            bf16x8 pb;
+    };
+
+    if (my_begin < my_end) load_round(k_cur, v_cur, my_begin);
+    for (int kb0 = my_begin; kb0 < my_end; kb0 += kRound) {
+        if (kb0 + kRound < my_end) load_round(k_nxt, v_nxt, kb0 + kRound);
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
+        for (int i = 0; i < kRound; ++i) {
+            const int kb = kb0 + i;
+            if (kb >= my_end) break;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float pv = none ? 0.f : __expf(s[kt][v] - m_new);
-                    sum += pv;
-                    pb[kt * 4 + v] = static_cast<__bf16>(pv);
+            for (int t = 0; t < QT; ++t) {
+                float s[2][4];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k_cur[i][kt][kd]),
+                                                                      q[t][kd], acc, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = kb * 32 + kt * 16 + lg * 4 + v;
+                        const bool vis = key <= p_row[t] && key >= lo_row[t];
+                        s[kt][v] = vis ? acc[v] * scale : -INFINITY;
+                        mx = fmaxf(mx, s[kt][v]);
+                    }
                 }
-            l_run[t] = l_run[t] * alpha + sum;
-            m_run[t] = m_new;
+                mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+                const float m_new = fmaxf(m_run[t], mx);
+                const bool none = m_new == -INFINITY;             // no visible key yet for this row
+                const float alpha = none ? 1.f : __expf(m_run[t] - m_new);
+                float sum = 0.f;
+                bf16x8 pb;
 #pragma unroll
-            for (int d = 0; d < DT; ++d) {
-                const uint4 a = uint4{v_cur[0][d].x, v_cur[0][d].y, v_cur[1][d].x, v_cur[1][d].y};
-                f32x4 acc = o[t][d];
-                acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
-                o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb, acc, 0, 0, 0);
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float pv = none ? 0.f : __expf(s[kt][v] - m_new);
+                        sum += pv;
+                        pb[kt * 4 + v] = static_cast<__bf16>(pv);
+                    }
+                l_run[t] = l_run[t] * alpha + sum;
+                m_run[t] = m_new;
+#pragma unroll
+                for (int d = 0; d < DT; ++d) {
+                    const uint4 a = uint4{v_cur[i][0][d].x, v_cur[i][0][d].y, v_cur[i][1][d].x, v_cur[i][1][d].y};
+                    f32x4 acc = o[t][d];
+                    acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+                    o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb, acc, 0, 0, 0);
+                }
             }
         }
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
+        for (int i = 0; i < kRound; ++i)
 #pragma unroll
-            for (int kd = 0; kd < KD; ++kd) k_cur[kt][kd] = k_nxt[kt][kd];
+            for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-            for (int d = 0; d < DT; ++d) v_cur[kt][d] = v_nxt[kt][d];
-        }
+                for (int kd = 0; kd < KD; ++kd) k_cur[i][kt][kd] = k_nxt[i][kt][kd];
+#pragma unroll
+                for (int d = 0; d < DT; ++d) v_cur[i][kt][d] = v_nxt[i][kt][d];
+            }
     }
 
 #pragma unroll

@@ -75,6 +75,60 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
     }
 }
 
+// The same for bfloat16 activations with eight features per thread and load (16-byte loads of the
+// activations, 32 bytes of the residual stream): the form that prompt portions of many tokens take.
+__global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict__ h, const bf16_t* __restrict__ delta,
+                                                               const int32_t* __restrict__ rows,
+                                                               const bf16_t* __restrict__ weight, float eps,
+                                                               bf16_t* __restrict__ out, int hidden) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+    float* hrow = h + src * hidden;
+    const bf16_t* drow = delta ? delta + src * hidden : nullptr;
+    const bool write_back = (rows == nullptr) && (delta != nullptr);
+    float ss = 0.f;
+    for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
+        float4 a = *reinterpret_cast<const float4*>(hrow + j), b = *reinterpret_cast<const float4*>(hrow + j + 4);
+        if (drow) {
+            const uint4 d = *reinterpret_cast<const uint4*>(drow + j);
+            a.x += __uint_as_float(d.x << 16); a.y += __uint_as_float(d.x & 0xffff0000u);
+            a.z += __uint_as_float(d.y << 16); a.w += __uint_as_float(d.y & 0xffff0000u);
+            b.x += __uint_as_float(d.z << 16); b.y += __uint_as_float(d.z & 0xffff0000u);
+            b.z += __uint_as_float(d.w << 16); b.w += __uint_as_float(d.w & 0xffff0000u);
+            if (write_back) {
+                *reinterpret_cast<float4*>(hrow + j) = a;
+                *reinterpret_cast<float4*>(hrow + j + 4) = b;
+            }
+        }
+        ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
+    bf16_t* orow = out + static_cast<size_t>(r) * hidden;
+    for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
+        float4 a = *reinterpret_cast<const float4*>(hrow + j), b = *reinterpret_cast<const float4*>(hrow + j + 4);
+        if (drow && !write_back) {
+            const uint4 d = *reinterpret_cast<const uint4*>(drow + j);
+            a.x += __uint_as_float(d.x << 16); a.y += __uint_as_float(d.x & 0xffff0000u);
+            a.z += __uint_as_float(d.y << 16); a.w += __uint_as_float(d.y & 0xffff0000u);
+            b.x += __uint_as_float(d.z << 16); b.y += __uint_as_float(d.z & 0xffff0000u);
+            b.z += __uint_as_float(d.w << 16); b.w += __uint_as_float(d.w & 0xffff0000u);
+        }
+        const uint4 w = *reinterpret_cast<const uint4*>(weight + j);
+        const float v[8] = {a.x * inv * __uint_as_float(w.x << 16), a.y * inv * __uint_as_float(w.x & 0xffff0000u),
+                            a.z * inv * __uint_as_float(w.y << 16), a.w * inv * __uint_as_float(w.y & 0xffff0000u),
+                            b.x * inv * __uint_as_float(w.z << 16), b.y * inv * __uint_as_float(w.z & 0xffff0000u),
+                            b.z * inv * __uint_as_float(w.w << 16), b.w * inv * __uint_as_float(w.w & 0xffff0000u)};
+        uint4 o;
+        o.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
+        o.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
+        o.z = f32_to_bf16_bits(v[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5])) << 16);
+        o.w = f32_to_bf16_bits(v[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7])) << 16);
+        *reinterpret_cast<uint4*>(orow + j) = o;
+    }
+}
+
 // ----------------------------------------------------------------------------- SwiGLU
 // out = up * gate / (1 + exp(-gate))   (/root/reference/src/cuda/ops/mlp.cu:152-162); [gate | up] per row.
 template <typename T>
@@ -86,6 +140,29 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
         const float g = gate_up.at(t * 2 * inter + j);
         const float u = gate_up.at(t * 2 * inter + inter + j);
         out[i] = from_float<T>(u * (g / (1.0f + expf(-g))));
+    }
+}
+
+// bfloat16, eight features per thread (inter % 8 == 0, one tensor, no partial sums)
+__global__ __launch_bounds__(256) void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out,
+                                                          int n_tokens, int inter) {
+    const size_t chunks_per_row = inter / 8;
+    const size_t total = static_cast<size_t>(n_tokens) * chunks_per_row;
+    for (size_t c = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; c < total;
+         c += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t t = c / chunks_per_row, j = (c % chunks_per_row) * 8;
+        const uint4 g = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + j);
+        const uint4 u = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + inter + j);
+        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+        uint32_t ow[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+            const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+            const float r0 = u0 * (g0 / (1.0f + expf(-g0))), r1 = u1 * (g1 / (1.0f + expf(-g1)));
+            ow[i] = f32_to_bf16_bits(r0) | (static_cast<uint32_t>(f32_to_bf16_bits(r1)) << 16);
+        }
+        *reinterpret_cast<uint4*>(out + t * inter + j) = uint4{ow[0], ow[1], ow[2], ow[3]};
     }
 }
 
@@ -157,6 +234,55 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __rest
     }
 }
 
+// The same for many tokens (prompt portions), full rotation (rotary_dim == hd), one tensor in and out: a
+// thread owns one (token, pair index) and walks the heads, so the angle's sine and cosine are computed once
+// for all heads instead of once per head.
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const T* __restrict__ qkv_in, T* __restrict__ qkv_out,
+                                                                  const T* __restrict__ bias,
+                                                                  const int32_t* __restrict__ positions,
+                                                                  const float* __restrict__ inv_freq,
+                                                                  const int32_t* __restrict__ slots,
+                                                                  T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                                  int n_tokens, int nq, int nkv, int hd, int page_size) {
+    const int half = hd / 2;
+    const int tokens_per_block = blockDim.x / half;
+    const int t = blockIdx.x * tokens_per_block + threadIdx.x / half;
+    const int i = threadIdx.x % half;
+    if (t >= n_tokens || static_cast<int>(threadIdx.x) >= tokens_per_block * half) return;
+    const int n_heads = nq + 2 * nkv;
+    const size_t base = static_cast<size_t>(t) * n_heads * hd;
+    float sn, cs;
+    sincosf(static_cast<float>(positions[t]) * inv_freq[i], &sn, &cs);
+    const long slot = slots ? slots[t] : -1;
+    const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    for (int head = 0; head < n_heads; ++head) {
+        const int lo = head * hd + i, hi = lo + half;
+        float a = to_float(qkv_in[base + lo]) + (bias ? to_float(bias[lo]) : 0.f);
+        float b = to_float(qkv_in[base + hi]) + (bias ? to_float(bias[hi]) : 0.f);
+        const bool is_v = head >= nq + nkv;
+        if (!is_v) {
+            const float ra = a * cs - b * sn, rb = a * sn + b * cs;
+            a = ra;
+            b = rb;
+        }
+        const T ta = from_float<T>(a), tb = from_float<T>(b);
+        qkv_out[base + lo] = ta;
+        qkv_out[base + hi] = tb;
+        if (slot >= 0 && head >= nq) {
+            if (!is_v) {
+                T* dst = k_cache + ((page * nkv + (head - nq)) * page_size + off) * hd;
+                dst[i] = ta;
+                dst[i + half] = tb;
+            } else {
+                T* dst = v_cache + ((page * nkv + (head - nq - nkv)) * hd) * page_size + off;
+                dst[static_cast<long>(i) * page_size] = ta;
+                dst[static_cast<long>(i + half) * page_size] = tb;
+            }
+        }
+    }
+}
+
 }  // namespace egpt
 
 using namespace egpt;
@@ -196,6 +322,13 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, i
     // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for
     const int threads = (delta_splits > 1 || hidden >= 4096) ? 1024 : (hidden >= 2048 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
+    if (dtype == 1 && delta_splits == 0 && hidden % 8 == 0 && n_rows >= 32) {
+        add_rmsnorm_vec8_kernel<<<n_rows, hidden >= 2048 ? 256 : 128, 0, s>>>(
+            h, static_cast<const bf16_t*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
+            static_cast<bf16_t*>(out), hidden);
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     if (dtype == 0)
         add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, make_view<float>(delta, delta_splits, stride), rows,
                                                              static_cast<const float*>(weight), eps,
@@ -218,6 +351,14 @@ extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_t
     const size_t total = static_cast<size_t>(n_tokens) * inter;
     const int blocks = static_cast<int>(total / 256 + 1 > 8192 ? 8192 : total / 256 + 1);
     const size_t stride = total * 2;
+    if (dtype == 1 && n_splits == 0 && inter % 8 == 0) {
+        const size_t chunks = total / 8;
+        const int vblocks = static_cast<int>(chunks / 256 + 1 > 16384 ? 16384 : chunks / 256 + 1);
+        swiglu_vec8_kernel<<<vblocks, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
+                                                   n_tokens, inter);
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     if (dtype == 0)
         swiglu_kernel<float><<<blocks, 256, 0, s>>>(make_view<float>(gate_up, n_splits, stride),
                                                     static_cast<float*>(out), n_tokens, inter);
@@ -246,6 +387,28 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
     const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
+    if (dtype == 1 && n_splits == 0 && !row_ss && rotary_dim == hd && n_tokens >= 64 && hd <= 512) {
+        // many tokens: one thread per (token, pair), the angle shared by all heads.  (bfloat16 only: the
+        // float32 path keeps one kernel per operation whatever the batch, so that its results do not depend
+        // on the batch in any bit.)
+        const int half = hd / 2;
+        const int tpb = 256 / half > 0 ? 256 / half : 1;
+        const int blocks = (n_tokens + tpb - 1) / tpb;
+        if (dtype == 0)
+            qkv_rope_store_rows_kernel<float><<<blocks, 256, 0, s>>>(
+                static_cast<const float*>(qkv_in), static_cast<float*>(qkv_out), static_cast<const float*>(bias),
+                positions, inv_freq, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), n_tokens, nq,
+                nkv, hd, page_size);
+        else if (dtype == 1)
+            qkv_rope_store_rows_kernel<bf16_t><<<blocks, 256, 0, s>>>(
+                static_cast<const bf16_t*>(qkv_in), static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias),
+                positions, inv_freq, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens,
+                nq, nkv, hd, page_size);
+        else
+            return EGPT_BAD_ARGUMENT;
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     const dim3 grid(n_tokens, (nq + 2 * nkv + kHeadsPerBlock - 1) / kHeadsPerBlock);
     const int block = kHeadsPerBlock * hd >= 256 ? 256 : (kHeadsPerBlock * hd >= 128 ? 128 : 64);
     if (dtype == 0)

@@ -43,13 +43,14 @@ def test_embed(k, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,eps", [(72, 1e-6), (896, 1e-5), (3000, 1e-2)])
-def test_add_rmsnorm(k, dtype, hidden, eps):
-    h = rnd(7, hidden, seed=1, scale=2.0)
-    delta = rnd(7, hidden, dtype=dtype, seed=2)
+@pytest.mark.parametrize("hidden,eps,n_rows", [(72, 1e-6, 7), (896, 1e-5, 7), (3000, 1e-2, 7), (896, 1e-6, 70), (3000, 1e-5, 33),
+                                               (100, 1e-6, 40)])
+def test_add_rmsnorm(k, dtype, hidden, eps, n_rows):
+    h = rnd(n_rows, hidden, seed=1, scale=2.0)
+    delta = rnd(n_rows, hidden, dtype=dtype, seed=2)
     w = (1 + rnd(hidden, seed=3, scale=0.1)).to(dtype)
     h0 = h.clone()
-    out = torch.empty(7, hidden, dtype=dtype, device=DEV)
+    out = torch.empty(n_rows, hidden, dtype=dtype, device=DEV)
     k.add_rmsnorm(h, delta, w, eps, out)
     summed = h0 + delta.float()                                   # the residual sum is made in float32
     assert torch.equal(h, summed)
@@ -60,8 +61,9 @@ def test_add_rmsnorm(k, dtype, hidden, eps):
     k.add_rmsnorm(h, None, w, eps, out)
     assert torch.equal(h, h1)
     # rows variant: gathers, adds, does not write back
-    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
-    out3 = torch.empty(3, hidden, dtype=dtype, device=DEV)
+    picked = [6, 0, 3] + (list(range(n_rows - 1, -1, -1)) if n_rows >= 33 else [])
+    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
+    out3 = torch.empty(len(picked), hidden, dtype=dtype, device=DEV)
     k.rows_add_rmsnorm(h, delta, rows, w, eps, out3)
     assert torch.equal(h, h1)
     ref3 = plain.rms_norm((h1 + delta.float())[rows.long()].double().cpu(), w.double().cpu(), eps)
@@ -241,11 +243,12 @@ def test_linear_vector_of_the_reference(k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_swiglu(k, dtype):
-    gu = rnd(9, 2 * 211, dtype=dtype, scale=3.0)
-    out = torch.empty(9, 211, dtype=dtype, device=DEV)
+@pytest.mark.parametrize("inter", [211, 216, 4864])
+def test_swiglu(k, dtype, inter):
+    gu = rnd(9, 2 * inter, dtype=dtype, scale=3.0)
+    out = torch.empty(9, inter, dtype=dtype, device=DEV)
     k.swiglu(gu, out)
-    g, u = gu[:, :211].double().cpu(), gu[:, 211:].double().cpu()
+    g, u = gu[:, :inter].double().cpu(), gu[:, inter:].double().cpu()
     ref = u * g / (1 + torch.exp(-g))
     assert float((out.double().cpu() - ref).abs().max()) <= tol(dtype, float(ref.abs().max()))
     z = torch.zeros(2, 2 * 16, dtype=dtype, device=DEV)
@@ -256,12 +259,14 @@ def test_swiglu(k, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq,nkv,hd,rd,theta", [(6, 3, 48, 48, 1e4), (5, 1, 80, 80, 1e6), (4, 4, 32, 16, 5e5)])
-def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta):
-    t, ps, pages = 11, 4, 9
+@pytest.mark.parametrize("t", [11, 77])
+@pytest.mark.parametrize("nq,nkv,hd,rd,theta", [(6, 3, 48, 48, 1e4), (5, 1, 80, 80, 1e6), (4, 4, 32, 16, 5e5), (14, 2, 64, 64, 1e6)])
+def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta, t):
+    ps, pages = 4, 9 if t == 11 else 30
     qkv = rnd(t, (nq + 2 * nkv) * hd, dtype=dtype, seed=1)
     bias = rnd((nq + 2 * nkv) * hd, dtype=dtype, seed=2)
-    positions = torch.tensor([0, 1, 2, 3, 250, 251, 7, 8, 9, 4000, 31], dtype=torch.int32, device=DEV)
+    base_pos = [0, 1, 2, 3, 250, 251, 7, 8, 9, 4000, 31]
+    positions = torch.tensor((base_pos * 8)[:t], dtype=torch.int32, device=DEV)
     inv = torch.pow(torch.tensor(theta, dtype=torch.float32), -2.0 * torch.arange(rd // 2, dtype=torch.float32) / rd).to(DEV)
     perm = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(3))[:t]
     slots = perm.to(torch.int32).to(DEV)
