@@ -74,6 +74,17 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
             q[t][kd] = __builtin_bit_cast(bf16x8, v);
         }
     }
+    const float scale2 = scale * 1.4426950408889634f;   // scores are kept in units of log 2
+    // the smallest causal limit and the largest window start among the valid rows of each tile
+    int p_min[QT], lo_max[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        const int r_first = row_base + t * 16, r_last = min(rows, r_first + 16) - 1;
+        const bool any = r_first < rows;
+        p_min[t] = any ? kv - n + r_first / group_size : -1;
+        const int p_last = any ? kv - n + r_last / group_size : -1;
+        lo_max[t] = window > 0 ? max(0, p_last - window + 1) : 0;
+    }
     // key blocks (32 keys) this wave needs, and this split's share of them
     const int last_row = min(rows, row_base + 16 * QT) - 1;
     const int p_hi = kv - n + last_row / group_size;
@@ -141,8 +152,12 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
             if (kb >= my_end) break;
 #pragma unroll
             for (int t = 0; t < QT; ++t) {
+                // scores in units of log 2: s = (q . k) * scale * log2(e), so that exp is one v_exp_f32
                 float s[2][4];
                 float mx = -INFINITY;
+                // most blocks lie wholly below the diagonal (and inside the window) for every row of the tile:
+                // they need no masking
+                const bool all_visible = kb * 32 + 31 <= p_min[t] && kb * 32 >= lo_max[t];
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt) {
                     f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -150,26 +165,36 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
                     for (int kd = 0; kd < KD; ++kd)
                         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, k_cur[i][kt][kd]),
                                                                       q[t][kd], acc, 0, 0, 0);
+                    if (all_visible) {
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const int key = kb * 32 + kt * 16 + lg * 4 + v;
-                        const bool vis = key <= p_row[t] && key >= lo_row[t];
-                        s[kt][v] = vis ? acc[v] * scale : -INFINITY;
-                        mx = fmaxf(mx, s[kt][v]);
+                        for (int v = 0; v < 4; ++v) {
+                            s[kt][v] = acc[v] * scale2;
+                            mx = fmaxf(mx, s[kt][v]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const int key = kb * 32 + kt * 16 + lg * 4 + v;
+                            const bool vis = key <= p_row[t] && key >= lo_row[t];
+                            s[kt][v] = vis ? acc[v] * scale2 : -INFINITY;
+                            mx = fmaxf(mx, s[kt][v]);
+                        }
                     }
                 }
                 mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
                 const float m_new = fmaxf(m_run[t], mx);
-                const bool none = m_new == -INFINITY;             // no visible key yet for this row
-                const float alpha = none ? 1.f : __expf(m_run[t] - m_new);
+                // a row without any visible key so far keeps maximum -inf; subtracting a finite stand-in makes
+                // every exp below 0 without a special case (exp2(-inf) = 0)
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_use);
                 float sum = 0.f;
                 bf16x8 pb;
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        const float pv = none ? 0.f : __expf(s[kt][v] - m_new);
+                        const float pv = __builtin_amdgcn_exp2f(s[kt][v] - m_use);
                         sum += pv;
                         pb[kt * 4 + v] = static_cast<__bf16>(pv);
                     }
@@ -218,7 +243,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
 #pragma unroll
             for (int d = 0; d < DT; ++d) *reinterpret_cast<f32x4*>(pp + d * 16) = o[t][d];
             if (lg == 0) {
-                part_ml[prow * 2] = m_run[t];
+                part_ml[prow * 2] = m_run[t] * 0.6931471805599453f;      // back to natural units for the combine
                 part_ml[prow * 2 + 1] = l;
             }
         }

@@ -368,7 +368,7 @@ class HipKernels:
             self._run("egpt_paged_attention_mfma", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
                       self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
                       q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t, nq, nkv, hd, page_size,
-                      float(scale), int(window), n_splits, 16 if max_q_len == 1 else 32, 1 if combine else 0,
+                      float(scale), int(window), n_splits, 16, 1 if combine else 0,
                       self._stream())
             return (part_o, part_ml) if (n_splits > 1 and not combine) else None
         self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
