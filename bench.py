@@ -45,6 +45,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -99,7 +100,7 @@ def main() -> int:
 
     # ---------------------------------------------------------------- prefill of 2,048 tokens, one request, one step
     prefill = None
-    if not args.no_points:
+    if not args.no_points or args.prefill_only:
         ids = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
         times = []
         for rep in range(5):
@@ -114,6 +115,9 @@ def main() -> int:
         prefill = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
                    "frac": round(prefill_flops(PREFILL_TOKENS) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+    if args.prefill_only:
+        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen2.5-0.5B)", "prefill": prefill}), flush=True)
+        return 0
 
     # ---------------------------------------------------------------- decoding at each batch size
     def decode_run(batch: int, warmup: int, steps: int):

@@ -92,6 +92,7 @@ class Engine:
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe
         self._decode_plans: dict = {}
         self._graph_pool = None
+        self._has_windows = any(g.window is not None for g in groups)
 
     @classmethod
     def from_dir(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
@@ -228,13 +229,37 @@ class Engine:
         once per (batch size, block-table width) into a device graph and replayed with new metadata.  The
         launch of some two hundred kernels costs more host time than they run on the device; the graph
         removes that."""
-        rcs = self._check(entries)
-        self._reserve_all(rcs, entries)
+        # the checks of `_check`, for one token each, in one pass
+        requests = self.cache.requests
+        rcs, tokens, seen = [], [], set()
+        vocab, limit = self.vocab_size, self.max_position
+        for e in entries:
+            rc = requests.get(e.request_id)
+            if rc is None:
+                raise KeyError(f"request {e.request_id!r} is not live (add_request first)")
+            tok = int(e.tokens[0])
+            if not 0 <= tok < vocab:
+                raise IndexError(f"token id {tok} of request {e.request_id!r} is outside [0, {vocab})")
+            if e.want[0] != 0:
+                raise IndexError(f"wanted place {e.want[0]} of request {e.request_id!r} is outside its 1 tokens")
+            if rc.num_tokens >= limit:
+                raise ValueError(
+                    f"request {e.request_id!r} would reach {rc.num_tokens + 1} tokens, "
+                    f"max_position_embeddings is {limit}"
+                )
+            rcs.append(rc)
+            tokens.append(tok)
+            seen.add(e.request_id)
+        if len(seen) != len(entries):
+            raise ValueError("a request appears twice in one step")
         ps = self.page_size
+        # a token needs a new page only when it starts one (tables hold exactly the pages of the tokens so far)
+        starters = [i for i, rc in enumerate(rcs) if rc.num_tokens % ps == 0]
+        if starters:
+            self._reserve_all([rcs[i] for i in starters], [entries[i] for i in starters])
         b = len(rcs)
-        n_groups = len(self.cache.groups)
         widths = []
-        for g in range(n_groups):
+        for g in range(len(self.cache.groups)):
             need = max(len(rc.tables[g]) for rc in rcs)
             w = 4
             while w < need:
@@ -244,7 +269,7 @@ class Engine:
         plan = self._decode_plans.get(key)
         if plan is None:
             plan = self._decode_plans[key] = _DecodePlan(self, b, widths)
-        plan.fill(rcs, [e.tokens[0] for e in entries])
+        plan.fill(rcs, tokens)
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
             plan.runs += 1
@@ -253,8 +278,12 @@ class Engine:
         else:
             plan.graph.replay()
             logits = plan.logits
-        for rc in rcs:
-            self.cache.commit(rc, 1)
+        if self._has_windows:
+            for rc in rcs:
+                self.cache.commit(rc, 1)
+        else:
+            for rc in rcs:
+                rc.num_tokens += 1
         return logits
 
 
