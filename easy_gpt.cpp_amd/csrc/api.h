@@ -61,8 +61,9 @@ int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_split
                           float* out, int m, int n, int n_splits, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
+// weights: scratch for n_rows * vocab floats.
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
-                const float* uniform, int32_t* out, int n_rows, int vocab, void* stream);
+                const float* uniform, int32_t* out, float* weights, int n_rows, int vocab, void* stream);
 
 #ifdef __cplusplus
 }

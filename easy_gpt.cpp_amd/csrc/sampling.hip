@@ -3,14 +3,36 @@
 // The reference samples from probabilities on the host (/root/reference/src/sampler.cpp:39-105):
 // p^(1/T) (== softmax(logits / T) after normalisation), keep the k most likely, then the smallest
 // set of most likely tokens whose normalised mass reaches top_p, then one uniform draw over the
-// kept mass.  Here the kept set is found without sorting, by bisection on the weight threshold
-// (32 passes over the row, which stays in cache), and the draw walks the kept weights in index order.
+// kept mass.  Here the kept set is found without sorting, by radix selection on the bit patterns of the
+// weights (four passes of eight bits over the row, which stays in cache; masses are added in fixed point so
+// that no decision depends on the order of additions), and the draw walks the kept weights in index order.
 #include "api.h"
 #include "common.h"
 
 namespace egpt {
 
 constexpr int kSampleThreads = 1024;
+
+// Calls f(index, value) for every element of p[0..n) once, spread over the workgroup's threads (thread `tid` of
+// `n_threads`).  The body reads 16 bytes per thread and keeps four such loads in flight: a pass over a row is a
+// chain of dependent loads otherwise, and its time is their latency, not the row's size.
+template <typename F>
+__device__ __forceinline__ void for_each_in_row(const float* __restrict__ p, int n, int tid, int n_threads, F f) {
+    const int head = min(n, static_cast<int>((4u - ((reinterpret_cast<uintptr_t>(p) >> 2) & 3u)) & 3u));
+    for (int j = tid; j < head; j += n_threads) f(j, p[j]);
+    const float4* p4 = reinterpret_cast<const float4*>(p + head);
+    const int n4 = (n - head) / 4;
+#pragma unroll 4
+    for (int i = tid; i < n4; i += n_threads) {
+        const float4 v = p4[i];
+        const int j = head + 4 * i;
+        f(j, v.x);
+        f(j + 1, v.y);
+        f(j + 2, v.z);
+        f(j + 3, v.w);
+    }
+    for (int j = head + 4 * n4 + tid; j < n; j += n_threads) f(j, p[j]);
+}
 
 // lowest index among equal maxima (/root/reference/src/sampler.cpp:13-20: std::max_element)
 __device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int oi) {
@@ -23,13 +45,12 @@ __device__ __forceinline__ void argmax_combine(float& v, int& i, float ov, int o
 __device__ int block_argmax(const float* __restrict__ row, int vocab, float* s_val, int* s_idx) {
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
-        const float v = row[j];
-        if (v > best) {          // strictly greater keeps the lowest index of this thread's stride
+    for_each_in_row(row, vocab, threadIdx.x, blockDim.x, [&](int j, float v) {
+        if (v > best || (v == best && j < best_i)) {
             best = v;
             best_i = j;
         }
-    }
+    });
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, kWave);
@@ -99,17 +120,189 @@ __global__ __launch_bounds__(64) void argmax_pick_kernel(const float* __restrict
     if (lane == 0) out[r] = i;
 }
 
-// weight of token j: exp((x_j - max) / T), in (0, 1]
+// weight of token j: exp((x_j - max) / T), in [0, 1]
 __device__ __forceinline__ float weight_of(float x, float mx, float inv_t) { return expf((x - mx) * inv_t); }
 
+// Fixed-point image of a weight in [0, 1] (40 fractional bits): sums of these are integers, so a sum over the
+// row does not depend on the order in which threads add, and neither does any decision taken from it.
+__device__ __forceinline__ unsigned long long fixed_of(float w) {
+    return static_cast<unsigned long long>(static_cast<double>(w) * 1099511627776.0);
+}
+
+// The largest bit pattern tau with count(w >= tau) >= need (non-negative floats order like their bits): radix
+// selection, eight bits a level, histogram in LDS.  The weights of a row crowd into a few exponents, so the
+// lanes of a wavefront that hit the same bin first agree on one addition (a ballot and a population count).
+__device__ uint32_t select_by_count(const float* __restrict__ w, int vocab, unsigned int need, unsigned int* hist,
+                                    uint32_t* shared_prefix, unsigned int* shared_need) {
+    uint32_t prefix = 0u, mask = 0u;
+    const int lane = threadIdx.x % kWave;
+    int first_level = 3;
+    {
+        // The highest digit of a weight's pattern is its exponent (two exponents a bin), and the k-th largest
+        // weight is almost always within 2^-16 of the largest (1.0, digit 0x3f): count those eight bins in
+        // registers.  If the k-th weight is smaller still, the general histogram below takes over.
+        unsigned int c[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+        for_each_in_row(w, vocab, threadIdx.x, blockDim.x, [&](int, float wj) {
+            const uint32_t bits = __float_as_uint(wj);
+            if (bits >= 0x38000000u) {
+                const uint32_t d = 0x3fu - (bits >> 24);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) c[i] += d == static_cast<uint32_t>(i) ? 1u : 0u;
+            }
+        });
+        for (int i = threadIdx.x; i < 8; i += blockDim.x) hist[i] = 0u;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            unsigned int v = c[i];
+#pragma unroll
+            for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+            if (lane == 0 && v) atomicAdd(&hist[i], v);          // integer sums: order does not matter
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned int cum = 0u;
+            int found = -1;
+            for (int i = 0; i < 8; ++i) {
+                if (cum + hist[i] >= need) {
+                    found = i;
+                    break;
+                }
+                cum += hist[i];
+            }
+            *shared_prefix = found >= 0 ? (0x3fu - found) << 24 : 0xffffffffu;
+            *shared_need = found >= 0 ? need - cum : need;
+        }
+        __syncthreads();
+        if (*shared_prefix != 0xffffffffu) {
+            prefix = *shared_prefix;
+            need = *shared_need;
+            mask = 255u << 24;
+            first_level = 2;
+        }
+        __syncthreads();
+    }
+    for (int level = first_level; level >= 0; --level) {
+        const int shift = 8 * level;
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0u;
+        __syncthreads();
+        for_each_in_row(w, vocab, threadIdx.x, blockDim.x, [&](int, float wj) {
+            const uint32_t bits = __float_as_uint(wj);
+            const uint32_t bin = (bits & mask) == prefix ? (bits >> shift) & 255u : 0xffffffffu;
+            unsigned long long todo = __ballot(bin != 0xffffffffu);      // over the lanes that are here
+            while (todo) {
+                const int leader = __ffsll(static_cast<long long>(todo)) - 1;
+                const uint32_t b0 = __shfl(bin, leader, kWave);
+                const unsigned long long same = __ballot(bin == b0);
+                if (lane == leader) atomicAdd(&hist[b0], static_cast<unsigned int>(__popcll(same)));
+                todo &= ~same;
+            }
+        });
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned int cum = 0u;
+            int bin = 255;
+            for (; bin > 0; --bin) {
+                if (cum + hist[bin] >= need) break;
+                cum += hist[bin];
+            }
+            *shared_prefix = prefix | (static_cast<uint32_t>(bin) << shift);
+            *shared_need = need - cum;
+        }
+        __syncthreads();
+        prefix = *shared_prefix;
+        need = *shared_need;
+        mask |= 255u << shift;
+        __syncthreads();
+    }
+    return prefix;
+}
+
+// Among the weights >= floor_bits, the largest bit pattern tau with mass(w >= tau) >= need: the smallest set of
+// most likely tokens whose mass reaches need, ties at tau included whole.  Sixteen-way search on the bit
+// pattern: each pass sums, per thread and then over the workgroup in a fixed order, the fixed-point mass at or
+// above fifteen pivots; about eight passes.
+__device__ uint32_t select_by_mass(const float* __restrict__ w, int vocab, uint32_t floor_bits, unsigned long long need,
+                                   unsigned long long* wave_sums /* [16][15] */, uint32_t* shared_lo,
+                                   uint32_t* shared_hi, unsigned long long* shared_above) {
+    uint32_t lo = floor_bits, hi = 0x3f800001u;      // mass(w >= lo) >= need, mass(w >= hi) < need
+    unsigned long long above = 0ull;                 // mass(w >= hi), known from the pass that set hi
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
+    while (hi - lo > 1u) {
+        // the first pass puts its pivots on exponent boundaries near 1.0, where the mass is; later passes
+        // divide [lo, hi) evenly
+        const bool first = hi == 0x3f800001u && lo < 0x38000000u;
+        const uint32_t step = first ? 0x01000000u : (hi - lo + 15u) / 16u;
+        const uint32_t base = first ? 0x37000000u : lo;               // pivot i = base + (i + 1) * step
+        unsigned long long acc[15];
+#pragma unroll
+        for (int i = 0; i < 15; ++i) acc[i] = 0ull;
+        for_each_in_row(w, vocab, threadIdx.x, blockDim.x, [&](int, float wj) {
+            const uint32_t bits = __float_as_uint(wj);
+            if (bits > base && bits < hi && bits >= floor_bits) {     // only these can lie at or above a pivot
+                const unsigned long long f = fixed_of(wj);
+#pragma unroll
+                for (int i = 0; i < 15; ++i) acc[i] += bits >= base + (i + 1) * step ? f : 0ull;
+            }
+        });
+#pragma unroll
+        for (int i = 0; i < 15; ++i) {
+            unsigned long long v = acc[i];
+#pragma unroll
+            for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+            if (lane == 0) wave_sums[wave * 15 + i] = v;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint32_t new_lo = lo, new_hi = hi;
+            unsigned long long new_above = above;
+            for (int i = 0; i < 15; ++i) {
+                const uint32_t pivot = base + (i + 1) * step;
+                if (pivot >= hi) break;
+                if (pivot <= lo) continue;
+                unsigned long long mass = above;
+                for (int wv = 0; wv < n_waves; ++wv) mass += wave_sums[wv * 15 + i];
+                if (mass >= need) {
+                    new_lo = pivot;
+                } else {
+                    new_hi = pivot;
+                    new_above = mass;
+                    break;
+                }
+            }
+            *shared_lo = new_lo;
+            *shared_hi = new_hi;
+            *shared_above = new_above;
+        }
+        __syncthreads();
+        lo = *shared_lo;
+        hi = *shared_hi;
+        above = *shared_above;
+        __syncthreads();
+    }
+    return lo;
+}
+
+// One workgroup per row.  `weights` is scratch [rows][vocab] float32: the weights are computed once and the
+// selection passes read them back (from cache).
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
-    const float* __restrict__ top_p, const float* __restrict__ uniform, int32_t* __restrict__ out, int vocab) {
+    const float* __restrict__ top_p, const float* __restrict__ uniform, int32_t* __restrict__ out,
+    float* __restrict__ weights, int vocab) {
     __shared__ float s_val[16];
     __shared__ int s_idx[16];
-    __shared__ float s_scan[kSampleThreads];
+    __shared__ unsigned int hist[256];
+    __shared__ unsigned long long s_wave[16 * 15];
+    __shared__ unsigned int s_need;
+    __shared__ uint32_t s_a, s_b;
+    __shared__ unsigned long long s_above;
+    __shared__ float s_piece[16];
+    __shared__ int s_owner;
+    __shared__ float s_before;
     const int r = blockIdx.x;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
     const float* row = logits + static_cast<size_t>(r) * vocab;
+    float* w = weights + static_cast<size_t>(r) * vocab;
     const float temp = temperature[r];
     const int best = block_argmax(row, vocab, s_val, s_idx);
     if (!(temp > 0.f)) {  // greedy, as the reference for temperature <= 0 (sampler.cpp:46-49)
@@ -118,87 +311,86 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     }
     const float mx = row[best];
     const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+    for_each_in_row(row, vocab, threadIdx.x, blockDim.x, [&](int j, float x) { w[j] = weight_of(x, mx, inv_t); });
+    __syncthreads();   // each thread reads back what others wrote: same workgroup, so a barrier suffices
     // kept set = { j : w_j >= threshold }; the threshold starts at 0 (everything)
-    float threshold = 0.f;
+    uint32_t threshold = 0u;
     const int k = top_k[r];
-    if (k > 0 && k < vocab) {
-        // largest bit pattern tau with count(w >= tau) >= k; positive floats order like their bits
-        uint32_t lo = 0u, hi = 0x3f800000u;  // w in (0, 1]
-        while (lo < hi) {
-            const uint32_t mid = lo + (hi - lo + 1) / 2;
-            const float tau = __uint_as_float(mid);
-            float cnt = 0.f;
-            for (int j = threadIdx.x; j < vocab; j += blockDim.x) cnt += weight_of(row[j], mx, inv_t) >= tau ? 1.f : 0.f;
-            cnt = block_sum(cnt, s_val);
-            if (cnt >= static_cast<float>(k)) lo = mid; else hi = mid - 1;
-        }
-        threshold = __uint_as_float(lo);
-    }
-    float kept = 0.f;
-    for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
-        const float w = weight_of(row[j], mx, inv_t);
-        kept += w >= threshold ? w : 0.f;
-    }
-    kept = block_sum(kept, s_val);
+    if (k > 0 && k < vocab) threshold = select_by_count(w, vocab, static_cast<unsigned int>(k), hist, &s_a, &s_need);
     const float p = top_p[r];
     if (p > 0.f && p < 1.f) {
-        // largest tau with mass(w >= tau) >= p * kept: the smallest set of most likely tokens reaching p
-        uint32_t lo = __float_as_uint(threshold), hi = 0x3f800000u;
-        const float need = p * kept;
-        while (lo < hi) {
-            const uint32_t mid = lo + (hi - lo + 1) / 2;
-            const float tau = __uint_as_float(mid);
-            float mass = 0.f;
-            for (int j = threadIdx.x; j < vocab; j += blockDim.x) {
-                const float w = weight_of(row[j], mx, inv_t);
-                mass += w >= tau ? w : 0.f;
-            }
-            mass = block_sum(mass, s_val);
-            if (mass >= need) lo = mid; else hi = mid - 1;
-        }
-        threshold = fmaxf(threshold, __uint_as_float(lo));
+        // mass of what top-k kept, in fixed point: per-thread sums, then over the wavefronts in order
+        unsigned long long mine = 0ull;
+        for_each_in_row(w, vocab, threadIdx.x, blockDim.x, [&](int, float wj) {
+            if (__float_as_uint(wj) >= threshold) mine += fixed_of(wj);
+        });
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, kWave);
+        if (lane == 0) s_wave[wave] = mine;
+        __syncthreads();
+        unsigned long long kept = 0ull;
+        for (int i = 0; i < n_waves; ++i) kept += s_wave[i];
+        __syncthreads();
+        unsigned long long need = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(kept));
+        if (need == 0ull) need = 1ull;
+        threshold = select_by_mass(w, vocab, threshold, need, s_wave, &s_a, &s_b, &s_above);
     }
-    // inverse CDF in index order: every thread owns a contiguous piece of the row
-    const int chunk = (vocab + blockDim.x - 1) / blockDim.x;
-    const int begin = min(vocab, static_cast<int>(threadIdx.x) * chunk), end = min(vocab, begin + chunk);
+    // inverse CDF in index order.  Every wavefront owns a contiguous piece of the row; the piece that holds the
+    // drawn point is then walked 64 tokens at a time with a prefix sum over the lanes.
+    const int piece = ((vocab + n_waves - 1) / n_waves + kWave - 1) / kWave * kWave;
+    const int p_begin = min(vocab, wave * piece), p_end = min(vocab, p_begin + piece);
     float mine = 0.f;
-    for (int j = begin; j < end; ++j) {
-        const float w = weight_of(row[j], mx, inv_t);
-        mine += w >= threshold ? w : 0.f;
-    }
-    s_scan[threadIdx.x] = mine;
+    for_each_in_row(w + p_begin, p_end - p_begin, lane, kWave, [&](int, float wj) {
+        mine += __float_as_uint(wj) >= threshold ? wj : 0.f;
+    });
+    mine = wave_sum(mine);
+    if (lane == 0) s_piece[wave] = mine;
     __syncthreads();
     if (threadIdx.x == 0) {
         float total = 0.f;
-        for (int i = 0; i < blockDim.x; ++i) total += s_scan[i];
-        float u = uniform[r];
-        u = fminf(fmaxf(u, 0.f), 0.99999994f);
+        for (int i = 0; i < n_waves; ++i) total += s_piece[i];
+        const float u = fminf(fmaxf(uniform[r], 0.f), 0.99999994f);
         const float target = u * total;
         float cum = 0.f;
         int owner = -1;
-        for (int i = 0; i < blockDim.x; ++i) {
-            if (s_scan[i] > 0.f) {
-                owner = i;                      // last piece with mass catches rounding at the end
-                if (cum + s_scan[i] > target) break;
+        float before = 0.f;
+        for (int i = 0; i < n_waves; ++i) {
+            if (s_piece[i] > 0.f) {
+                owner = i;                      // the last piece with mass catches rounding at the end
+                before = cum;
+                if (cum + s_piece[i] > target) break;
             }
-            cum += s_scan[i];
+            cum += s_piece[i];
         }
-        int pick = best;
-        if (owner >= 0) {
-            // cum must be the mass before `owner`
-            cum = 0.f;
-            for (int i = 0; i < owner; ++i) cum += s_scan[i];
-            const int b0 = min(vocab, owner * chunk), e0 = min(vocab, b0 + chunk);
-            for (int j = b0; j < e0; ++j) {
-                const float w = weight_of(row[j], mx, inv_t);
-                if (w >= threshold) {
-                    pick = j;
-                    cum += w;
-                    if (cum > target) break;
-                }
+        s_owner = owner;
+        s_before = target - before;             // what is left of the target inside the owner's piece
+        if (owner < 0) out[r] = best;
+    }
+    __syncthreads();
+    if (wave == s_owner) {
+        const float target = s_before;
+        float cum = 0.f;
+        int pick = -1, last_kept = -1;
+        for (int base = p_begin; base < p_end && pick < 0; base += kWave) {
+            const int j = base + lane;
+            float wj = 0.f;
+            if (j < p_end) {
+                const float v = w[j];
+                wj = __float_as_uint(v) >= threshold ? v : 0.f;
             }
+            float incl = wj;                     // inclusive prefix sum over the lanes
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const float up = __shfl_up(incl, o, kWave);
+                if (lane >= o) incl += up;
+            }
+            const unsigned long long kept_mask = __ballot(wj > 0.f);
+            const unsigned long long hit = __ballot(wj > 0.f && cum + incl > target);
+            if (kept_mask) last_kept = base + 63 - __clzll(static_cast<long long>(kept_mask));
+            if (hit) pick = base + __ffsll(static_cast<long long>(hit)) - 1;
+            cum += __shfl(incl, kWave - 1, kWave);
         }
-        out[r] = pick;
+        if (lane == 0) out[r] = pick >= 0 ? pick : (last_kept >= 0 ? last_kept : best);
     }
 }
 
@@ -224,13 +416,14 @@ extern "C" int egpt_argmax(const float* logits, int32_t* out, void* scratch, int
     return EGPT_OK;
 }
 
+// weights: scratch for n_rows * vocab floats.
 extern "C" int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
-                           const float* uniform, int32_t* out, int n_rows, int vocab, void* stream) {
-    if (!logits || !temperature || !top_k || !top_p || !uniform || !out || n_rows < 0 || vocab <= 0)
+                           const float* uniform, int32_t* out, float* weights, int n_rows, int vocab, void* stream) {
+    if (!logits || !temperature || !top_k || !top_p || !uniform || !out || !weights || n_rows < 0 || vocab <= 0)
         return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
     sample_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, top_k,
-                                                                                   top_p, uniform, out, vocab);
+                                                                                   top_p, uniform, out, weights, vocab);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

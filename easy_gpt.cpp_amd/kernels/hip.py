@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 4:
+    if lib.egpt_abi_version() != 5:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -57,7 +57,7 @@ class HipKernels:
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
-            "egpt_sample": [vp, vp, vp, vp, vp, vp, i, i, vp],
+            "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
         }
         for name, argtypes in sigs.items():
             fn = getattr(lib, name)
@@ -397,5 +397,6 @@ class HipKernels:
         self._need(top_p, "top_p", _F32, (r,))
         self._need(uniform, "uniform", _F32, (r,))
         self._need(out, "out", _I32, (r,))
+        weights = torch.empty((r, v), dtype=_F32, device=logits.device)
         self._run("egpt_sample", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
-                  uniform.data_ptr(), out.data_ptr(), r, v, self._stream())
+                  uniform.data_ptr(), out.data_ptr(), weights.data_ptr(), r, v, self._stream())
