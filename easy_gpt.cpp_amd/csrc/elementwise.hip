@@ -75,9 +75,23 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
     }
 }
 
+// eight consecutive values, stored as bfloat16 (one 16-byte load) or float32 (two), as floats
+__device__ __forceinline__ void load8_as_float(const bf16_t* p, float* v) {
+    const uint4 d = *reinterpret_cast<const uint4*>(p);
+    v[0] = __uint_as_float(d.x << 16); v[1] = __uint_as_float(d.x & 0xffff0000u);
+    v[2] = __uint_as_float(d.y << 16); v[3] = __uint_as_float(d.y & 0xffff0000u);
+    v[4] = __uint_as_float(d.z << 16); v[5] = __uint_as_float(d.z & 0xffff0000u);
+    v[6] = __uint_as_float(d.w << 16); v[7] = __uint_as_float(d.w & 0xffff0000u);
+}
+__device__ __forceinline__ void load8_as_float(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 // The same for bfloat16 activations with eight features per thread and load (16-byte loads of the
 // activations, 32 bytes of the residual stream): the form that prompt portions of many tokens take.
-__global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict__ h, const bf16_t* __restrict__ delta,
+template <typename DT>   // delta as bfloat16, or as float32 (a product that was written out in float32)
+__global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict__ h, const DT* __restrict__ delta,
                                                                const int32_t* __restrict__ rows,
                                                                const bf16_t* __restrict__ weight, float eps,
                                                                bf16_t* __restrict__ out, int hidden) {
@@ -85,46 +99,43 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
     const int r = blockIdx.x;
     const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
     float* hrow = h + src * hidden;
-    const bf16_t* drow = delta ? delta + src * hidden : nullptr;
+    const DT* drow = delta ? delta + src * hidden : nullptr;
     const bool write_back = (rows == nullptr) && (delta != nullptr);
     float ss = 0.f;
     for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
-        float4 a = *reinterpret_cast<const float4*>(hrow + j), b = *reinterpret_cast<const float4*>(hrow + j + 4);
+        float v[8];
+        load8_as_float(hrow + j, v);
         if (drow) {
-            const uint4 d = *reinterpret_cast<const uint4*>(drow + j);
-            a.x += __uint_as_float(d.x << 16); a.y += __uint_as_float(d.x & 0xffff0000u);
-            a.z += __uint_as_float(d.y << 16); a.w += __uint_as_float(d.y & 0xffff0000u);
-            b.x += __uint_as_float(d.z << 16); b.y += __uint_as_float(d.z & 0xffff0000u);
-            b.z += __uint_as_float(d.w << 16); b.w += __uint_as_float(d.w & 0xffff0000u);
+            float d[8];
+            load8_as_float(drow + j, d);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += d[i];
             if (write_back) {
-                *reinterpret_cast<float4*>(hrow + j) = a;
-                *reinterpret_cast<float4*>(hrow + j + 4) = b;
+                *reinterpret_cast<float4*>(hrow + j) = float4{v[0], v[1], v[2], v[3]};
+                *reinterpret_cast<float4*>(hrow + j + 4) = float4{v[4], v[5], v[6], v[7]};
             }
         }
-        ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
     bf16_t* orow = out + static_cast<size_t>(r) * hidden;
     for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
-        float4 a = *reinterpret_cast<const float4*>(hrow + j), b = *reinterpret_cast<const float4*>(hrow + j + 4);
+        float v[8], w[8];
+        load8_as_float(hrow + j, v);
         if (drow && !write_back) {
-            const uint4 d = *reinterpret_cast<const uint4*>(drow + j);
-            a.x += __uint_as_float(d.x << 16); a.y += __uint_as_float(d.x & 0xffff0000u);
-            a.z += __uint_as_float(d.y << 16); a.w += __uint_as_float(d.y & 0xffff0000u);
-            b.x += __uint_as_float(d.z << 16); b.y += __uint_as_float(d.z & 0xffff0000u);
-            b.z += __uint_as_float(d.w << 16); b.w += __uint_as_float(d.w & 0xffff0000u);
+            float d[8];
+            load8_as_float(drow + j, d);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] += d[i];
         }
-        const uint4 w = *reinterpret_cast<const uint4*>(weight + j);
-        const float v[8] = {a.x * inv * __uint_as_float(w.x << 16), a.y * inv * __uint_as_float(w.x & 0xffff0000u),
-                            a.z * inv * __uint_as_float(w.y << 16), a.w * inv * __uint_as_float(w.y & 0xffff0000u),
-                            b.x * inv * __uint_as_float(w.z << 16), b.y * inv * __uint_as_float(w.z & 0xffff0000u),
-                            b.z * inv * __uint_as_float(w.w << 16), b.w * inv * __uint_as_float(w.w & 0xffff0000u)};
+        load8_as_float(weight + j, w);
         uint4 o;
-        o.x = f32_to_bf16_bits(v[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1])) << 16);
-        o.y = f32_to_bf16_bits(v[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3])) << 16);
-        o.z = f32_to_bf16_bits(v[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5])) << 16);
-        o.w = f32_to_bf16_bits(v[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7])) << 16);
+        o.x = f32_to_bf16_bits(v[0] * inv * w[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1] * inv * w[1])) << 16);
+        o.y = f32_to_bf16_bits(v[2] * inv * w[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3] * inv * w[3])) << 16);
+        o.z = f32_to_bf16_bits(v[4] * inv * w[4]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[5] * inv * w[5])) << 16);
+        o.w = f32_to_bf16_bits(v[6] * inv * w[6]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[7] * inv * w[7])) << 16);
         *reinterpret_cast<uint4*>(orow + j) = o;
     }
 }
@@ -144,22 +155,22 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
 }
 
 // bfloat16, eight features per thread (inter % 8 == 0, one tensor, no partial sums)
-__global__ __launch_bounds__(256) void swiglu_vec8_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out,
+template <typename GT>
+__global__ __launch_bounds__(256) void swiglu_vec8_kernel(const GT* __restrict__ gate_up, bf16_t* __restrict__ out,
                                                           int n_tokens, int inter) {
     const size_t chunks_per_row = inter / 8;
     const size_t total = static_cast<size_t>(n_tokens) * chunks_per_row;
     for (size_t c = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; c < total;
          c += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const size_t t = c / chunks_per_row, j = (c % chunks_per_row) * 8;
-        const uint4 g = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + j);
-        const uint4 u = *reinterpret_cast<const uint4*>(gate_up + t * 2 * inter + inter + j);
-        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+        float g[8], u[8];
+        load8_as_float(gate_up + t * 2 * inter + j, g);
+        load8_as_float(gate_up + t * 2 * inter + inter + j, u);
         uint32_t ow[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
-            const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
-            const float r0 = u0 * (g0 / (1.0f + expf(-g0))), r1 = u1 * (g1 / (1.0f + expf(-g1)));
+            const float r0 = u[2 * i] * (g[2 * i] / (1.0f + expf(-g[2 * i])));
+            const float r1 = u[2 * i + 1] * (g[2 * i + 1] / (1.0f + expf(-g[2 * i + 1])));
             ow[i] = f32_to_bf16_bits(r0) | (static_cast<uint32_t>(f32_to_bf16_bits(r1)) << 16);
         }
         *reinterpret_cast<uint4*>(out + t * inter + j) = uint4{ow[0], ow[1], ow[2], ow[3]};
@@ -237,8 +248,8 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __rest
 // The same for many tokens (prompt portions), full rotation (rotary_dim == hd), one tensor in and out: a
 // thread owns one (token, pair index) and walks the heads, so the angle's sine and cosine are computed once
 // for all heads instead of once per head.
-template <typename T>
-__global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const T* __restrict__ qkv_in, T* __restrict__ qkv_out,
+template <typename T, typename IN>
+__global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const IN* __restrict__ qkv_in, T* __restrict__ qkv_out,
                                                                   const T* __restrict__ bias,
                                                                   const int32_t* __restrict__ positions,
                                                                   const float* __restrict__ inv_freq,
@@ -322,10 +333,16 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, i
     // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for
     const int threads = (delta_splits > 1 || hidden >= 4096) ? 1024 : (hidden >= 2048 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
-    if (dtype == 1 && delta_splits == 0 && hidden % 8 == 0 && n_rows >= 32) {
-        add_rmsnorm_vec8_kernel<<<n_rows, hidden >= 2048 ? 256 : 128, 0, s>>>(
-            h, static_cast<const bf16_t*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
-            static_cast<bf16_t*>(out), hidden);
+    if (dtype == 1 && delta_splits <= 1 && hidden % 8 == 0 && n_rows >= 32) {
+        const int threads = hidden >= 2048 ? 256 : 128;
+        if (delta_splits == 0)
+            add_rmsnorm_vec8_kernel<bf16_t><<<n_rows, threads, 0, s>>>(
+                h, static_cast<const bf16_t*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
+                static_cast<bf16_t*>(out), hidden);
+        else   // one float32 "partial sum": a product written out in float32
+            add_rmsnorm_vec8_kernel<float><<<n_rows, threads, 0, s>>>(
+                h, static_cast<const float*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
+                static_cast<bf16_t*>(out), hidden);
         EGPT_CHECK_LAUNCH();
         return EGPT_OK;
     }
@@ -351,11 +368,15 @@ extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_t
     const size_t total = static_cast<size_t>(n_tokens) * inter;
     const int blocks = static_cast<int>(total / 256 + 1 > 8192 ? 8192 : total / 256 + 1);
     const size_t stride = total * 2;
-    if (dtype == 1 && n_splits == 0 && inter % 8 == 0) {
+    if (dtype == 1 && n_splits <= 1 && inter % 8 == 0) {
         const size_t chunks = total / 8;
         const int vblocks = static_cast<int>(chunks / 256 + 1 > 16384 ? 16384 : chunks / 256 + 1);
-        swiglu_vec8_kernel<<<vblocks, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
-                                                   n_tokens, inter);
+        if (n_splits == 0)
+            swiglu_vec8_kernel<bf16_t><<<vblocks, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up),
+                                                               static_cast<bf16_t*>(out), n_tokens, inter);
+        else
+            swiglu_vec8_kernel<float><<<vblocks, 256, 0, s>>>(static_cast<const float*>(gate_up),
+                                                              static_cast<bf16_t*>(out), n_tokens, inter);
         EGPT_CHECK_LAUNCH();
         return EGPT_OK;
     }
@@ -387,25 +408,23 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
     const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
-    if (dtype == 1 && n_splits == 0 && !row_ss && rotary_dim == hd && n_tokens >= 64 && hd <= 512) {
+    if (dtype == 1 && n_splits <= 1 && !row_ss && rotary_dim == hd && n_tokens >= 64 && hd <= 512) {
         // many tokens: one thread per (token, pair), the angle shared by all heads.  (bfloat16 only: the
         // float32 path keeps one kernel per operation whatever the batch, so that its results do not depend
-        // on the batch in any bit.)
+        // on the batch in any bit.)  The input is bfloat16, or one float32 "partial sum".
         const int half = hd / 2;
         const int tpb = 256 / half > 0 ? 256 / half : 1;
         const int blocks = (n_tokens + tpb - 1) / tpb;
-        if (dtype == 0)
-            qkv_rope_store_rows_kernel<float><<<blocks, 256, 0, s>>>(
-                static_cast<const float*>(qkv_in), static_cast<float*>(qkv_out), static_cast<const float*>(bias),
-                positions, inv_freq, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), n_tokens, nq,
-                nkv, hd, page_size);
-        else if (dtype == 1)
-            qkv_rope_store_rows_kernel<bf16_t><<<blocks, 256, 0, s>>>(
+        if (n_splits == 0)
+            qkv_rope_store_rows_kernel<bf16_t, bf16_t><<<blocks, 256, 0, s>>>(
                 static_cast<const bf16_t*>(qkv_in), static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias),
                 positions, inv_freq, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens,
                 nq, nkv, hd, page_size);
         else
-            return EGPT_BAD_ARGUMENT;
+            qkv_rope_store_rows_kernel<bf16_t, float><<<blocks, 256, 0, s>>>(
+                static_cast<const float*>(qkv_in), static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias),
+                positions, inv_freq, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens,
+                nq, nkv, hd, page_size);
         EGPT_CHECK_LAUNCH();
         return EGPT_OK;
     }

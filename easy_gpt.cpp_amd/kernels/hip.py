@@ -270,9 +270,12 @@ class HipKernels:
         self._run("egpt_attention_combine", part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), t * nq, hd,
                   int(a_splits), self._stream())
 
-    def product(self, x, w):
+    def product(self, x, w, unrounded=False):
         """x w^T for a consumer that takes partial sums: returns act [m, n], or float32 [splits, m, n] whose sum
-        over splits is the product (few rows in bfloat16: the k range is split over workgroups)."""
+        over splits is the product (few rows in bfloat16: the k range is split over workgroups).  unrounded=True
+        asks for float32 also from the many-row library product (as [1, m, n]): for consumers that go on computing
+        with the values before they round, such as the bias and rotation of queries and keys, where a rounding
+        in between is the largest single contribution to the bfloat16 error of the logits."""
         m, k = x.shape
         n = w.shape[0]
         if x.dtype == _BF16 and 0 < m <= 64 and k % 8 == 0:
@@ -282,6 +285,14 @@ class HipKernels:
             out = torch.empty((s, m, n), dtype=_F32, device=x.device)
             self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s,
                       self._stream())
+            return out
+        if unrounded and x.dtype == _BF16 and m > 64 and k % 8 == 0:
+            # many rows: the library's product (the reference uses cuBLAS for every linear layer), written out in
+            # float32; it goes on as a single "partial sum" [1, m, n]
+            self._need(x, "x")
+            self._need(w, "w", x.dtype, (n, k))
+            out = torch.empty((1, m, n), dtype=_F32, device=x.device)
+            torch.mm(x, w.t(), out_dtype=_F32, out=out[0])
             return out
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
         return self.linear(x, w, None, out)

@@ -113,7 +113,7 @@ class GQAttention(Mixer):
             else:
                 x = x.materialize()
         if prod is None:
-            prod = k.product(x, self.w_qkv)             # act [T, W], or float32 partial sums [S, T, W]
+            prod = k.product(x, self.w_qkv, unrounded=True)      # act [T, W], or float32 partial sums [S, T, W]
             dtype, device, t = x.dtype, x.device, x.shape[0]
         qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=dtype, device=device)
         slots = cache.slots if cache.writes else None

@@ -22,7 +22,7 @@ def _whole(t):
 class EmulatedKernels:
     name = "emulated"
 
-    def product(self, x, w):
+    def product(self, x, w, unrounded=False):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype)
         self.linear(x, w, None, out)
         return out

@@ -232,6 +232,51 @@ def test_output_projection_combines_attention_parts(k, nq, nkv, hd, batch, ctx):
     assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
 
 
+def test_consumers_take_a_float32_product_of_many_rows(k):
+    # many-row products are written out in float32 and handed on as one "partial sum" [1, T, N]
+    dtype = torch.bfloat16
+    t, hid = 70, 896
+    delta = rnd(1, t, hid, seed=1)
+    h = rnd(t, hid, seed=2, scale=2.0)
+    h0 = h.clone()
+    w = (1 + rnd(hid, seed=3, scale=0.1)).to(dtype)
+    out = torch.empty(t, hid, dtype=dtype, device=DEV)
+    k.add_rmsnorm(h, delta, w, 1e-6, out)
+    assert torch.equal(h, h0 + delta[0])
+    ref = plain.rms_norm((h0 + delta[0]).double().cpu(), w.double().cpu(), 1e-6)
+    assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    rows = torch.arange(t - 1, -1, -2, dtype=torch.int32, device=DEV)
+    out2 = torch.empty(rows.shape[0], hid, dtype=dtype, device=DEV)
+    k.rows_add_rmsnorm(h0.clone(), delta, rows, w, 1e-6, out2)
+    assert float((out2.double().cpu() - ref[rows.long().cpu()]).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    inter = 328
+    gu = rnd(1, t, 2 * inter, seed=4, scale=2.0)
+    act = torch.empty(t, inter, dtype=dtype, device=DEV)
+    k.swiglu(gu, act)
+    g, u = gu[0, :, :inter].double().cpu(), gu[0, :, inter:].double().cpu()
+    refa = u * g / (1 + torch.exp(-g))
+    assert float((act.double().cpu() - refa).abs().max()) <= 1.6e-2 * float(refa.abs().max())
+    nq, nkv, hd, ps = 6, 2, 64, 16
+    width = (nq + 2 * nkv) * hd
+    qp = rnd(1, t, width, seed=5)
+    bias = rnd(width, dtype=dtype, seed=6)
+    positions = torch.arange(100, 100 + t, dtype=torch.int32, device=DEV)
+    inv = plain.rope_inv_freq(hd, 1e6).to(DEV)
+    slots = torch.randperm(6 * ps, generator=torch.Generator().manual_seed(7))[:t].to(torch.int32).to(DEV)
+    kc = torch.zeros(6, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros(6, nkv, hd, ps, dtype=dtype, device=DEV)
+    got = torch.empty(t, width, dtype=dtype, device=DEV)
+    k.qkv_rope_store(qp, bias, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=got)
+    x = (qp[0].double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
+    refq = x.clone()
+    refq[:, : nq + nkv] = plain.rope(x[:, : nq + nkv], positions.cpu(), 1e6)
+    assert float((got.double().cpu().view(t, -1, hd) - refq).abs().max()) <= 1.6e-2 * float(refq.abs().max())
+    for i in (0, 33, 69):
+        pg, off = int(slots[i]) // ps, int(slots[i]) % ps
+        assert torch.equal(kc[pg, :, off, :], got.view(t, -1, hd)[i, nq : nq + nkv])
+        assert torch.equal(vc[pg, :, :, off], got.view(t, -1, hd)[i, nq + nkv :])
+
+
 def test_linear_vector_of_the_reference(k):
     # /root/reference/test/matmul_3d_test.cpp:60-87
     x = torch.tensor([[1.0, 2, 3], [4, 5, 6]], device=DEV)
