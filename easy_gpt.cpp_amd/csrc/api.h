@@ -44,6 +44,12 @@ int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* 
                               const int32_t* q_start, const int32_t* q_len, const int32_t* kv_len, int n_seqs,
                               int n_tokens, int nq, int nkv, int hd, int page_size, float scale, int window,
                               int n_splits, int rows_per_wave, int combine, void* stream);
+// Prompt portions: the wavefronts of a workgroup share key/value tiles through LDS (n_splits == 1 semantics);
+// page sizes that are powers of two; shape = 10 * row tiles + key splits per workgroup (41, 42, 44, 22, 24).
+int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                               const int32_t* block_table, int table_width, const int32_t* q_start,
+                               const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
+                               int hd, int page_size, float scale, int window, int shape, void* stream);
 // One decoded token per request: workgroups of n_waves wavefronts per (request, kv head, key split).
 int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                                 const void* v_cache, const int32_t* block_table, int table_width,

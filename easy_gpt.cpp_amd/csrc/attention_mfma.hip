@@ -250,6 +250,263 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     }
 }
 
+// Prompt portions.  A workgroup takes RT tiles of 16 rows (of one request and kv head) and walks the keys in
+// tiles of 64 * KS, which are staged through LDS and shared by its RT * KS wavefronts; wavefront (rt, ks)
+// multiplies row tile rt with the ks-th 64 keys of each tile, and the KS partial results of a row tile are
+// combined through LDS at the end.  The next tile's loads are in flight while this one is computed.
+// Without the sharing every wavefront reads all of its keys from L2 itself (about 0.5 GB per layer for a
+// 2,048-token prompt at these sizes).  A wavefront issues a vector instruction in four cycles, and a prompt
+// of a few thousand tokens gives each SIMD only a few wavefronts, so what a tile costs is the vector
+// instructions and the waits between them rather than the matrix cores: hence 64 keys per softmax step, the
+// accumulator rescaled only when a row's maximum moved, and the split of the keys over wavefronts.
+// The arithmetic is that of attention_mfma_kernel.
+template <int HD, int RT, int KS>
+__global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
+    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window) {
+    constexpr int KD = HD / 32, DT = HD / 16;
+    constexpr int ROWS = 16 * RT;                // rows per workgroup
+    constexpr int KT = 64 * KS;                  // keys per LDS tile
+    constexpr int KROW = HD + 8, VROW = KT + 8;  // padded rows (bf16 elements)
+    constexpr int THREADS = 64 * RT * KS;
+    constexpr int CH = HD / (8 * RT);            // 16-byte chunks per thread and tile, of keys and of values
+    constexpr int STAGE = KT * KROW + HD * VROW;  // bf16 elements per stage
+    constexpr int COMBINE = (KS - 1) * RT * 64 * (DT * 4 + 2) * 2;    // the combination's floats, in bf16 elements
+    static_assert(CH >= 1 && HD % (8 * RT) == 0, "a thread takes whole chunks");
+    __shared__ __attribute__((aligned(16))) bf16_t smem[(2 * STAGE > COMBINE) ? 2 * STAGE : COMBINE];
+    auto ks_at = [&](int stage, int key, int col) -> bf16_t* { return smem + stage * STAGE + key * KROW + col; };
+    auto vs_at = [&](int stage, int d, int key) -> bf16_t* { return smem + stage * STAGE + KT * KROW + d * VROW + key; };
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int rt = wave % RT, ksi = wave / RT;
+    const int lj = lane % 16, lg = lane / 16;
+    const int kh = blockIdx.y;
+    const int group_size = nq / nkv;
+
+    int b = 0, grp = blockIdx.x;
+    for (; b < n_seqs; ++b) {
+        const int groups = (q_len[b] * group_size + ROWS - 1) / ROWS;
+        if (grp < groups) {
+            grp = groups - 1 - grp;          // the last rows first: they have the most keys to walk
+            break;
+        }
+        grp -= groups;
+    }
+    if (b >= n_seqs) return;
+    const int n = q_len[b], kv = kv_len[b], qs = q_start[b];
+    const int rows = n * group_size;
+    const int width = (nq + 2 * nkv) * HD;
+    const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+
+    // the workgroup's rows and the keys they need
+    const int blk_first = grp * ROWS, blk_last = min(rows, blk_first + ROWS) - 1;
+    const int blk_p_hi = kv - n + blk_last / group_size;
+    const int blk_first_pos = kv - n + blk_first / group_size;
+    const int blk_lo = window > 0 ? max(0, blk_first_pos - window + 1) : 0;
+    const int t_begin = blk_lo / KT, t_end = blk_p_hi / KT + 1;
+
+    // this wavefront's tile of 16 rows, this lane's row
+    const int row_base = blk_first + rt * 16;
+    const int r = row_base + lj;
+    const bool valid = r < rows;
+    const int i_tok = valid ? r / group_size : 0;
+    const int tok = qs + i_tok;
+    const int head = kh * group_size + (valid ? r % group_size : 0);
+    const int p_row = valid ? kv - n + i_tok : -1;
+    const int lo_row = (window > 0 && valid) ? max(0, p_row - window + 1) : 0;
+    const bool wave_any = row_base < rows;
+    const int w_last = min(rows, row_base + 16) - 1;
+    const int w_p_hi = wave_any ? kv - n + w_last / group_size : -1;       // largest causal limit in the tile
+    const int w_p_min = wave_any ? kv - n + row_base / group_size : -1;    // smallest
+    const int w_lo_first = (window > 0 && wave_any) ? max(0, w_p_min - window + 1) : 0;
+    const int w_lo_max = (window > 0 && wave_any) ? max(0, w_p_hi - window + 1) : 0;
+    bf16x8 q[KD];
+    {
+        const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+            q[kd] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    const float scale2 = scale * 1.4426950408889634f;
+
+    f32x4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;     // the maximum in units of the raw scores
+
+    // The loads of a tile go through three stages, each one iteration ahead of the next, so that no load
+    // waits for another inside an iteration: page numbers (tile + 2), keys and values into registers
+    // (tile + 1), registers into LDS after the products of this tile.  A thread's chunks of a tile lie in
+    // one page (keys: CH chunks of one key; values: eight keys of CH features), so a tile costs it two
+    // table entries and two addresses.
+    const int page_mask = page_size - 1;             // page sizes here are powers of two
+    const int k_row = tid / RT, k_col = (tid % RT) * CH * 8;                 // key within the tile, first feature
+    const int v_key = (tid % (KT / 8)) * 8, v_row = tid / (KT / 8);          // first of eight keys, feature (+ 8 RT u)
+    uint4 k_regs[CH], v_regs[CH];
+    int k_page, v_page;                              // -1: nothing to read (zeros)
+    auto lookup = [&](int tile) {
+        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
+        k_page = (kk <= blk_p_hi && kk >= blk_lo) ? table[kk >> page_shift] : -1;
+        v_page = (vk <= blk_p_hi && vk + 7 >= blk_lo) ? table[vk >> page_shift] : -1;
+    };
+    auto fetch = [&](int tile) {
+        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
+        if (k_page >= 0) {
+            const bf16_t* src = k_cache + ((static_cast<long>(k_page) * nkv + kh) * page_size + (kk & page_mask)) * HD + k_col;
+#pragma unroll
+            for (int u = 0; u < CH; ++u) k_regs[u] = *reinterpret_cast<const uint4*>(src + u * 8);
+        } else {
+#pragma unroll
+            for (int u = 0; u < CH; ++u) k_regs[u] = uint4{0u, 0u, 0u, 0u};
+        }
+        if (v_page >= 0) {
+            const bf16_t* src = v_cache + ((static_cast<long>(v_page) * nkv + kh) * HD + v_row) * page_size + (vk & page_mask);
+#pragma unroll
+            for (int u = 0; u < CH; ++u)
+                v_regs[u] = *reinterpret_cast<const uint4*>(src + static_cast<long>(u) * (8 * RT) * page_size);
+        } else {
+#pragma unroll
+            for (int u = 0; u < CH; ++u) v_regs[u] = uint4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto stash = [&](int stage) {
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            *reinterpret_cast<uint4*>(ks_at(stage, k_row, k_col + u * 8)) = k_regs[u];
+            *reinterpret_cast<uint4*>(vs_at(stage, v_row + u * 8 * RT, v_key)) = v_regs[u];
+        }
+    };
+
+    lookup(t_begin);
+    fetch(t_begin);
+    lookup(t_begin + 1);
+    stash(0);
+    __syncthreads();
+    for (int tile = t_begin; tile < t_end; ++tile) {
+        const int stage = (tile - t_begin) & 1;
+        fetch(tile + 1);           // past the last tile every page number is -1: nothing is read
+        lookup(tile + 2);
+        const int key0 = tile * KT + ksi * 64;       // this wavefront's 64 keys
+        if (wave_any && key0 <= w_p_hi && key0 + 63 >= w_lo_first) {     // else nothing visible to these rows
+            // S^T = K Q^T: lane (lj, lg) holds keys kt*16 + lg*4 + v of row lj
+            f32x4 acc[4];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                acc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    const uint4 kk = *reinterpret_cast<const uint4*>(ks_at(stage, ksi * 64 + kt * 16 + lj, kd * 32 + lg * 8));
+                    acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kk), q[kd], acc[kt], 0, 0, 0);
+                }
+            }
+            if (!(key0 + 63 <= w_p_min && key0 >= w_lo_max)) {           // on the diagonal or the window's edge
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = key0 + kt * 16 + lg * 4 + v;
+                        if (!(key <= p_row && key >= lo_row)) acc[kt][v] = -INFINITY;
+                    }
+            }
+            float mx = fmaxf(fmaxf(acc[0][0], acc[0][1]), fmaxf(acc[0][2], acc[0][3]));
+#pragma unroll
+            for (int kt = 1; kt < 4; ++kt) mx = fmaxf(mx, fmaxf(fmaxf(acc[kt][0], acc[kt][1]), fmaxf(acc[kt][2], acc[kt][3])));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            if (__any(m_new != m_run)) {             // some row's maximum moved: rescale what is accumulated
+                const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
+                l_run *= alpha;
+#pragma unroll
+                for (int d = 0; d < DT; ++d) {
+                    o[d][0] *= alpha; o[d][1] *= alpha; o[d][2] *= alpha; o[d][3] *= alpha;
+                }
+                m_run = m_new;
+            }
+            const float shift = -m_use * scale2;
+            float sum = 0.f;
+            bf16x8 pb[2];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float pv = __builtin_amdgcn_exp2f(fmaf(acc[kt][v], scale2, shift));
+                    sum += pv;
+                    pb[kt / 2][(kt % 2) * 4 + v] = static_cast<__bf16>(pv);
+                }
+            l_run += sum;
+            // O^T += V^T P^T, two products of 32 keys per 16 features
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    const uint2 v0 = *reinterpret_cast<const uint2*>(vs_at(stage, d * 16 + lj, ksi * 64 + kb * 32 + lg * 4));
+                    const uint2 v1 = *reinterpret_cast<const uint2*>(vs_at(stage, d * 16 + lj, ksi * 64 + kb * 32 + 16 + lg * 4));
+                    const uint4 a = uint4{v0.x, v0.y, v1.x, v1.y};
+                    o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[kb], o[d], 0, 0, 0);
+                }
+        }
+        stash(stage ^ 1);
+        __syncthreads();
+    }
+    float l = l_run;
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if constexpr (KS > 1) {
+        // The wavefronts of one row tile hold partial results over their keys: those with ks > 0 leave
+        // theirs in LDS (the tiles are no longer read: the loop ended with a barrier), ks == 0 adds them up.
+        constexpr int PER_LANE = DT * 4 + 2;
+        float* comb = reinterpret_cast<float*>(smem);
+        if (ksi > 0) {
+            float* dst = comb + (static_cast<size_t>((ksi - 1) * RT + rt) * PER_LANE) * 64 + lane;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) dst[(d * 4 + v) * 64] = o[d][v];
+            dst[(DT * 4) * 64] = m_run;
+            dst[(DT * 4 + 1) * 64] = l;
+        }
+        __syncthreads();
+        if (ksi > 0) return;
+        float m_all = m_run;
+#pragma unroll
+        for (int j = 0; j < KS - 1; ++j)
+            m_all = fmaxf(m_all, comb[(static_cast<size_t>(j * RT + rt) * PER_LANE + DT * 4) * 64 + lane]);
+        const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+        const float w0 = __builtin_amdgcn_exp2f((m_run - m_ref) * scale2);
+        l *= w0;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            o[d][0] *= w0; o[d][1] *= w0; o[d][2] *= w0; o[d][3] *= w0;
+        }
+#pragma unroll
+        for (int j = 0; j < KS - 1; ++j) {
+            const float* src = comb + (static_cast<size_t>(j * RT + rt) * PER_LANE) * 64 + lane;
+            const float wj = __builtin_amdgcn_exp2f((src[(DT * 4) * 64] - m_ref) * scale2);
+            l += src[(DT * 4 + 1) * 64] * wj;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) o[d][v] += src[(d * 4 + v) * 64] * wj;
+        }
+    }
+    if (valid) {
+        const float inv = 1.0f / l;
+        bf16_t* op = out + (static_cast<size_t>(tok) * nq + head) * HD + lg * 4;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            uint2 packed;
+            packed.x = f32_to_bf16_bits(o[d][0] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[d][1] * inv)) << 16);
+            packed.y = f32_to_bf16_bits(o[d][2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[d][3] * inv)) << 16);
+            *reinterpret_cast<uint2*>(op + d * 16) = packed;
+        }
+    }
+}
+
 // Decoded tokens only (one query token per request, its heads of one kv group in one 16-row tile): a
 // workgroup of NW wavefronts shares one (request, kv head, key split); each wavefront walks its share of
 // the keys, PF blocks of 32 keys per round with all of the round's loads in flight together (the kernel is
@@ -503,6 +760,63 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
 }  // namespace egpt
 
 using namespace egpt;
+
+// Prompt portions (and mixed batches) with keys and values shared through LDS by the wavefronts of a
+// workgroup.  Same operands and meaning as egpt_paged_attention_mfma with n_splits == 1; page sizes that are
+// powers of two.  `shape` = 10 * (tiles of 16 rows per workgroup) + (wavefronts that split a tile's keys).
+template <int HD, int RT, int KS>
+static void launch_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                         const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
+                         const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size,
+                         int page_shift, float scale, int window, hipStream_t s) {
+    const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (16 * RT) + n_seqs;   // upper bound
+    dim3 grid(static_cast<unsigned>(groups), nkv);
+    attention_tiled_kernel<HD, RT, KS><<<grid, 64 * RT * KS, 0, s>>>(
+        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
+        static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
+        page_size, page_shift, scale, window);
+}
+
+extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                                          const int32_t* block_table, int table_width, const int32_t* q_start,
+                                          const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens,
+                                          int nq, int nkv, int hd, int page_size, float scale, int window,
+                                          int shape, void* stream) {
+    if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
+        return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0)
+        return EGPT_BAD_ARGUMENT;
+    if ((hd != 64 && hd != 128) || page_size < 16 || (page_size & (page_size - 1)) != 0 || nkv > 65535)
+        return EGPT_UNSUPPORTED_SIZE;
+    if (n_tokens == 0) return EGPT_OK;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define EGPT_TILED(HD_, RT_, KS_)                                                                                  \
+    launch_tiled<HD_, RT_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,      \
+                                n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, s)
+    // shape = 10 * row tiles + key splits of a workgroup
+    if (hd == 64) {
+        switch (shape) {
+            case 41: EGPT_TILED(64, 4, 1); break;
+            case 42: EGPT_TILED(64, 4, 2); break;
+            case 44: EGPT_TILED(64, 4, 4); break;
+            case 22: EGPT_TILED(64, 2, 2); break;
+            case 24: EGPT_TILED(64, 2, 4); break;
+            default: return EGPT_BAD_ARGUMENT;
+        }
+    } else {
+        switch (shape) {
+            case 41: EGPT_TILED(128, 4, 1); break;
+            case 42: EGPT_TILED(128, 4, 2); break;
+            case 22: EGPT_TILED(128, 2, 2); break;
+            default: return EGPT_BAD_ARGUMENT;
+        }
+    }
+#undef EGPT_TILED
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
 
 // One decoded token per request (n_tokens == n_seqs, q_len all 1), nq / nkv <= 16: workgroups of n_waves
 // wavefronts (1..8) per (request, kv head, key split).  Same operands and meaning as egpt_paged_attention_mfma.

@@ -457,4 +457,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 5; }
+extern "C" int egpt_abi_version(void) { return 6; }

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 5:
+    if lib.egpt_abi_version() != 6:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -51,6 +51,7 @@ class HipKernels:
             "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, vp],
             "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
+            "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
@@ -369,9 +370,23 @@ class HipKernels:
                           q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale), int(window),
                           n_splits, 4, 1 if combine else 0, self._stream())
                 return (part_o, part_ml) if (n_splits > 1 and not combine) else None
-            n_splits = 1
-            if max_q_len == 1:
-                n_splits = max(1, min(1024 // (b * nkv), -(-max_kv_len // 64), 64))
+            if max_q_len > 1 and page_size & (page_size - 1) == 0:
+                # prompt portions (and mixed batches): key/value tiles shared through LDS by the wavefronts of
+                # a workgroup.  Few rows: small workgroups whose wavefronts split the keys, so that the GPU
+                # has enough of them; many rows: 64 rows per workgroup, which read the keys fewer times.
+                row_tiles = -(-t * (nq // nkv) // 16) * nkv
+                if row_tiles <= 1024:
+                    shape = 24 if hd == 64 else 22
+                elif row_tiles <= 2048:
+                    shape = 44 if hd == 64 else 42
+                else:
+                    shape = 42
+                self._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(),
+                          v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(),
+                          kv_len.data_ptr(), b, t, nq, nkv, hd, page_size, float(scale), int(window), shape,
+                          self._stream())
+                return None
+            n_splits = max(1, min(1024 // (b * nkv), -(-max_kv_len // 64), 64))
             part_o = part_ml = None
             if n_splits > 1:
                 part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)

@@ -376,7 +376,7 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
     return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
 
 
-def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0):
+def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None):
     kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed)
     t = sum(q for q, _ in seqs)
     g = torch.Generator().manual_seed(seed + 100)
@@ -386,8 +386,16 @@ def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0):
     kv_len = torch.tensor([kv for _, kv in seqs], dtype=torch.int32)
     out = torch.empty(t, nq * hd, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(hd)
-    k.paged_attention(qkv, out, kc, vc, table, q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV), nq, nkv, hd, ps,
-                      scale, window, int(q_len.max()), int(kv_len.max()))
+    if tiled_shape is None:
+        k.paged_attention(qkv, out, kc, vc, table, q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV), nq, nkv, hd, ps,
+                          scale, window, int(q_len.max()), int(kv_len.max()))
+    else:
+        # the LDS-tiled kernel with a given workgroup shape (the wrapper picks one by the amount of work)
+        qs, ql, kl = q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV)
+        k._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), kc.data_ptr(), vc.data_ptr(),
+               table.data_ptr(), table.shape[1], qs.data_ptr(), ql.data_ptr(), kl.data_ptr(), len(seqs), t, nq, nkv,
+               hd, ps, scale, window, tiled_shape, k._stream())
+        torch.cuda.synchronize()
     got = out.double().cpu().view(t, nq, hd)
     worst = 0.0
     for b, (n, kv) in enumerate(seqs):
@@ -416,6 +424,24 @@ def test_paged_attention_window(k, dtype, window, hd):
     seqs = [(1, 100), (20, 90), (5, 5), (1, window), (1, window + 1), (3, 66), (40, 300)]
     err = run_paged(k, seqs, 6, 2, hd, 16, dtype, window=window)
     assert err <= (2e-6 if dtype == torch.float32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("hd,shape", [(64, 41), (64, 42), (64, 44), (64, 22), (64, 24), (128, 41), (128, 42), (128, 22)])
+@pytest.mark.parametrize("window,ps", [(0, 16), (0, 64), (100, 32), (300, 16)])
+def test_paged_attention_tiled_workgroup_shapes(k, hd, shape, window, ps):
+    # every workgroup shape of the LDS-tiled kernel (row tiles x key splits): prompts over several row groups and
+    # key tiles, a prefix in the cache, single tokens, lengths at and around the tile sizes
+    seqs = [(300, 700), (1, 1), (64, 64), (65, 129), (2, 513), (1, 257), (127, 128), (17, 1000)]
+    assert run_paged(k, seqs, 6, 2, hd, ps, torch.bfloat16, window=window, tiled_shape=shape) <= 1.2e-2
+    assert run_paged(k, seqs, 7, 1, hd, ps, torch.bfloat16, window=window, tiled_shape=shape, q_scale=6.0, seed=3) <= 4e-2
+
+
+def test_paged_attention_tiled_refuses_other_page_sizes(k):
+    z = torch.zeros(64, device=DEV)
+    p = z.data_ptr()
+    for ps, shape in ((48, 42), (8, 42), (16, 43)):          # not a power of two, too small, no such shape
+        with pytest.raises(RuntimeError):
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, None)
 
 
 @pytest.mark.parametrize("nq,nkv,hd", [(14, 2, 64), (12, 2, 128), (3, 1, 64)])
