@@ -84,47 +84,44 @@ __device__ __forceinline__ void load8f(const float* p, float* v) {
     v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
 }
 
-// v += sum over splits of p[s * stride .. + 8]; up to kInFlight splits' loads are in flight together (what a
-// dependent kernel chain pays for is round trips to L2, not bytes; more would cost registers and with them
-// the co-residency of all workgroups); additions in split order
-constexpr int kInFlight = 8;
-
+// Adding partial sums up.  What a dependent kernel chain pays for is round trips to L2, not bytes, so the
+// loads of one batch of splits are issued together, as straight-line code: a split past the last one reads
+// the last one again (a cached line) and counts with weight zero, instead of a branch that would end the
+// batch.  More loads in flight cost registers and with them the co-residency of workgroups, hence the batch
+// size is the caller's choice.  Additions are in split order.
+template <int INF>
 __device__ __forceinline__ void add_splits8(const float* p, int n_splits, size_t stride, float* v) {
-    for (int s0 = 0; s0 < n_splits; s0 += kInFlight) {
-        float t[kInFlight][8];
+    for (int s0 = 0; s0 < n_splits; s0 += INF) {
+        float t[INF][8];
 #pragma unroll
-        for (int i = 0; i < kInFlight; ++i) {
-            if (s0 + i < n_splits) {
-                load8f(p + (s0 + i) * stride, t[i]);
-            } else {
+        for (int i = 0; i < INF; ++i) load8f(p + min(s0 + i, n_splits - 1) * stride, t[i]);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) t[i][j] = 0.f;
-            }
+        for (int i = 0; i < INF; ++i) {
+            const float on = s0 + i < n_splits ? 1.f : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = fmaf(on, t[i][j], v[j]);
         }
-#pragma unroll
-        for (int i = 0; i < kInFlight; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] += t[i][j];
     }
 }
 
-// sum over splits of p[s * stride], up to 16 loads in flight
+// sum over splits of p[s * stride], 16 loads in flight
 __device__ __forceinline__ float sum_splits(const float* p, int n_splits, size_t stride) {
     float v = 0.f;
     for (int s0 = 0; s0 < n_splits; s0 += 16) {
         float t[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) t[i] = s0 + i < n_splits ? p[(s0 + i) * stride] : 0.f;
+        for (int i = 0; i < 16; ++i) t[i] = p[min(s0 + i, n_splits - 1) * stride];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v += t[i];
+        for (int i = 0; i < 16; ++i) v += s0 + i < n_splits ? t[i] : 0.f;
     }
     return v;
 }
 
-template <int MT, int PRO>
+// INF: how many splits' loads of the prologue's input are in flight together (kNorm, kAttn)
+template <int MT, int PRO, int INF>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][kLdsRow];
-    __shared__ float row_scale[16];                                      // kSwiglu: 1 / rms of each row
+    __shared__ float ss_part[2][16];                                     // kNorm: sums of squares of a short range
     __shared__ float head_wgt[PRO == kAttn ? 16 * kMaxLocalHeads * kMaxAttnSplits : 1];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int li = lane % 16, lg = lane / 16;
@@ -134,6 +131,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
     const int total_steps = (k + kStep - 1) / kStep;
     const int step_begin = split * a.steps_per_split;
     const int step_end = min(total_steps, step_begin + a.steps_per_split);
+    const int n_steps = step_end - step_begin;
     const int w_row = min(n0 + li, n - 1);
     const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + lg * 32;
 
@@ -141,177 +139,260 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- what the prologue needs once per workgroup
-    int head_begin = 0;
-    if constexpr (PRO == kSwiglu) {
-        if (tid < 16) {
-            float inv = 1.f;
-            if (a.ss_in && tid < m) {
-                const float ss = sum_splits(a.ss_in + tid, a.ss_splits, m);
-                inv = 1.0f / sqrtf(ss * a.inv_hidden + a.eps);
-            }
-            row_scale[tid] = inv;
-        }
-        __syncthreads();
-    }
-    if constexpr (PRO == kAttn) {
-        // weight of split s for (row r, head): exp(max_s - max) / sum_s exp(max_s - max) * l_s
-        head_begin = (step_begin * kStep) / a.hd;
-        const int head_end = min(a.nq, (min(k, step_end * kStep) + a.hd - 1) / a.hd);
-        const int n_local = head_end - head_begin;
-        const int rows = m * a.nq;
-        // 16 lanes per (row, head) pair, each lane four of the (at most 64) splits, so that all loads of a
-        // pair are in flight together
-        const int sub = tid % 16;
-        for (int pair = tid / 16; pair < 16 * kMaxLocalHeads; pair += 16) {
-            const int r = pair / kMaxLocalHeads, hl = pair % kMaxLocalHeads;
-            if (r >= m || hl >= n_local) continue;                 // the same for all 16 lanes of the pair
-            const size_t row = static_cast<size_t>(r) * a.nq + head_begin + hl;
-            float ms[4], ls[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int sp = sub + 16 * i;
-                const bool has = sp < a.a_splits;
-                const float* p = a.part_ml + (static_cast<size_t>(has ? sp : 0) * rows + row) * 2;
-                ms[i] = has ? p[0] : -INFINITY;
-                ls[i] = has ? p[1] : 0.f;
-            }
-            float mx = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
-            mx = fmaxf(mx, __shfl_xor(mx, 1, kWave));
-            mx = fmaxf(mx, __shfl_xor(mx, 2, kWave));
-            mx = fmaxf(mx, __shfl_xor(mx, 4, kWave));
-            mx = fmaxf(mx, __shfl_xor(mx, 8, kWave));
-            float wg[4], denom = 0.f;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                wg[i] = ms[i] == -INFINITY ? 0.f : __expf(ms[i] - mx);
-                denom += wg[i] * ls[i];
-            }
-            denom += __shfl_xor(denom, 1, kWave);
-            denom += __shfl_xor(denom, 2, kWave);
-            denom += __shfl_xor(denom, 4, kWave);
-            denom += __shfl_xor(denom, 8, kWave);
-            const float inv = 1.0f / denom;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) head_wgt[pair * kMaxAttnSplits + sub + 16 * i] = wg[i] * inv;
-        }
-        __syncthreads();
-    }
-
-    float ss_acc = 0.f;   // kNorm: this thread's share of its row's sum of squares
-    // staging of x: MT*16 rows x 128 columns = MT*16*16 chunks of 16 bytes, 256 threads
-    auto stage = [&](int buf, int step) {
-        const int k0 = step * kStep;
-#pragma unroll
-        for (int c = tid; c < MT * 16 * 16; c += 256) {
-            const int r = c / 16, col = (c % 16) * 8;
-            const int kc = k0 + col;
-            const bool ok = r < m && kc < k;
-            uint4 v = uint4{0u, 0u, 0u, 0u};
-            if constexpr (PRO == kPlain) {
-                v = load16(a.x + static_cast<size_t>(r) * k + kc, ok);
-            } else if (ok) {
-                float f[8];
-                if constexpr (PRO == kNorm) {
-                    const size_t idx = static_cast<size_t>(r) * k + kc;
-                    load8f(a.h_in + idx, f);
-                    if (a.delta) add_splits8(a.delta + idx, a.delta_splits, static_cast<size_t>(m) * k, f);
-                    if (blockIdx.x == 0) {
-                        *reinterpret_cast<f32x4*>(a.h_out + idx) = f32x4{f[0], f[1], f[2], f[3]};
-                        *reinterpret_cast<f32x4*>(a.h_out + idx + 4) = f32x4{f[4], f[5], f[6], f[7]};
-                    }
-                    const uint4 wv = *reinterpret_cast<const uint4*>(a.norm_w + kc);
-                    const uint32_t wb[4] = {wv.x, wv.y, wv.z, wv.w};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        ss_acc += f[j] * f[j];
-                        const uint32_t bits = (j & 1) ? (wb[j / 2] & 0xffff0000u) : (wb[j / 2] << 16);
-                        f[j] *= __uint_as_float(bits);
-                    }
-                } else if constexpr (PRO == kSwiglu) {
-                    float g[8] = {}, u[8] = {};
-                    const size_t idx = static_cast<size_t>(r) * 2 * k + kc;
-                    const size_t stride = static_cast<size_t>(m) * 2 * k;
-                    add_splits8(a.gu + idx, a.gu_splits, stride, g);
-                    add_splits8(a.gu + idx + k, a.gu_splits, stride, u);
-                    const float inv = row_scale[r];
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float gg = g[j] * inv;
-                        f[j] = (u[j] * inv) * (gg / (1.0f + __expf(-gg)));
-                    }
-                } else {  // kAttn
-                    const int head = kc / a.hd, d = kc % a.hd;
-                    const float* wl = head_wgt + (r * kMaxLocalHeads + head - head_begin) * kMaxAttnSplits;
-                    const size_t rows = static_cast<size_t>(m) * a.nq;
-                    const float* po = a.part_o + (static_cast<size_t>(r) * a.nq + head) * a.hd + d;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) f[j] = 0.f;
-                    for (int s0 = 0; s0 < a.a_splits; s0 += kInFlight) {
-                        float t[kInFlight][8];
-#pragma unroll
-                        for (int i = 0; i < kInFlight; ++i) {
-                            if (s0 + i < a.a_splits) {
-                                load8f(po + (s0 + i) * rows * a.hd, t[i]);
-                            } else {
-#pragma unroll
-                                for (int j = 0; j < 8; ++j) t[i][j] = 0.f;
-                            }
-                        }
-#pragma unroll
-                        for (int i = 0; i < kInFlight; ++i) {
-                            const float wt = s0 + i < a.a_splits ? wl[s0 + i] : 0.f;
-#pragma unroll
-                            for (int j = 0; j < 8; ++j) f[j] += wt * t[i][j];
-                        }
-                    }
-                }
-                v = pack8(f);
-            }
-            *reinterpret_cast<uint4*>(&xs[buf][r][col]) = v;
-        }
-    };
     uint4 a_cur[4], a_next[4];
     auto load_w = [&](uint4* av, int step) {
         const int k0 = step * kStep + lg * 32;
 #pragma unroll
         for (int q = 0; q < 4; ++q) av[q] = load16(wp + static_cast<size_t>(step) * kStep + q * 8, k0 + q * 8 < k);
     };
+    // the stream of w starts before anything else
+    if (n_steps > 0) load_w(a_cur, step_begin);
+    if (n_steps > 1) load_w(a_next, step_begin + 1);
 
-    if (step_begin < step_end) {
-        load_w(a_cur, step_begin);
-        stage(0, step_begin);
-    }
-    __syncthreads();
-    for (int step = step_begin; step < step_end; ++step) {
-        const int buf = (step - step_begin) & 1;
-        if (step + 1 < step_end) {
-            load_w(a_next, step + 1);
-            stage(buf ^ 1, step + 1);
+    // ---- kAttn with many key splits: the weights of the splits once per workgroup, through LDS
+    int head_begin = 0;
+    const bool attn_wide = PRO == kAttn && a.a_splits > INF;
+    if constexpr (PRO == kAttn) {
+        head_begin = (step_begin * kStep) / a.hd;
+        if (attn_wide) {
+            // weight of split s for (row r, head): exp(max_s - max) / sum_s exp(max_s - max) * l_s
+            const int head_end = min(a.nq, (min(k, step_end * kStep) + a.hd - 1) / a.hd);
+            const int n_local = head_end - head_begin;
+            const int rows = m * a.nq;
+            // 16 lanes per (row, head) pair, each lane four of the (at most 64) splits, so that all loads of a
+            // pair are in flight together
+            const int sub = tid % 16;
+            for (int pair = tid / 16; pair < 16 * kMaxLocalHeads; pair += 16) {
+                const int r = pair / kMaxLocalHeads, hl = pair % kMaxLocalHeads;
+                if (r >= m || hl >= n_local) continue;                 // the same for all 16 lanes of the pair
+                const size_t row = static_cast<size_t>(r) * a.nq + head_begin + hl;
+                float ms[4], ls[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int sp = sub + 16 * i;
+                    const bool has = sp < a.a_splits;
+                    const float* p = a.part_ml + (static_cast<size_t>(has ? sp : 0) * rows + row) * 2;
+                    ms[i] = has ? p[0] : -INFINITY;
+                    ls[i] = has ? p[1] : 0.f;
+                }
+                float mx = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
+                mx = fmaxf(mx, __shfl_xor(mx, 1, kWave));
+                mx = fmaxf(mx, __shfl_xor(mx, 2, kWave));
+                mx = fmaxf(mx, __shfl_xor(mx, 4, kWave));
+                mx = fmaxf(mx, __shfl_xor(mx, 8, kWave));
+                float wg[4], denom = 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    wg[i] = ms[i] == -INFINITY ? 0.f : __expf(ms[i] - mx);
+                    denom += wg[i] * ls[i];
+                }
+                denom += __shfl_xor(denom, 1, kWave);
+                denom += __shfl_xor(denom, 2, kWave);
+                denom += __shfl_xor(denom, 4, kWave);
+                denom += __shfl_xor(denom, 8, kWave);
+                const float inv = 1.0f / denom;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) head_wgt[pair * kMaxAttnSplits + sub + 16 * i] = wg[i] * inv;
+            }
+            __syncthreads();
         }
+    }
+
+    // ---- one chunk of x: the 8 values of row r at columns col.. of step `step`, computed by the prologue and
+    // stored where the MFMA operand loads expect them.  Returns the chunk's sum of squares (kNorm).
+    // Rows >= m are never written: an MFMA output column depends on its own column of x only, and the
+    // columns of those rows are not stored.
+    auto chunk = [&](int buf, int step, int r, int col) -> float {
+        const int kc = step * kStep + col;
+        uint4 v = uint4{0u, 0u, 0u, 0u};          // past k the operand is zero, as w's is
+        float ssq = 0.f;
+        if constexpr (PRO == kPlain) {
+            v = load16(a.x + static_cast<size_t>(r) * k + kc, kc < k);
+        } else if (kc < k) {
+            float f[8];
+            if constexpr (PRO == kNorm) {
+                const size_t idx = static_cast<size_t>(r) * k + kc;
+                load8f(a.h_in + idx, f);
+                const uint4 wv = *reinterpret_cast<const uint4*>(a.norm_w + kc);
+                if (a.delta) add_splits8<INF>(a.delta + idx, a.delta_splits, static_cast<size_t>(m) * k, f);
+                if (blockIdx.x == 0) {
+                    *reinterpret_cast<f32x4*>(a.h_out + idx) = f32x4{f[0], f[1], f[2], f[3]};
+                    *reinterpret_cast<f32x4*>(a.h_out + idx + 4) = f32x4{f[4], f[5], f[6], f[7]};
+                }
+                const uint32_t wb[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    ssq += f[j] * f[j];
+                    const uint32_t bits = (j & 1) ? (wb[j / 2] & 0xffff0000u) : (wb[j / 2] << 16);
+                    f[j] *= __uint_as_float(bits);
+                }
+            } else if constexpr (PRO == kSwiglu) {
+                // gate, up and the row's sums of squares: every load is issued before the first is waited
+                // for (the counter of outstanding loads is in order, so a wait for any of them is a wait for
+                // the stream of w as well: one round trip in all)
+                constexpr int GU = 4, SS = 8;     // splits per batch of loads
+                const size_t idx = static_cast<size_t>(r) * 2 * k + kc;
+                const size_t stride = static_cast<size_t>(m) * 2 * k;
+                float tg[GU][8], tu[GU][8], sst[SS];
+#pragma unroll
+                for (int i = 0; i < GU; ++i) {
+                    const float* p = a.gu + idx + min(i, a.gu_splits - 1) * stride;
+                    load8f(p, tg[i]);
+                    load8f(p + k, tu[i]);
+                }
+                const float* ssp = a.ss_in ? a.ss_in + r : a.gu;       // without a scale: any readable address
+                const int ss_n = a.ss_in ? a.ss_splits : 1;
+#pragma unroll
+                for (int i = 0; i < SS; ++i) sst[i] = ssp[min(i, ss_n - 1) * m];
+                float g[8] = {}, u[8] = {};
+#pragma unroll
+                for (int i = 0; i < GU; ++i) {
+                    const float on = i < a.gu_splits ? 1.f : 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        g[j] = fmaf(on, tg[i][j], g[j]);
+                        u[j] = fmaf(on, tu[i][j], u[j]);
+                    }
+                }
+                if (a.gu_splits > GU) {
+                    add_splits8<GU>(a.gu + idx + GU * stride, a.gu_splits - GU, stride, g);
+                    add_splits8<GU>(a.gu + idx + GU * stride + k, a.gu_splits - GU, stride, u);
+                }
+                float ss = 0.f;
+#pragma unroll
+                for (int i = 0; i < SS; ++i) ss += i < ss_n ? sst[i] : 0.f;
+                if (ss_n > SS) ss += sum_splits(ssp + SS * m, ss_n - SS, m);
+                const float inv = a.ss_in ? 1.0f / sqrtf(ss * a.inv_hidden + a.eps) : 1.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float gg = g[j] * inv;
+                    f[j] = (u[j] * inv) * gg * __builtin_amdgcn_rcpf(1.0f + __expf(-gg));
+                }
+            } else {  // kAttn
+                const int head = kc / a.hd, d = kc % a.hd;
+                const size_t rows = static_cast<size_t>(m) * a.nq;
+                const size_t row = static_cast<size_t>(r) * a.nq + head;
+                const float* po = a.part_o + row * a.hd + d;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[j] = 0.f;
+                if (!attn_wide) {
+                    // few splits: their (maximum, sum) pairs and outputs in one batch of loads, the weights
+                    // computed by every thread for itself
+                    float ms[INF], ls[INF], t[INF][8];
+#pragma unroll
+                    for (int i = 0; i < INF; ++i) {
+                        const int sp = min(i, a.a_splits - 1);
+                        const float* pm = a.part_ml + (sp * rows + row) * 2;
+                        ms[i] = pm[0];
+                        ls[i] = pm[1];
+                        load8f(po + sp * rows * a.hd, t[i]);
+                    }
+                    float mx = -INFINITY;
+#pragma unroll
+                    for (int i = 0; i < INF; ++i) {
+                        if (i >= a.a_splits) ms[i] = -INFINITY;
+                        mx = fmaxf(mx, ms[i]);
+                    }
+                    float wg[INF], denom = 0.f;
+#pragma unroll
+                    for (int i = 0; i < INF; ++i) {
+                        wg[i] = ms[i] == -INFINITY ? 0.f : __expf(ms[i] - mx);
+                        denom += wg[i] * ls[i];
+                    }
+                    const float inv = 1.0f / denom;
+#pragma unroll
+                    for (int i = 0; i < INF; ++i) {
+                        const float wt = wg[i] * inv;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) f[j] = fmaf(wt, t[i][j], f[j]);
+                    }
+                } else {
+                    const float* wl = head_wgt + (r * kMaxLocalHeads + head - head_begin) * kMaxAttnSplits;
+                    for (int s0 = 0; s0 < a.a_splits; s0 += INF) {
+                        float t[INF][8];
+#pragma unroll
+                        for (int i = 0; i < INF; ++i) load8f(po + min(s0 + i, a.a_splits - 1) * rows * a.hd, t[i]);
+#pragma unroll
+                        for (int i = 0; i < INF; ++i) {
+                            const float wt = s0 + i < a.a_splits ? wl[s0 + i] : 0.f;
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) f[j] = fmaf(wt, t[i][j], f[j]);
+                        }
+                    }
+                }
+            }
+            v = pack8(f);
+        }
+        *reinterpret_cast<uint4*>(&xs[buf][r][col]) = v;
+        return ssq;
+    };
+    auto products = [&](int buf, const uint4* av4) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const bf16x8 av = __builtin_bit_cast(bf16x8, a_cur[q]);
+            const bf16x8 av = __builtin_bit_cast(bf16x8, av4[q]);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
                 const uint4 bv = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + li][lg * 32 + q * 8]);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
             }
         }
+    };
+
+    if (n_steps <= 2) {
+        // A short range (the usual case when the k range is split): both steps are staged at once, the
+        // chunks of the valid rows dealt out over all threads, so that the prologue is one round of loads.
+        const int per_step = m * 16;
+        for (int it = tid; it < n_steps * per_step; it += 256) {
+            const int s = it / per_step, rem = it % per_step;
+            const int r = rem / 16;
+            float ssq = chunk(s, step_begin + s, r, (rem % 16) * 8);
+            if constexpr (PRO == kNorm) {
+                // the 16 threads of a (step, row) sit side by side in one wavefront
+                ssq += __shfl_xor(ssq, 1, kWave);
+                ssq += __shfl_xor(ssq, 2, kWave);
+                ssq += __shfl_xor(ssq, 4, kWave);
+                ssq += __shfl_xor(ssq, 8, kWave);
+                if (rem % 16 == 0) ss_part[s][r] = ssq;
+            }
+        }
         __syncthreads();
+        if (n_steps > 0) products(0, a_cur);
+        if (n_steps > 1) products(1, a_next);
+        if constexpr (PRO == kNorm) {
+            if (blockIdx.x == 0 && tid < m)
+                a.ss_out[split * m + tid] = (n_steps > 0 ? ss_part[0][tid] : 0.f) + (n_steps > 1 ? ss_part[1][tid] : 0.f);
+        }
+    } else {
+        // A long range: x double-buffered in LDS, a thread keeps its (row, column) over the steps.
+        float ss_acc = 0.f;
+        auto stage = [&](int buf, int step) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) a_cur[q] = a_next[q];
-    }
-    if constexpr (PRO == kNorm) {
-        // the 16 threads that staged a row sit side by side in one wavefront
-        if (blockIdx.x == 0) {
-            float ss = ss_acc;
-            ss += __shfl_xor(ss, 1, kWave);
-            ss += __shfl_xor(ss, 2, kWave);
-            ss += __shfl_xor(ss, 4, kWave);
-            ss += __shfl_xor(ss, 8, kWave);
-            const int r = tid / 16;
-            if (tid % 16 == 0 && r < m) a.ss_out[split * m + r] = ss;
+            for (int c = tid; c < MT * 16 * 16; c += 256) {
+                const int r = c / 16;
+                if (r < m) ss_acc += chunk(buf, step, r, (c % 16) * 8);
+            }
+        };
+        stage(0, step_begin);
+        __syncthreads();
+        for (int step = step_begin; step < step_end; ++step) {
+            const int buf = (step - step_begin) & 1;
+            if (step > step_begin && step + 1 < step_end) load_w(a_next, step + 1);
+            if (step + 1 < step_end) stage(buf ^ 1, step + 1);
+            products(buf, a_cur);
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) a_cur[q] = a_next[q];
+        }
+        if constexpr (PRO == kNorm) {
+            if (blockIdx.x == 0) {
+                float ss = ss_acc;
+                ss += __shfl_xor(ss, 1, kWave);
+                ss += __shfl_xor(ss, 2, kWave);
+                ss += __shfl_xor(ss, 4, kWave);
+                ss += __shfl_xor(ss, 8, kWave);
+                const int r = tid / 16;
+                if (tid % 16 == 0 && r < m) a.ss_out[split * m + r] = ss;
+            }
         }
     }
     // D layout: lane (li, lg) holds rows lg*4 + v of the 16 x 16 tile (an n index) at column li (an m index)
@@ -368,10 +449,10 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
     const dim3 grid = skinny_grid(n, n_splits);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch ((m + 15) / 16) {
-        case 1: gemm_skinny_kernel<1, kPlain><<<grid, 256, 0, s>>>(a); break;
-        case 2: gemm_skinny_kernel<2, kPlain><<<grid, 256, 0, s>>>(a); break;
-        case 3: gemm_skinny_kernel<3, kPlain><<<grid, 256, 0, s>>>(a); break;
-        default: gemm_skinny_kernel<4, kPlain><<<grid, 256, 0, s>>>(a); break;
+        case 1: gemm_skinny_kernel<1, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
+        case 2: gemm_skinny_kernel<2, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
+        case 3: gemm_skinny_kernel<3, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
+        default: gemm_skinny_kernel<4, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
     }
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
@@ -394,7 +475,12 @@ extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const floa
     a.h_in = h_in; a.h_out = h_out; a.delta = delta; a.delta_splits = delta ? delta_splits : 0;
     a.norm_w = static_cast<const bf16_t*>(norm_w);
     a.ss_out = ss_out;
-    gemm_skinny_kernel<1, kNorm><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    // Many partial sums to add and few workgroups (which then need not share a CU): more loads in flight.
+    const dim3 grid = skinny_grid(n, n_splits);
+    if (a.delta_splits > 8 && grid.x * grid.y <= 512)
+        gemm_skinny_kernel<1, kNorm, 20><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    else
+        gemm_skinny_kernel<1, kNorm, 8><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(a);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -415,7 +501,7 @@ extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, cons
     a.gu = gate_up; a.gu_splits = gu_splits; a.ss_in = ss_in; a.ss_splits = ss_splits;
     a.inv_hidden = ss_in ? 1.0f / static_cast<float>(hidden) : 0.f;
     a.eps = eps;
-    gemm_skinny_kernel<1, kSwiglu><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    gemm_skinny_kernel<1, kSwiglu, 8><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -435,7 +521,7 @@ extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, 
     a.out_f32 = out;
     a.m = m; a.n = n; a.k = k;
     a.part_o = part_o; a.part_ml = part_ml; a.a_splits = a_splits; a.nq = nq; a.hd = hd;
-    gemm_skinny_kernel<1, kAttn><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    gemm_skinny_kernel<1, kAttn, 8><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -187,7 +187,7 @@ class HipKernels:
         bounded so that the partial sums stay smaller than the weights they came from."""
         steps = -(-k // 128)
         n_blocks = -(-n // 64)
-        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)), 16)
+        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)), 20)
         per = -(-steps // s)
         return -(-steps // per)
 
@@ -218,7 +218,7 @@ class HipKernels:
                   norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, self._stream())
         return out, ss, h_new
 
-    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=16):
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=20):
         """swiglu(scale * sum gate_up) w^T for float32 partial sums gate_up [S, T, 2I]; scale is the rows' 1/rms
         from row_ss [S2, T] (or 1).  Returns float32 partial sums [S3, T, N] or None if not covered."""
         if gate_up.dim() != 3 or gate_up.dtype != _F32 or w.dtype != _BF16:
