@@ -27,8 +27,9 @@ int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, i
                         const float* inv_freq, int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache,
                         int n_tokens, int nq, int nkv, int hd, int page_size, int dtype, void* stream);
 // bfloat16 product for m <= 64 rows on the matrix cores, optionally split over k (see gemm_skinny.hip).
+// waves: wavefronts (of 16 columns of the result each) per workgroup, 4, 8 or 16; here and below.
 int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m, int n,
-                     int k, int n_splits, void* stream);
+                     int k, int n_splits, int waves, void* stream);
 // out = x w^T + bias; x [m,k], w [n,k], out [m,n]; out_f32 != 0 writes float32 whatever dtype is.
 int egpt_linear(const void* x, const void* w, const void* bias, void* out, int m, int n, int k, int dtype,
                 int out_f32, void* stream);
@@ -60,11 +61,13 @@ int egpt_attention_combine(const float* part_o, const float* part_ml, void* out,
                            void* stream);
 // Products for m <= 16 rows whose x operand is computed while it is staged (see gemm_skinny.hip).
 int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits, const void* norm_w,
-                          const void* w, float* out, float* ss_out, int m, int n, int k, int n_splits, void* stream);
+                          const void* w, float* out, float* ss_out, int m, int n, int k, int n_splits, int waves,
+                          void* stream);
 int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits, int hidden,
-                            float eps, const void* w, float* out, int m, int n, int k, int n_splits, void* stream);
+                            float eps, const void* w, float* out, int m, int n, int k, int n_splits, int waves,
+                            void* stream);
 int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd, const void* w,
-                          float* out, int m, int n, int n_splits, void* stream);
+                          float* out, int m, int n, int n_splits, int waves, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 // weights: scratch for n_rows * vocab floats.

@@ -31,7 +31,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kStep = 128;          // k elements per step
 constexpr int kRowsPerWave = 16;
-constexpr int kWavesPerBlock = 4;
 constexpr int kLdsRow = kStep + 8;  // bf16 elements per staged row of x (16 bytes of padding)
 constexpr int kMaxLocalHeads = 8;   // ATTN prologue: heads that one workgroup's k range may touch
 constexpr int kMaxAttnSplits = 64;
@@ -118,8 +117,11 @@ __device__ __forceinline__ float sum_splits(const float* p, int n_splits, size_t
 }
 
 // INF: how many splits' loads of the prologue's input are in flight together (kNorm, kAttn)
-template <int MT, int PRO, int INF>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
+// NW: wavefronts per workgroup (each 16 rows of w); they share the staged x, so a wide workgroup reads the
+// prologue's inputs fewer times
+template <int MT, int PRO, int INF, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
+    constexpr int kThreads = 64 * NW;
     __shared__ __attribute__((aligned(16))) bf16_t xs[2][MT * 16][kLdsRow];
     __shared__ float ss_part[2][16];                                     // kNorm: sums of squares of a short range
     __shared__ float head_wgt[PRO == kAttn ? 16 * kMaxLocalHeads * kMaxAttnSplits : 1];
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
     const int li = lane % 16, lg = lane / 16;
     const int split = blockIdx.y;
     const int m = a.m, n = a.n, k = a.k;
-    const int n0 = (blockIdx.x * kWavesPerBlock + wave) * kRowsPerWave;
+    const int n0 = (blockIdx.x * NW + wave) * kRowsPerWave;
     const int total_steps = (k + kStep - 1) / kStep;
     const int step_begin = split * a.steps_per_split;
     const int step_end = min(total_steps, step_begin + a.steps_per_split);
@@ -162,7 +164,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
             // 16 lanes per (row, head) pair, each lane four of the (at most 64) splits, so that all loads of a
             // pair are in flight together
             const int sub = tid % 16;
-            for (int pair = tid / 16; pair < 16 * kMaxLocalHeads; pair += 16) {
+            for (int pair = tid / 16; pair < 16 * kMaxLocalHeads; pair += kThreads / 16) {
                 const int r = pair / kMaxLocalHeads, hl = pair % kMaxLocalHeads;
                 if (r >= m || hl >= n_local) continue;                 // the same for all 16 lanes of the pair
                 const size_t row = static_cast<size_t>(r) * a.nq + head_begin + hl;
@@ -342,7 +344,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
         // A short range (the usual case when the k range is split): both steps are staged at once, the
         // chunks of the valid rows dealt out over all threads, so that the prologue is one round of loads.
         const int per_step = m * 16;
-        for (int it = tid; it < n_steps * per_step; it += 256) {
+        for (int it = tid; it < n_steps * per_step; it += kThreads) {
             const int s = it / per_step, rem = it % per_step;
             const int r = rem / 16;
             float ssq = chunk(s, step_begin + s, r, (rem % 16) * 8);
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
         float ss_acc = 0.f;
         auto stage = [&](int buf, int step) {
 #pragma unroll
-            for (int c = tid; c < MT * 16 * 16; c += 256) {
+            for (int c = tid; c < MT * 16 * 16; c += kThreads) {
                 const int r = c / 16;
                 if (r < m) ss_acc += chunk(buf, step, r, (c % 16) * 8);
             }
@@ -422,9 +424,19 @@ static int check_splits(int k, int n_splits, int* steps_per_split) {
     return EGPT_OK;
 }
 
-static dim3 skinny_grid(int n, int n_splits) {
-    return dim3((n + kRowsPerWave * kWavesPerBlock - 1) / (kRowsPerWave * kWavesPerBlock), n_splits);
+static dim3 skinny_grid(int n, int n_splits, int waves) {
+    return dim3((n + kRowsPerWave * waves - 1) / (kRowsPerWave * waves), n_splits);
 }
+
+// launches the instance for `waves` wavefronts per workgroup (4, 8 or 16)
+#define EGPT_SKINNY(MT_, PRO_, INF_)                                                                         \
+    do {                                                                                                     \
+        const dim3 grid = skinny_grid(a.n, n_splits, waves);                                                 \
+        hipStream_t s_ = static_cast<hipStream_t>(stream);                                                   \
+        if (waves == 4) gemm_skinny_kernel<MT_, PRO_, INF_, 4><<<grid, 256, 0, s_>>>(a);                     \
+        else if (waves == 8) gemm_skinny_kernel<MT_, PRO_, INF_, 8><<<grid, 512, 0, s_>>>(a);                \
+        else gemm_skinny_kernel<MT_, PRO_, INF_, 16><<<grid, 1024, 0, s_>>>(a);                              \
+    } while (0)
 
 }  // namespace egpt
 
@@ -433,8 +445,9 @@ using namespace egpt;
 // out_f32 != null: float32 [n_splits][m][n] partial sums (bias only allowed with n_splits == 1).
 // out_bf16 != null: bfloat16 [m][n], n_splits must be 1.
 extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m,
-                                int n, int k, int n_splits, void* stream) {
-    if (!x || !w || (!out_f32 && !out_bf16) || (out_f32 && out_bf16) || m <= 0 || n <= 0 || k <= 0 || n_splits <= 0)
+                                int n, int k, int n_splits, int waves, void* stream) {
+    if (!x || !w || (!out_f32 && !out_bf16) || (out_f32 && out_bf16) || m <= 0 || n <= 0 || k <= 0 || n_splits <= 0 ||
+        (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     if (m > 64 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
     if (n_splits > 1 && (bias || out_bf16)) return EGPT_BAD_ARGUMENT;
@@ -446,13 +459,11 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
     a.out_f32 = out_f32;
     a.out_bf16 = static_cast<bf16_t*>(out_bf16);
     a.m = m; a.n = n; a.k = k;
-    const dim3 grid = skinny_grid(n, n_splits);
-    hipStream_t s = static_cast<hipStream_t>(stream);
     switch ((m + 15) / 16) {
-        case 1: gemm_skinny_kernel<1, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
-        case 2: gemm_skinny_kernel<2, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
-        case 3: gemm_skinny_kernel<3, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
-        default: gemm_skinny_kernel<4, kPlain, 8><<<grid, 256, 0, s>>>(a); break;
+        case 1: EGPT_SKINNY(1, kPlain, 8); break;
+        case 2: EGPT_SKINNY(2, kPlain, 8); break;
+        case 3: EGPT_SKINNY(3, kPlain, 8); break;
+        default: EGPT_SKINNY(4, kPlain, 8); break;
     }
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
@@ -462,9 +473,9 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
 // ss_out[split][m] = sums of squares of h_out over the split's k range.  m <= 16, k % 8 == 0.
 extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits,
                                      const void* norm_w, const void* w, float* out, float* ss_out, int m, int n, int k,
-                                     int n_splits, void* stream) {
+                                     int n_splits, int waves, void* stream) {
     if (!h_in || !h_out || h_in == h_out || !norm_w || !w || !out || !ss_out || m <= 0 || n <= 0 || k <= 0 ||
-        delta_splits < 0 || (delta && delta_splits == 0))
+        delta_splits < 0 || (delta && delta_splits == 0) || (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
     SkinnyArgs a = {};
@@ -476,11 +487,15 @@ extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const floa
     a.norm_w = static_cast<const bf16_t*>(norm_w);
     a.ss_out = ss_out;
     // Many partial sums to add and few workgroups (which then need not share a CU): more loads in flight.
-    const dim3 grid = skinny_grid(n, n_splits);
-    if (a.delta_splits > 8 && grid.x * grid.y <= 512)
-        gemm_skinny_kernel<1, kNorm, 20><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    // As many loads in flight as there are partial sums to add, if registers allow: few workgroups need not
+    // share a CU.
+    const dim3 g = skinny_grid(n, n_splits, waves);
+    if (a.delta_splits <= 4)
+        EGPT_SKINNY(1, kNorm, 4);
+    else if (a.delta_splits > 8 && g.x * g.y <= 512 && waves == 4)
+        EGPT_SKINNY(1, kNorm, 20);
     else
-        gemm_skinny_kernel<1, kNorm, 8><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+        EGPT_SKINNY(1, kNorm, 8);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -489,8 +504,9 @@ extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const floa
 // inv_rms[m] = 1 / sqrt(sum_s ss_in[s][m] / hidden + eps), or 1 if ss_in is null.
 extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits,
                                        int hidden, float eps, const void* w, float* out, int m, int n, int k,
-                                       int n_splits, void* stream) {
-    if (!gate_up || gu_splits < 1 || !w || !out || m <= 0 || n <= 0 || k <= 0 || (ss_in && (ss_splits < 1 || hidden < 1)))
+                                       int n_splits, int waves, void* stream) {
+    if (!gate_up || gu_splits < 1 || !w || !out || m <= 0 || n <= 0 || k <= 0 || (ss_in && (ss_splits < 1 || hidden < 1)) ||
+        (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
     SkinnyArgs a = {};
@@ -501,7 +517,7 @@ extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, cons
     a.gu = gate_up; a.gu_splits = gu_splits; a.ss_in = ss_in; a.ss_splits = ss_splits;
     a.inv_hidden = ss_in ? 1.0f / static_cast<float>(hidden) : 0.f;
     a.eps = eps;
-    gemm_skinny_kernel<1, kSwiglu, 8><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    EGPT_SKINNY(1, kSwiglu, 8);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -509,8 +525,9 @@ extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, cons
 // out[split][m][n] = partial sums of (combined attention output) w^T; part_o [a_splits][m*nq][hd] unnormalised
 // partial outputs, part_ml [a_splits][m*nq][2] their (maximum, sum); k = nq * hd.
 extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd,
-                                     const void* w, float* out, int m, int n, int n_splits, void* stream) {
-    if (!part_o || !part_ml || a_splits < 1 || nq < 1 || hd < 1 || !w || !out || m <= 0 || n <= 0)
+                                     const void* w, float* out, int m, int n, int n_splits, int waves, void* stream) {
+    if (!part_o || !part_ml || a_splits < 1 || nq < 1 || hd < 1 || !w || !out || m <= 0 || n <= 0 ||
+        (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     const int k = nq * hd;
     if (m > 16 || (hd % 8) != 0 || a_splits > kMaxAttnSplits) return EGPT_UNSUPPORTED_SIZE;
@@ -521,7 +538,7 @@ extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, 
     a.out_f32 = out;
     a.m = m; a.n = n; a.k = k;
     a.part_o = part_o; a.part_ml = part_ml; a.a_splits = a_splits; a.nq = nq; a.hd = hd;
-    gemm_skinny_kernel<1, kAttn, 8><<<skinny_grid(n, n_splits), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    EGPT_SKINNY(1, kAttn, 8);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

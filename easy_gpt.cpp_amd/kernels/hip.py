@@ -47,14 +47,14 @@ class HipKernels:
             "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
             "egpt_swiglu": [vp, i, vp, i, i, i, vp],
             "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
-            "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, vp],
-            "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, vp],
-            "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, vp],
+            "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
             "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
-            "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, vp],
+            "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
@@ -169,7 +169,7 @@ class HipKernels:
                     xo, oo = x[r0:r1], out[r0:r1]
                     self._run("egpt_gemm_skinny", xo.data_ptr(), w.data_ptr(), self._ptr(bias),
                               oo.data_ptr() if to_f32 else None, None if to_f32 else oo.data_ptr(), r1 - r0, n, k, 1,
-                              self._stream())
+                              4, self._stream())
                 return out
             # many rows: the library's matrix product (the reference uses cuBLAS for every linear layer)
             if bias is None:
@@ -193,7 +193,7 @@ class HipKernels:
 
     fused_rows = 16     # products with a computed x operand take at most this many rows
 
-    def product_normed(self, h, delta, norm_weight, w):
+    def product_normed(self, h, delta, norm_weight, w, waves=4, splits=None):
         """((h + delta) * norm_weight) w^T without the rows' 1/rms factor, for few rows in bfloat16.
         Returns (float32 partial sums [S, T, N], row sums of squares [S, T], h + delta as a new tensor),
         or None if this case is not covered (the caller then runs the norm by itself)."""
@@ -210,15 +210,15 @@ class HipKernels:
         if delta is not None:
             d_splits = int(delta.shape[0])
             self._need(delta, "delta", _F32, (d_splits, t, k))
-        s = self._n_splits(t, n, k)
+        s = splits or self._n_splits(t, n, k)
         out = torch.empty((s, t, n), dtype=_F32, device=h.device)
         ss = torch.empty((s, t), dtype=_F32, device=h.device)
         h_new = torch.empty_like(h)
         self._run("egpt_gemm_skinny_norm", h.data_ptr(), h_new.data_ptr(), self._ptr(delta), d_splits,
-                  norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, self._stream())
+                  norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, waves, self._stream())
         return out, ss, h_new
 
-    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=20):
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=20, waves=None):
         """swiglu(scale * sum gate_up) w^T for float32 partial sums gate_up [S, T, 2I]; scale is the rows' 1/rms
         from row_ss [S2, T] (or 1).  Returns float32 partial sums [S3, T, N] or None if not covered."""
         if gate_up.dim() != 3 or gate_up.dtype != _F32 or w.dtype != _BF16:
@@ -236,12 +236,16 @@ class HipKernels:
         s = min(self._n_splits(t, n, k), max_splits)
         steps = -(-k // 128)
         s = -(-steps // -(-steps // s))
+        if waves is None:
+            # every workgroup computes its share of x from all of gate_up's partial sums: with few columns,
+            # wider workgroups (which share the staged x) do that work fewer times
+            waves = 8 if -(-n // 64) * s <= 512 else 4
         out = torch.empty((s, t, n), dtype=_F32, device=w.device)
         self._run("egpt_gemm_skinny_swiglu", gate_up.data_ptr(), int(g_splits), self._ptr(row_ss), ss_splits, int(hidden),
-                  float(eps), w.data_ptr(), out.data_ptr(), t, n, k, s, self._stream())
+                  float(eps), w.data_ptr(), out.data_ptr(), t, n, k, s, waves, self._stream())
         return out
 
-    def product_attention(self, part_o, part_ml, w, max_splits=4):
+    def product_attention(self, part_o, part_ml, w, max_splits=4, waves=4):
         """(combined attention output) w^T from the parts of a split attention: part_o [S, T, nq, hd],
         part_ml [S, T, nq, 2].  Returns float32 partial sums [S2, T, N] or None if not covered."""
         a_splits, t, nq, hd = part_o.shape
@@ -259,7 +263,7 @@ class HipKernels:
             return None
         out = torch.empty((s, t, n), dtype=_F32, device=w.device)
         self._run("egpt_gemm_skinny_attn", part_o.data_ptr(), part_ml.data_ptr(), int(a_splits), int(nq), int(hd),
-                  w.data_ptr(), out.data_ptr(), t, n, s, self._stream())
+                  w.data_ptr(), out.data_ptr(), t, n, s, waves, self._stream())
         return out
 
     def combine_attention(self, part_o, part_ml, out):
@@ -284,7 +288,7 @@ class HipKernels:
             self._need(w, "w", x.dtype, (n, k))
             s = self._n_splits(m, n, k)
             out = torch.empty((s, m, n), dtype=_F32, device=x.device)
-            self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s,
+            self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s, 4,
                       self._stream())
             return out
         if unrounded and x.dtype == _BF16 and m > 64 and k % 8 == 0:

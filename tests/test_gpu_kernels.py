@@ -100,9 +100,11 @@ def test_skinny_product_and_partial_sums(k, m, n, kk):
         steps = -(-kk // 128)
         if s > steps or (s - 1) * -(-steps // s) >= steps:
             continue
-        out = torch.full((s, m, n), 7.0, dtype=torch.float32, device=DEV)
-        k._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, kk, s, k._stream())
-        assert float((out.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale, s
+        for waves in (4, 8, 16):                 # wavefronts per workgroup
+            out = torch.full((s, m, n), 7.0, dtype=torch.float32, device=DEV)
+            k._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, kk, s, waves,
+                   k._stream())
+            assert float((out.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale, (s, waves)
     out32 = torch.empty(m, n, dtype=torch.float32, device=DEV)
     k.linear(x, w, b, out32)
     assert float((out32.double().cpu() - ref - b.double().cpu()).abs().max()) <= 3e-6 * scale
@@ -163,19 +165,24 @@ def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
     nw = (1 + rnd(hid, seed=3, scale=0.1)).to(dtype)
     w = rnd(n, hid, dtype=dtype, seed=4, scale=0.05)
     h0 = h.clone()
-    prod, ss, h_new = k.product_normed(h, delta, nw, w)
-    assert torch.equal(h, h0)                                           # the input stream is left alone
     summed = h0.clone()
     for s in range(d_splits):
         summed += delta[s]
-    assert torch.equal(h_new, summed)
     sd = summed.double().cpu()
-    assert torch.allclose(ss.double().sum(0).cpu(), (sd * sd).sum(-1), rtol=1e-5)
     eps = 1e-6
-    inv = 1.0 / torch.sqrt(ss.double().sum(0).cpu() / hid + eps)
-    got = prod.double().sum(0).cpu() * inv[:, None]
     ref = plain.linear(plain.rms_norm(sd, nw.double().cpu(), eps), w.double().cpu())
-    assert float((got - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+    # every workgroup width; the k range in as many pieces as the wrapper likes (short ranges, staged at once),
+    # in one piece and in two (long ranges, staged step by step)
+    for waves, splits in ((4, None), (8, None), (16, None), (4, 1), (16, 1), (8, 2)):
+        if splits and splits > -(-hid // 128):
+            continue
+        prod, ss, h_new = k.product_normed(h, delta, nw, w, waves=waves, splits=splits)
+        assert torch.equal(h, h0)                                           # the input stream is left alone
+        assert torch.equal(h_new, summed)
+        assert torch.allclose(ss.double().sum(0).cpu(), (sd * sd).sum(-1), rtol=1e-5)
+        inv = 1.0 / torch.sqrt(ss.double().sum(0).cpu() / hid + eps)
+        got = prod.double().sum(0).cpu() * inv[:, None]
+        assert float((got - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, splits)
     # and the QKV epilogue applies that factor
     if n == 1152:
         nq, nkv, hd, ps = 14, 2, 64, 16
@@ -188,7 +195,7 @@ def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
         assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())   # position 0: no rotation
 
 
-@pytest.mark.parametrize("t,inter,n,g_splits", [(8, 4864, 896, 4), (3, 200, 120, 1), (16, 328, 192, 2)])
+@pytest.mark.parametrize("t,inter,n,g_splits", [(8, 4864, 896, 4), (3, 200, 120, 1), (16, 328, 192, 2), (7, 640, 100, 6)])
 def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
     gu = rnd(g_splits, t, 2 * inter, seed=1, scale=1.5)
     ss = torch.rand(3, t, generator=torch.Generator().manual_seed(2)).to(DEV) * 50 + 1
@@ -199,9 +206,10 @@ def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
         z = gu.double().sum(0).cpu() * scale
         g, u = z[:, :inter], z[:, inter:]
         ref = plain.linear(u * g / (1 + torch.exp(-g)), w.double().cpu())
-        prod = k.product_swiglu(gu, row_ss, hidden, eps, w)
-        assert prod is not None and prod.dim() == 3
-        assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+        for waves, max_splits in ((4, 20), (8, 20), (16, 20), (4, 1), (16, 2)):      # short and long k ranges
+            prod = k.product_swiglu(gu, row_ss, hidden, eps, w, max_splits=max_splits, waves=waves)
+            assert prod is not None and prod.dim() == 3
+            assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, max_splits)
 
 
 @pytest.mark.parametrize("nq,nkv,hd,batch,ctx", [(14, 2, 64, 8, 700), (12, 2, 128, 3, 300), (14, 2, 64, 1, 2113), (3, 1, 64, 16, 90)])
@@ -227,9 +235,13 @@ def test_output_projection_combines_attention_parts(k, nq, nkv, hd, batch, ctx):
     k.combine_attention(parts[0], parts[1], again)
     assert float((again.float() - out.float()).abs().max()) <= 2e-2      # other splits, other rounding
     w = rnd(200, nq * hd, dtype=dtype, seed=7, scale=0.05)
-    prod = k.product_attention(parts[0], parts[1], w)
     ref = plain.linear(again.double().cpu(), w.double().cpu())
-    assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max())
+    for waves, max_splits in ((4, 4), (8, 4), (16, 4), (4, 1), (8, 2)):
+        prod = k.product_attention(parts[0], parts[1], w, max_splits=max_splits, waves=waves)
+        if prod is None:             # a long k range over too many heads
+            assert max_splits < 4
+            continue
+        assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, max_splits)
 
 
 def test_consumers_take_a_float32_product_of_many_rows(k):
