@@ -507,21 +507,46 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
     }
 }
 
+// What the fused variant of the decode kernel computes its queries (and the new token's key and value) from:
+// the QKV product as it comes out of the skinny product kernel, before bias, rotation and rounding.
+struct FusedQkv {
+    const float* prod;        // [in_splits][n_tokens][(nq + 2 nkv) * hd] float32 partial sums
+    int in_splits;
+    const float* row_ss;      // [ss_splits][n_tokens] sums of squares of the rows (1/rms still to apply), or null
+    int ss_splits;
+    float inv_hidden, eps;
+    const bf16_t* bias;       // [(nq + 2 nkv) * hd] or null
+    const int32_t* positions; // [n_tokens]
+    const float* inv_freq;    // [hd / 2]
+    const int32_t* slots;     // [n_tokens] page * page_size + offset of the token's key and value
+    bf16_t* k_cache_w;        // the caches again, writable
+    bf16_t* v_cache_w;
+};
+
 // Decoded tokens only (one query token per request, its heads of one kv group in one 16-row tile): a
 // workgroup of NW wavefronts shares one (request, kv head, key split); each wavefront walks its share of
 // the keys, PF blocks of 32 keys per round with all of the round's loads in flight together (the kernel is
 // a chain of round trips to memory, not of arithmetic), and the wavefronts' results are combined through
 // LDS.  With n_splits > 1 the combined, still unnormalised result goes to part_o / part_ml.
-template <int HD, int PF>
+//
+// FUSED: the kernel also does what the QKV epilogue kernel does for these tokens, which takes that kernel
+// out of the chain of a decode step.  Every workgroup adds up the product's partial sums for its query
+// heads, applies the rows' 1/rms, bias and rotation (same operations in the same order as
+// qkv_rope_store_kernel, so the same bits) and keeps the queries in LDS.  The workgroup whose key range ends
+// with the new token does the same for that token's key and value, writes them to the cache and, because
+// its own loads of that cache line may have been issued before, puts them into its operands itself.
+template <int HD, int PF, bool FUSED>
 __global__ __launch_bounds__(512) void attention_decode_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ kv_len, int n_tokens, int nq, int nkv, int page_size, float scale, int window,
-    int n_splits) {
+    int n_splits, FusedQkv f) {
     constexpr int KD = HD / 32, DT = HD / 16;
+    constexpr int kRow = HD + 2;
     extern __shared__ float wave_state[];          // [n_waves][16][HD + 2]: O, then maximum, then sum
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
+    const int lane = threadIdx.x % kWave, n_waves = blockDim.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // known to be the same for the wavefront
     const int lj = lane % 16, lg = lane / 16;
     const int b = blockIdx.x, kh = blockIdx.y, split = blockIdx.z;
     const int group_size = nq / nkv;
@@ -533,20 +558,98 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     const int width = (nq + 2 * nkv) * HD;
     const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
 
+    const int kb_begin = lo / 32, kb_end = p / 32 + 1;
+    const int per_split = (kb_end - kb_begin + n_splits - 1) / n_splits;
+    const int s_begin = kb_begin + split * per_split, s_end = min(kb_end, s_begin + per_split);
+    const int per_wave = (max(s_end - s_begin, 0) + n_waves - 1) / n_waves;
+    const int w_begin = s_begin + wave * per_wave, w_end = min(s_end, w_begin + per_wave);
+    // FUSED: does this workgroup's key range end with the new token?
+    const bool writer = FUSED && split == (kb_end - 1 - kb_begin) / per_split;
+    bf16_t* q_lds = reinterpret_cast<bf16_t*>(wave_state + n_waves * 16 * kRow);   // FUSED: [16][HD], then k, v [HD]
+    bf16_t* k_lds = q_lds + 16 * HD;
+    bf16_t* v_lds = k_lds + HD;
+
     bf16x8 q[KD];
-    {
+    if constexpr (!FUSED) {
         const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lg * 8;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
             const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
             q[kd] = __builtin_bit_cast(bf16x8, v);
         }
+    } else {
+        constexpr int half = HD / 2, INF = 8;
+        const float pos = static_cast<float>(f.positions[tok]);
+        float row_scale = 1.f;
+        if (f.row_ss) {
+            float ss = 0.f;
+            for (int s0 = 0; s0 < f.ss_splits; s0 += 16) {
+                float part[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) part[i] = f.row_ss[min(s0 + i, f.ss_splits - 1) * n_tokens + tok];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ss += s0 + i < f.ss_splits ? part[i] : 0.f;
+            }
+            row_scale = 1.0f / sqrtf(ss * f.inv_hidden + f.eps);
+        }
+        const long slot = f.slots[tok];
+        const long page = slot / page_size, off = slot % page_size;
+        const size_t stride = static_cast<size_t>(n_tokens) * width;
+        const int n_items = (group_size + (writer ? 2 : 0)) * half;      // pairs (i, i + half) of a head
+        for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+            const int h = it / half, i = it % half;
+            const int col = (h < group_size ? kh * group_size + h : h == group_size ? nq + kh : nq + nkv + kh) * HD + i;
+            const float* src = f.prod + static_cast<size_t>(tok) * width + col;
+            float x0 = 0.f, x1 = 0.f;
+            for (int s0 = 0; s0 < f.in_splits; s0 += INF) {
+                float ta[INF], tb[INF];
+#pragma unroll
+                for (int j = 0; j < INF; ++j) {
+                    const float* pj = src + min(s0 + j, f.in_splits - 1) * stride;
+                    ta[j] = pj[0];
+                    tb[j] = pj[half];
+                }
+#pragma unroll
+                for (int j = 0; j < INF; ++j) {
+                    if (s0 + j < f.in_splits) {
+                        x0 += ta[j];
+                        x1 += tb[j];
+                    }
+                }
+            }
+            x0 = x0 * row_scale + (f.bias ? to_float(f.bias[col]) : 0.f);
+            x1 = x1 * row_scale + (f.bias ? to_float(f.bias[col + half]) : 0.f);
+            if (h <= group_size) {                   // queries and the key are rotated, the value is not
+                float sn, cs;
+                sincosf(pos * f.inv_freq[i], &sn, &cs);
+                const float r0 = x0 * cs - x1 * sn, r1 = x0 * sn + x1 * cs;
+                x0 = r0;
+                x1 = r1;
+            }
+            const bf16_t y0 = from_float<bf16_t>(x0), y1 = from_float<bf16_t>(x1);
+            if (h < group_size) {
+                q_lds[h * HD + i] = y0;
+                q_lds[h * HD + i + half] = y1;
+            } else if (h == group_size) {            // keys: [page][kv head][offset][feature]
+                k_lds[i] = y0;
+                k_lds[i + half] = y1;
+                bf16_t* dst = f.k_cache_w + ((page * nkv + kh) * page_size + off) * HD;
+                dst[i] = y0;
+                dst[i + half] = y1;
+            } else {                                 // values: [page][kv head][feature][offset]
+                v_lds[i] = y0;
+                v_lds[i + half] = y1;
+                f.v_cache_w[((page * nkv + kh) * HD + i) * page_size + off] = y0;
+                f.v_cache_w[((page * nkv + kh) * HD + i + half) * page_size + off] = y1;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const uint4 v = valid ? *reinterpret_cast<const uint4*>(q_lds + lj * HD + kd * 32 + lg * 8) : uint4{0u, 0u, 0u, 0u};
+            q[kd] = __builtin_bit_cast(bf16x8, v);
+        }
     }
-    const int kb_begin = lo / 32, kb_end = p / 32 + 1;
-    const int per_split = (kb_end - kb_begin + n_splits - 1) / n_splits;
-    const int s_begin = kb_begin + split * per_split, s_end = min(kb_end, s_begin + per_split);
-    const int per_wave = (max(s_end - s_begin, 0) + n_waves - 1) / n_waves;
-    const int w_begin = s_begin + wave * per_wave, w_end = min(s_end, w_begin + per_wave);
 
     f32x4 o[DT];
 #pragma unroll
@@ -585,6 +688,34 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
                     vv[i][kt][d] = ok ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
                                       : uint2{0u, 0u};
             }
+        if constexpr (FUSED) {
+            // the new token's key and value come from LDS, not from the cache line that was just written
+            if (writer && kb0 <= kb_end - 1 && kb_end - 1 < min(w_end, kb0 + PF)) {
+                const int i_new = kb_end - 1 - kb0;
+#pragma unroll
+                for (int i = 0; i < PF; ++i) {
+                    if (i != i_new) continue;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt) {
+                        const int key0 = (kb0 + i) * 32 + kt * 16;
+                        if (key0 + lj == p) {
+#pragma unroll
+                            for (int kd = 0; kd < KD; ++kd)
+                                kk[i][kt][kd] = *reinterpret_cast<const uint4*>(k_lds + kd * 32 + lg * 8);
+                        }
+                        const int e = p - (key0 + lg * 4);          // which of this lane's four keys, if any
+                        if (e >= 0 && e < 4) {
+#pragma unroll
+                            for (int d = 0; d < DT; ++d) {
+                                const uint32_t nv = v_lds[d * 16 + lj].bits;
+                                uint32_t& word = (e < 2) ? vv[i][kt][d].x : vv[i][kt][d].y;
+                                word = (e & 1) ? ((word & 0x0000ffffu) | (nv << 16)) : ((word & 0xffff0000u) | nv);
+                            }
+                        }
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
             if (kb0 + i >= w_end) break;
@@ -636,7 +767,6 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     l += __shfl_xor(l, 32, kWave);
 
     // every wavefront leaves its state in LDS; then all threads combine
-    constexpr int kRow = HD + 2;
     float* mine = wave_state + (wave * 16 + lj) * kRow;
 #pragma unroll
     for (int d = 0; d < DT; ++d)
@@ -740,14 +870,22 @@ template <int HD>
 static int launch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                          const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size, float scale,
-                         int window, int n_splits, int n_waves, int combine, hipStream_t s) {
+                         int window, int n_splits, int n_waves, int combine, const FusedQkv* fused, hipStream_t s) {
     constexpr int PF = HD == 64 ? 4 : 2;
     dim3 grid(n_seqs, nkv, n_splits);
-    const size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
-    attention_decode_kernel<HD, PF><<<grid, n_waves * kWave, lds, s>>>(
-        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
-        static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
-        kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits);
+    size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
+    if (fused) lds += 18 * HD * sizeof(bf16_t);          // 16 query heads, the new key and value
+    if (lds > 64 * 1024) return EGPT_UNSUPPORTED_SIZE;
+    if (fused)
+        attention_decode_kernel<HD, PF, true><<<grid, n_waves * kWave, lds, s>>>(
+            nullptr, static_cast<bf16_t*>(out), part_o, part_ml, static_cast<const bf16_t*>(k_cache),
+            static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, kv_len, n_tokens, nq, nkv,
+            page_size, scale, window, n_splits, *fused);
+    else
+        attention_decode_kernel<HD, PF, false><<<grid, n_waves * kWave, lds, s>>>(
+            static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
+            static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
+            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, FusedQkv{});
     EGPT_CHECK_LAUNCH();
     if (n_splits > 1 && combine) {
         attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
@@ -836,9 +974,46 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
     if (hd == 64)
         return launch_decode<64>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start,
                                  kv_len, n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine,
-                                 s);
+                                 nullptr, s);
     return launch_decode<128>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, s);
+                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, nullptr, s);
+}
+
+// The same with the QKV epilogue folded in: the queries, and the new token's key and value, are computed from
+// the float32 QKV product (partial sums qkv_prod [in_splits][n_seqs][(nq + 2 nkv) * hd], the rows' sums of
+// squares row_ss [ss_splits][n_seqs] or null, bias or null), rotated over the whole head (inv_freq [hd / 2]) at
+// positions[t], and the key and value are stored at slots[t] of the caches.  Token t belongs to request t.
+extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const float* row_ss, int ss_splits,
+                                           int hidden, float eps, const void* bias, const int32_t* positions,
+                                           const float* inv_freq, const int32_t* slots, void* out, float* part_o,
+                                           float* part_ml, void* k_cache, void* v_cache, const int32_t* block_table,
+                                           int table_width, const int32_t* q_start, const int32_t* kv_len, int n_seqs,
+                                           int nq, int nkv, int hd, int page_size, float scale, int window,
+                                           int n_splits, int n_waves, int combine, void* stream) {
+    if (!qkv_prod || in_splits < 1 || !positions || !inv_freq || !slots || !out || !k_cache || !v_cache ||
+        !block_table || !q_start || !kv_len || (row_ss && (ss_splits < 1 || hidden < 1)))
+        return EGPT_BAD_ARGUMENT;
+    if (n_seqs <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 || n_splits < 1 ||
+        (n_splits > 1 && (!part_o || !part_ml)))
+        return EGPT_BAD_ARGUMENT;
+    if ((hd != 64 && hd != 128) || page_size % 16 != 0 || nq / nkv > 16 || nkv > 65535 || n_splits > 64 ||
+        n_waves < 1 || n_waves > 8)
+        return EGPT_UNSUPPORTED_SIZE;
+    FusedQkv f = {};
+    f.prod = qkv_prod; f.in_splits = in_splits;
+    f.row_ss = row_ss; f.ss_splits = row_ss ? ss_splits : 0;
+    f.inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
+    f.eps = eps;
+    f.bias = static_cast<const bf16_t*>(bias);
+    f.positions = positions; f.inv_freq = inv_freq; f.slots = slots;
+    f.k_cache_w = static_cast<bf16_t*>(k_cache); f.v_cache_w = static_cast<bf16_t*>(v_cache);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (hd == 64)
+        return launch_decode<64>(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start,
+                                 kv_len, n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine,
+                                 &f, s);
+    return launch_decode<128>(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
+                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, &f, s);
 }
 
 // bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.

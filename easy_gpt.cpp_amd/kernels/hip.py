@@ -53,6 +53,8 @@ class HipKernels:
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
             "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
+            "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
+                                            i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
@@ -356,15 +358,8 @@ class HipKernels:
             # matrix-core kernel; the key range is split when there are too few (request, kv head) pairs to fill
             # the GPU, which is the case when only decoded tokens are in the batch
             if max_q_len == 1 and t == b and nq // nkv <= 16:
-                # only decoded tokens: workgroups of four wavefronts per (request, kv head, key split); the key
-                # range is split over workgroups when the requests alone do not fill the GPU.  Parts that the
-                # output projection combines are read by every column of workgroups there, so they stay few.
-                # The kernel is a chain of round trips to memory: a wavefront takes one round per 4 (head size
-                # 64) or 2 key blocks of 32 keys, so the split aims at one round per wavefront.
-                key_blocks = -(-max_kv_len // 32)
-                per_round = 4 * (4 if hd == 64 else 2)
-                n_splits = max(1, min(-(-key_blocks // per_round), 8 if not combine else 16,
-                                      max(1, 2048 // (b * nkv))))
+                # only decoded tokens: workgroups of several wavefronts per (request, kv head, key split)
+                n_splits, n_waves = self._decode_shape(b, nkv, hd, max_kv_len, combine)
                 part_o = part_ml = None
                 if n_splits > 1:
                     part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)
@@ -372,7 +367,7 @@ class HipKernels:
                 self._run("egpt_paged_attention_decode", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
                           self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
                           q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale), int(window),
-                          n_splits, 4, 1 if combine else 0, self._stream())
+                          n_splits, n_waves, 1 if combine else 0, self._stream())
                 return (part_o, part_ml) if (n_splits > 1 and not combine) else None
             if max_q_len > 1 and page_size & (page_size - 1) == 0:
                 # prompt portions (and mixed batches): key/value tiles shared through LDS by the wavefronts of
@@ -404,6 +399,62 @@ class HipKernels:
         self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
                   nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())
+
+    @staticmethod
+    def _decode_shape(b, nkv, hd, max_kv_len, combine):
+        """(key splits, wavefronts per workgroup) of the decode attention kernel.  The kernel is a chain of round
+        trips to memory, and a wavefront takes one per round of 4 (head size 64) or 2 key blocks of 32 keys, so
+        there should be enough wavefronts for one round each, and with few requests for one key block each.
+        The key range is split over workgroups when the requests alone do not fill the GPU; parts that the
+        output projection combines are read by every column of workgroups there, so they stay few."""
+        key_blocks = -(-max_kv_len // 32)
+        pairs = b * nkv
+        n_waves = 8 if (hd == 64 and pairs * key_blocks <= 8192) else 4
+        per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (4 if hd == 64 else 2))
+        n_splits = max(1, min(-(-key_blocks // per_round), 8 if not combine else 16, max(1, 2048 // pairs)))
+        return n_splits, n_waves
+
+    def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
+                               k_cache, v_cache, block_table, q_start, kv_len, nq, nkv, hd, page_size, scale, window,
+                               max_kv_len, combine=True):
+        """Attention for a batch of single decoded tokens (token t belongs to request t) straight from the QKV
+        product's float32 partial sums prod [S, T, W]: what qkv_rope_store and paged_attention do together, in
+        one kernel.  Returns False if the case is not covered (nothing was done), else what paged_attention
+        returns."""
+        if prod.dim() != 3 or prod.dtype != _F32 or out.dtype != _BF16 or hd not in (64, 128) or page_size % 16:
+            return False
+        if rotary_dim != hd or nq // nkv > 16 or slots is None or inv_freq is None:
+            return False
+        in_splits, t, width = prod.shape
+        b, table_width = block_table.shape
+        if t != b or width != (nq + 2 * nkv) * hd:
+            return False
+        self._need(prod, "prod", _F32)
+        self._need(out, "out", _BF16, (t, nq * hd))
+        self._caches(k_cache, v_cache, _BF16, nkv, page_size, hd)
+        self._need(block_table, "block_table", _I32)
+        for name, v in (("q_start", q_start), ("kv_len", kv_len), ("positions", positions), ("slots", slots)):
+            self._need(v, name, _I32, (b,))
+        self._need(inv_freq, "inv_freq", _F32, (hd // 2,))
+        if bias is not None:
+            self._need(bias, "bias", _BF16, (width,))
+        ss_splits = 0
+        if row_ss is not None:
+            ss_splits = int(row_ss.shape[0])
+            self._need(row_ss, "row_ss", _F32, (ss_splits, t))
+        if max_kv_len > table_width * page_size:
+            raise ValueError(f"block table of width {table_width} cannot hold {max_kv_len} tokens at page size {page_size}")
+        n_splits, n_waves = self._decode_shape(b, nkv, hd, max_kv_len, combine)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=prod.device)
+            part_ml = torch.empty((n_splits, t, nq, 2), dtype=_F32, device=prod.device)
+        self._run("egpt_attention_decode_fused", prod.data_ptr(), int(in_splits), self._ptr(row_ss), ss_splits, int(hidden),
+                  float(eps), self._ptr(bias), positions.data_ptr(), inv_freq.data_ptr(), slots.data_ptr(), out.data_ptr(),
+                  self._ptr(part_o), self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                  table_width, q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale),
+                  int(window), n_splits, n_waves, 1 if combine else 0, self._stream())
+        return (part_o, part_ml) if (n_splits > 1 and not combine) else None
 
     def swiglu(self, gate_up, out):
         t, inter = out.shape

@@ -115,12 +115,42 @@ class GQAttention(Mixer):
         if prod is None:
             prod = k.product(x, self.w_qkv, unrounded=True)      # act [T, W], or float32 partial sums [S, T, W]
             dtype, device, t = x.dtype, x.device, x.shape[0]
-        qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=dtype, device=device)
         slots = cache.slots if cache.writes else None
         common = dict(
             k_cache=cache.k, v_cache=cache.v, nq=self.n_heads, nkv=self.n_kv_heads,
             hd=self.head_dim, page_size=cache.page_size,
         )
+        attn = torch.empty((t, self.q_size), dtype=dtype, device=device)
+        want_parts = self.b_o is None and hasattr(k, "product_attention") and t <= getattr(k, "fused_rows", 0)
+        # ---- single decoded tokens: bias, rotation, the store of the new key and value and the attention over
+        # the cache in one kernel, straight from the product's partial sums
+        parts = False
+        if (prod.dim() == 3 and rot is not None and slots is not None and ctx.max_q_len == 1
+                and hasattr(k, "attention_decode_fused")):
+            parts = k.attention_decode_fused(
+                prod, scale_args.get("row_ss"), scale_args.get("hidden", 0), scale_args.get("eps", 0.0), self.b_qkv,
+                ctx.positions, rot[0], rot[1], slots, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.kv_len,
+                self.n_heads, self.n_kv_heads, self.head_dim, cache.page_size, self.scale, self.window or 0,
+                ctx.max_kv_len, combine=not want_parts)
+        if parts is False:
+            parts = self._epilogue_and_attention(k, prod, t, width, dtype, device, rot, slots, common, scale_args, ctx,
+                                                 cache, attn, want_parts)
+        if parts is not None:
+            out = k.product_attention(parts[0], parts[1], self.w_o)
+            if out is not None:
+                return out
+            k.combine_attention(parts[0], parts[1], attn)
+        if self.b_o is None:
+            return k.product(attn, self.w_o)            # the residual add that follows sums partial sums up
+        out = torch.empty((t, self.hidden_size), dtype=dtype, device=device)
+        k.linear(attn, self.w_o, self.b_o, out)
+        return out
+
+    def _epilogue_and_attention(self, k, prod, t, width, dtype, device, rot, slots, common, scale_args, ctx, cache, attn,
+                                want_parts):
+        """Bias, position encoding and the store into the cache, then attention over the cache; returns what
+        paged_attention returns (the parts of a split key range, or None when `attn` is written)."""
+        qkv = prod if prod.dim() == 2 else torch.empty((t, width), dtype=dtype, device=device)
         if rot is not None:
             inv_freq, rotary_dim = rot
             k.qkv_rope_store(prod, self.b_qkv, ctx.positions, inv_freq, rotary_dim, slots, out=qkv, **common, **scale_args)
@@ -134,26 +164,14 @@ class GQAttention(Mixer):
             if slots is not None:
                 k.qkv_rope_store(qkv, None, ctx.positions, None, 0, slots, out=qkv, **common)
         # ---- attention over the cache.  If the kernel splits the keys, the output projection combines the parts.
-        attn = torch.empty((t, self.q_size), dtype=dtype, device=device)
-        want_parts = self.b_o is None and hasattr(k, "product_attention") and t <= getattr(k, "fused_rows", 0)
         args = dict(
             nq=self.n_heads, nkv=self.n_kv_heads, hd=self.head_dim, page_size=cache.page_size,
             scale=self.scale, window=self.window or 0, max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len,
         )
         if want_parts:
             args["combine"] = False
-        parts = k.paged_attention(qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
-                                  **args)
-        if parts is not None:
-            out = k.product_attention(parts[0], parts[1], self.w_o)
-            if out is not None:
-                return out
-            k.combine_attention(parts[0], parts[1], attn)
-        if self.b_o is None:
-            return k.product(attn, self.w_o)            # the residual add that follows sums partial sums up
-        out = torch.empty((t, self.hidden_size), dtype=dtype, device=device)
-        k.linear(attn, self.w_o, self.b_o, out)
-        return out
+        return k.paged_attention(qkv, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.q_len, ctx.kv_len,
+                                 **args)
 
 
 register_part("mixer", "gq_attention", GQAttention)

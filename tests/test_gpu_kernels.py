@@ -466,6 +466,47 @@ def test_paged_attention_decode_batches_split_the_key_range(k, nq, nkv, hd, batc
     assert run_paged(k, seqs, nq, nkv, hd, 16, torch.bfloat16, q_scale=6.0) <= 4e-2
 
 
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(14, 2, 64, 16), (12, 2, 128, 16), (3, 3, 64, 32), (16, 1, 64, 16)])
+@pytest.mark.parametrize("batch,ctx,window", [(8, 700, 0), (1, 2113, 0), (64, 130, 0), (3, 33, 0), (5, 1, 0), (8, 300, 100)])
+@pytest.mark.parametrize("with_scale,with_bias", [(True, True), (False, False)])
+def test_decode_attention_with_the_qkv_epilogue_folded_in(k, nq, nkv, hd, ps, batch, ctx, window, with_scale, with_bias):
+    # one kernel for bias + rotation + store + attention must leave the same bits, in its output and in the
+    # caches, as the two kernels it replaces (same operations in the same order), for every position of the new
+    # token in its page and key block
+    dtype = torch.bfloat16
+    seqs = [(1, max(1, ctx - 37 * i % ctx)) for i in range(batch)]
+    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed=11)
+    t, width = batch, (nq + 2 * nkv) * hd
+    kv_len = torch.tensor([kv for _, kv in seqs], dtype=torch.int32)
+    positions = (kv_len - 1).to(DEV)
+    slots = torch.stack([table[b, (int(kv_len[b]) - 1) // ps].cpu() * ps + (int(kv_len[b]) - 1) % ps for b in range(t)]).to(torch.int32).to(DEV)
+    prod = rnd(5, t, width, seed=12)
+    row_ss = (torch.rand(3, t, generator=torch.Generator().manual_seed(13)) * 30 + 1).to(DEV) if with_scale else None
+    bias = rnd(width, dtype=dtype, seed=14) if with_bias else None
+    inv_freq = torch.as_tensor(plain.rope_inv_freq(hd, 1e4), dtype=torch.float32).to(DEV)
+    q_start, q_len = torch.arange(t, dtype=torch.int32, device=DEV), torch.ones(t, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    for combine in (True, False):
+        kc1, vc1, kc2, vc2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+        qkv = torch.empty(t, width, dtype=dtype, device=DEV)
+        k.qkv_rope_store(prod, bias, positions, inv_freq, hd, slots, kc1, vc1, nq, nkv, hd, ps, out=qkv,
+                         row_ss=row_ss, hidden=96, eps=1e-5)
+        out1 = torch.zeros(t, nq * hd, dtype=dtype, device=DEV)
+        parts1 = k.paged_attention(qkv, out1, kc1, vc1, table, q_start, q_len, kv_len.to(DEV), nq, nkv, hd, ps, scale, window,
+                                   1, int(kv_len.max()), combine=combine)
+        out2 = torch.zeros(t, nq * hd, dtype=dtype, device=DEV)
+        parts2 = k.attention_decode_fused(prod, row_ss, 96, 1e-5, bias, positions, inv_freq, hd, slots, out2, kc2, vc2, table,
+                                          q_start, kv_len.to(DEV), nq, nkv, hd, ps, scale, window, int(kv_len.max()),
+                                          combine=combine)
+        assert parts2 is not False
+        assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+        assert (parts1 is None) == (parts2 is None)
+        if parts1 is None:
+            assert torch.equal(out1, out2)
+        else:
+            assert torch.equal(parts1[0], parts2[0]) and torch.equal(parts1[1], parts2[1])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_peaked_scores(k, dtype):
     # large queries make the softmax pick single keys, far ones included: a key skipped or read from the
