@@ -22,10 +22,14 @@ int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_ro
 int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype, void* stream);
 // qkv_out [n_tokens, (nq + 2 nkv) hd] of the activation type; may be qkv_in itself when n_splits == 0.
 // row_ss != null: the product still lacks each row's factor 1 / sqrt(sum_s row_ss[s][row] / hidden + eps).
+// cos_sin != null: the angles' cosines and sines from egpt_rope_table ([n_tokens][rotary_dim / 2][2]) instead of
+// computing them from positions and inv_freq.
 int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, int ss_splits, int hidden, float eps,
-                        void* qkv_out, const void* bias, const int32_t* positions,
-                        const float* inv_freq, int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache,
+                        void* qkv_out, const void* bias, const int32_t* positions, const float* inv_freq,
+                        const float* cos_sin, int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache,
                         int n_tokens, int nq, int nkv, int hd, int page_size, int dtype, void* stream);
+// cos_sin [n_tokens][half][2] = (cos, sin)(float(positions[t]) * inv_freq[i]) in float32: once per step for all layers.
+int egpt_rope_table(const int32_t* positions, const float* inv_freq, float* cos_sin, int n_tokens, int half, void* stream);
 // bfloat16 product for m <= 64 rows on the matrix cores, optionally split over k (see gemm_skinny.hip).
 // waves: wavefronts (of 16 columns of the result each) per workgroup, 4, 8 or 16; here and below.
 int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m, int n,
@@ -60,8 +64,8 @@ int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float
 // The same with the QKV epilogue (partial sums, 1/rms, bias, rotation, store of the new key and value) folded in;
 // token t belongs to request t; rotation over the whole head.
 int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const float* row_ss, int ss_splits, int hidden,
-                                float eps, const void* bias, const int32_t* positions, const float* inv_freq,
-                                const int32_t* slots, void* out, float* part_o, float* part_ml, void* k_cache,
+                                float eps, const void* bias, const float* cos_sin, const int32_t* slots, void* out,
+                                float* part_o, float* part_ml, void* k_cache,
                                 void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                                 const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
                                 int window, int n_splits, int n_waves, int combine, void* stream);

@@ -516,8 +516,7 @@ struct FusedQkv {
     int ss_splits;
     float inv_hidden, eps;
     const bf16_t* bias;       // [(nq + 2 nkv) * hd] or null
-    const int32_t* positions; // [n_tokens]
-    const float* inv_freq;    // [hd / 2]
+    const float* cos_sin;     // [n_tokens][hd / 2][2]: (cos, sin) of the tokens' rotation angles (egpt_rope_table)
     const int32_t* slots;     // [n_tokens] page * page_size + offset of the token's key and value
     bf16_t* k_cache_w;        // the caches again, writable
     bf16_t* v_cache_w;
@@ -569,97 +568,12 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     bf16_t* k_lds = q_lds + 16 * HD;
     bf16_t* v_lds = k_lds + HD;
 
-    bf16x8 q[KD];
-    if constexpr (!FUSED) {
-        const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lg * 8;
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) {
-            const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
-            q[kd] = __builtin_bit_cast(bf16x8, v);
-        }
-    } else {
-        constexpr int half = HD / 2, INF = 8;
-        const float pos = static_cast<float>(f.positions[tok]);
-        float row_scale = 1.f;
-        if (f.row_ss) {
-            float ss = 0.f;
-            for (int s0 = 0; s0 < f.ss_splits; s0 += 16) {
-                float part[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) part[i] = f.row_ss[min(s0 + i, f.ss_splits - 1) * n_tokens + tok];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) ss += s0 + i < f.ss_splits ? part[i] : 0.f;
-            }
-            row_scale = 1.0f / sqrtf(ss * f.inv_hidden + f.eps);
-        }
-        const long slot = f.slots[tok];
-        const long page = slot / page_size, off = slot % page_size;
-        const size_t stride = static_cast<size_t>(n_tokens) * width;
-        const int n_items = (group_size + (writer ? 2 : 0)) * half;      // pairs (i, i + half) of a head
-        for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
-            const int h = it / half, i = it % half;
-            const int col = (h < group_size ? kh * group_size + h : h == group_size ? nq + kh : nq + nkv + kh) * HD + i;
-            const float* src = f.prod + static_cast<size_t>(tok) * width + col;
-            float x0 = 0.f, x1 = 0.f;
-            for (int s0 = 0; s0 < f.in_splits; s0 += INF) {
-                float ta[INF], tb[INF];
-#pragma unroll
-                for (int j = 0; j < INF; ++j) {
-                    const float* pj = src + min(s0 + j, f.in_splits - 1) * stride;
-                    ta[j] = pj[0];
-                    tb[j] = pj[half];
-                }
-#pragma unroll
-                for (int j = 0; j < INF; ++j) {
-                    if (s0 + j < f.in_splits) {
-                        x0 += ta[j];
-                        x1 += tb[j];
-                    }
-                }
-            }
-            x0 = x0 * row_scale + (f.bias ? to_float(f.bias[col]) : 0.f);
-            x1 = x1 * row_scale + (f.bias ? to_float(f.bias[col + half]) : 0.f);
-            if (h <= group_size) {                   // queries and the key are rotated, the value is not
-                float sn, cs;
-                sincosf(pos * f.inv_freq[i], &sn, &cs);
-                const float r0 = x0 * cs - x1 * sn, r1 = x0 * sn + x1 * cs;
-                x0 = r0;
-                x1 = r1;
-            }
-            const bf16_t y0 = from_float<bf16_t>(x0), y1 = from_float<bf16_t>(x1);
-            if (h < group_size) {
-                q_lds[h * HD + i] = y0;
-                q_lds[h * HD + i + half] = y1;
-            } else if (h == group_size) {            // keys: [page][kv head][offset][feature]
-                k_lds[i] = y0;
-                k_lds[i + half] = y1;
-                bf16_t* dst = f.k_cache_w + ((page * nkv + kh) * page_size + off) * HD;
-                dst[i] = y0;
-                dst[i + half] = y1;
-            } else {                                 // values: [page][kv head][feature][offset]
-                v_lds[i] = y0;
-                v_lds[i + half] = y1;
-                f.v_cache_w[((page * nkv + kh) * HD + i) * page_size + off] = y0;
-                f.v_cache_w[((page * nkv + kh) * HD + i + half) * page_size + off] = y1;
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kd = 0; kd < KD; ++kd) {
-            const uint4 v = valid ? *reinterpret_cast<const uint4*>(q_lds + lj * HD + kd * 32 + lg * 8) : uint4{0u, 0u, 0u, 0u};
-            q[kd] = __builtin_bit_cast(bf16x8, v);
-        }
-    }
-
-    f32x4 o[DT];
-#pragma unroll
-    for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
-
-    for (int kb0 = w_begin; kb0 < w_end; kb0 += PF) {
-        uint4 kk[PF][2][KD];
-        uint2 vv[PF][2][DT];
-        // first all page numbers of the round (one wait for all of them), then all key and value loads
+    // One round of loads: PF blocks of 32 keys and their values for this wavefront, first all page numbers
+    // (one wait for all of them), then all key and value loads.  The first round is issued before anything
+    // else, so that the queries (a round trip of their own, two in the fused variant) arrive meanwhile.
+    uint4 kk[PF][2][KD];
+    uint2 vv[PF][2][DT];
+    auto load_round = [&](int kb0) {
         int pages[PF][2];
         bool live[PF][2];
 #pragma unroll
@@ -688,6 +602,143 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
                     vv[i][kt][d] = ok ? *reinterpret_cast<const uint2*>(vp + static_cast<long>(d) * 16 * page_size)
                                       : uint2{0u, 0u};
             }
+    };
+    // The queries.  Their loads are issued here, ahead of the first round of keys and values, and used behind
+    // it: loads are waited for in the order of their issue, so what the fused variant computes from its loads
+    // (which come from L2) is done while the keys and values (from HBM) are still on their way.
+    bf16x8 q[KD];
+    constexpr int half = HD / 2, INF = 8;
+    struct Item {
+        float ta[INF], tb[INF], b0, b1, cs, sn;
+    };
+    [[maybe_unused]] Item first;
+    [[maybe_unused]] float sst[16];
+    [[maybe_unused]] int slot_page = 0, slot_off = 0;
+    const int n_items = FUSED ? (group_size + (writer ? 2 : 0)) * half : 0;      // pairs (i, i + half) of a head
+    const size_t stride = static_cast<size_t>(n_tokens) * width;
+    auto item_col = [&](int it) {
+        const int h = it / half, i = it % half;
+        return (h < group_size ? kh * group_size + h : h == group_size ? nq + kh : nq + nkv + kh) * HD + i;
+    };
+    auto item_load = [&](int it, Item& r) {
+        const int h = it / half, i = it % half, col = item_col(it);
+        const float* src = f.prod + static_cast<size_t>(tok) * width + col;
+#pragma unroll
+        for (int j = 0; j < INF; ++j) {
+            const float* pj = src + min(j, f.in_splits - 1) * stride;
+            r.ta[j] = pj[0];
+            r.tb[j] = pj[half];
+        }
+        r.b0 = f.bias ? to_float(f.bias[col]) : 0.f;
+        r.b1 = f.bias ? to_float(f.bias[col + half]) : 0.f;
+        r.cs = 1.f;
+        r.sn = 0.f;
+        if (h <= group_size) {                   // queries and the key are rotated, the value is not
+            r.cs = f.cos_sin[(static_cast<size_t>(tok) * half + i) * 2];
+            r.sn = f.cos_sin[(static_cast<size_t>(tok) * half + i) * 2 + 1];
+        }
+    };
+    auto item_finish = [&](int it, const Item& r, float row_scale) {
+        const int h = it / half, i = it % half, col = item_col(it);
+        float x0 = 0.f, x1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < INF; ++j) {
+            if (j < f.in_splits) {
+                x0 += r.ta[j];
+                x1 += r.tb[j];
+            }
+        }
+        const float* src = f.prod + static_cast<size_t>(tok) * width + col;
+        for (int j = INF; j < f.in_splits; ++j) {          // more partial sums than one batch of loads: rare
+            x0 += src[j * stride];
+            x1 += src[j * stride + half];
+        }
+        x0 = scale_then_bias(x0, row_scale, r.b0);
+        x1 = scale_then_bias(x1, row_scale, r.b1);
+        if (h <= group_size) {
+            float r0, r1;
+            rotate_pair(x0, x1, r.cs, r.sn, r0, r1);
+            x0 = r0;
+            x1 = r1;
+        }
+        const bf16_t y0 = from_float<bf16_t>(x0), y1 = from_float<bf16_t>(x1);
+        const long page = slot_page, off = slot_off;
+        if (h < group_size) {
+            q_lds[h * HD + i] = y0;
+            q_lds[h * HD + i + half] = y1;
+        } else if (h == group_size) {            // keys: [page][kv head][offset][feature]
+            k_lds[i] = y0;
+            k_lds[i + half] = y1;
+            bf16_t* dst = f.k_cache_w + ((page * nkv + kh) * page_size + off) * HD;
+            dst[i] = y0;
+            dst[i + half] = y1;
+        } else {                                 // values: [page][kv head][feature][offset]
+            v_lds[i] = y0;
+            v_lds[i + half] = y1;
+            f.v_cache_w[((page * nkv + kh) * HD + i) * page_size + off] = y0;
+            f.v_cache_w[((page * nkv + kh) * HD + i + half) * page_size + off] = y1;
+        }
+    };
+    if constexpr (!FUSED) {
+        const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lg * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + kd * 32) : uint4{0u, 0u, 0u, 0u};
+            q[kd] = __builtin_bit_cast(bf16x8, v);
+        }
+    } else {
+        if (f.row_ss) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sst[i] = f.row_ss[min(i, f.ss_splits - 1) * n_tokens + tok];
+        }
+        const int slot = f.slots[tok];
+        slot_page = slot / page_size;
+        slot_off = slot % page_size;
+        if (static_cast<int>(threadIdx.x) < n_items) item_load(threadIdx.x, first);
+    }
+    auto make_q = [&]() {
+        if constexpr (FUSED) {
+            float row_scale = 1.f;
+            if (f.row_ss) {
+                float ss = 0.f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) ss += i < f.ss_splits ? sst[i] : 0.f;
+                for (int s0 = 16; s0 < f.ss_splits; s0 += 16) {
+                    float part[16];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) part[i] = f.row_ss[min(s0 + i, f.ss_splits - 1) * n_tokens + tok];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ss += s0 + i < f.ss_splits ? part[i] : 0.f;
+                }
+                row_scale = inv_rms(ss, f.inv_hidden, f.eps);
+            }
+            if (static_cast<int>(threadIdx.x) < n_items) item_finish(threadIdx.x, first, row_scale);
+            for (int it = threadIdx.x + blockDim.x; it < n_items; it += blockDim.x) {
+                Item r;
+                item_load(it, r);
+                item_finish(it, r, row_scale);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const uint4 v = valid ? *reinterpret_cast<const uint4*>(q_lds + lj * HD + kd * 32 + lg * 8)
+                                      : uint4{0u, 0u, 0u, 0u};
+                q[kd] = __builtin_bit_cast(bf16x8, v);
+            }
+        }
+    };
+
+    f32x4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // Every wavefront goes through the body at least once (one with no keys loads nothing and multiplies
+    // nothing): the fused variant's queries are made there, behind the first round's loads, with a barrier.
+    int kb0 = w_begin;
+    do {
+        load_round(kb0);
+        if (kb0 == w_begin) make_q();
         if constexpr (FUSED) {
             // the new token's key and value come from LDS, not from the cache line that was just written
             if (writer && kb0 <= kb_end - 1 && kb_end - 1 < min(w_end, kb0 + PF)) {
@@ -761,7 +812,8 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
                 o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), pb, acc, 0, 0, 0);
             }
         }
-    }
+        kb0 += PF;
+    } while (kb0 < w_end);
     float l = l_run;
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
@@ -981,16 +1033,17 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
 
 // The same with the QKV epilogue folded in: the queries, and the new token's key and value, are computed from
 // the float32 QKV product (partial sums qkv_prod [in_splits][n_seqs][(nq + 2 nkv) * hd], the rows' sums of
-// squares row_ss [ss_splits][n_seqs] or null, bias or null), rotated over the whole head (inv_freq [hd / 2]) at
-// positions[t], and the key and value are stored at slots[t] of the caches.  Token t belongs to request t.
+// squares row_ss [ss_splits][n_seqs] or null, bias or null), rotated over the whole head by the angles whose
+// cosines and sines are in cos_sin [n_seqs][hd / 2][2] (egpt_rope_table), and the key and value are stored at
+// slots[t] of the caches.  Token t belongs to request t.
 extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const float* row_ss, int ss_splits,
-                                           int hidden, float eps, const void* bias, const int32_t* positions,
-                                           const float* inv_freq, const int32_t* slots, void* out, float* part_o,
+                                           int hidden, float eps, const void* bias, const float* cos_sin,
+                                           const int32_t* slots, void* out, float* part_o,
                                            float* part_ml, void* k_cache, void* v_cache, const int32_t* block_table,
                                            int table_width, const int32_t* q_start, const int32_t* kv_len, int n_seqs,
                                            int nq, int nkv, int hd, int page_size, float scale, int window,
                                            int n_splits, int n_waves, int combine, void* stream) {
-    if (!qkv_prod || in_splits < 1 || !positions || !inv_freq || !slots || !out || !k_cache || !v_cache ||
+    if (!qkv_prod || in_splits < 1 || !cos_sin || !slots || !out || !k_cache || !v_cache ||
         !block_table || !q_start || !kv_len || (row_ss && (ss_splits < 1 || hidden < 1)))
         return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 || n_splits < 1 ||
@@ -1005,7 +1058,7 @@ extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits,
     f.inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
     f.eps = eps;
     f.bias = static_cast<const bf16_t*>(bias);
-    f.positions = positions; f.inv_freq = inv_freq; f.slots = slots;
+    f.cos_sin = cos_sin; f.slots = slots;
     f.k_cache_w = static_cast<bf16_t*>(k_cache); f.v_cache_w = static_cast<bf16_t*>(v_cache);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (hd == 64)

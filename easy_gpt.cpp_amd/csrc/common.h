@@ -30,6 +30,18 @@ __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
 
+// The QKV epilogue's arithmetic, spelled out operation by operation: several kernels do it (one by one, four
+// pairs at a time, inside the decode attention) and must leave the same bits, which they would not if the
+// compiler were free to contract each one's multiplications and additions in its own way.
+__device__ __forceinline__ float scale_then_bias(float x, float scale, float bias) { return __fmaf_rn(x, scale, bias); }
+__device__ __forceinline__ float inv_rms(float ss, float inv_hidden, float eps) {
+    return 1.0f / sqrtf(__fmaf_rn(ss, inv_hidden, eps));
+}
+__device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, float& ra, float& rb) {
+    ra = __fmaf_rn(a, c, -__fmul_rn(b, s));
+    rb = __fmaf_rn(a, s, __fmul_rn(b, c));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

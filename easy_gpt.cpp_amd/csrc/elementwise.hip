@@ -189,7 +189,8 @@ template <typename T>
 __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __restrict__ row_ss, int ss_splits,
                                       float inv_hidden, float eps, T* __restrict__ qkv_out, const T* __restrict__ bias,
                                       const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
-                                      int rotary_dim, const int32_t* __restrict__ slots, T* __restrict__ k_cache,
+                                      const float* __restrict__ cos_sin, int rotary_dim,
+                                      const int32_t* __restrict__ slots, T* __restrict__ k_cache,
                                       T* __restrict__ v_cache, int nq, int nkv, int hd, int page_size) {
     const int t = blockIdx.x;
     const int n_heads = nq + 2 * nkv;
@@ -210,7 +211,7 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __rest
 #pragma unroll
             for (int i = 0; i < 16; ++i) ss += part[i];
         }
-        row_scale = 1.0f / sqrtf(ss * inv_hidden + eps);
+        row_scale = inv_rms(ss, inv_hidden, eps);
     }
     long slot = slots ? slots[t] : -1;
     const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
@@ -218,13 +219,19 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __rest
         const int head = item / hd, d = item % hd;
         const bool rotated = head < nq + nkv && d < rotary_dim;
         if (rotated && d >= half) continue;  // done by its partner
-        float a = qkv_in.at(base + item) * row_scale + (bias ? to_float(bias[item]) : 0.f);
+        float a = scale_then_bias(qkv_in.at(base + item), row_scale, bias ? to_float(bias[item]) : 0.f);
         float b = 0.f;
         if (rotated) {
-            b = qkv_in.at(base + item + half) * row_scale + (bias ? to_float(bias[item + half]) : 0.f);
+            b = scale_then_bias(qkv_in.at(base + item + half), row_scale, bias ? to_float(bias[item + half]) : 0.f);
             float s, c;
-            sincosf(pos * inv_freq[d], &s, &c);
-            const float ra = a * c - b * s, rb = a * s + b * c;
+            if (cos_sin) {                       // the step's table of the same values
+                c = cos_sin[(static_cast<size_t>(t) * half + d) * 2];
+                s = cos_sin[(static_cast<size_t>(t) * half + d) * 2 + 1];
+            } else {
+                sincosf(pos * inv_freq[d], &s, &c);
+            }
+            float ra, rb;
+            rotate_pair(a, b, c, s, ra, rb);
             a = ra;
             b = rb;
         }
@@ -245,50 +252,92 @@ __global__ void qkv_rope_store_kernel(ProductView<T> qkv_in, const float* __rest
     }
 }
 
-// The same for many tokens (prompt portions), full rotation (rotary_dim == hd), one tensor in and out: a
-// thread owns one (token, pair index) and walks the heads, so the angle's sine and cosine are computed once
-// for all heads instead of once per head.
-template <typename T, typename IN>
-__global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const IN* __restrict__ qkv_in, T* __restrict__ qkv_out,
-                                                                  const T* __restrict__ bias,
-                                                                  const int32_t* __restrict__ positions,
-                                                                  const float* __restrict__ inv_freq,
-                                                                  const int32_t* __restrict__ slots,
-                                                                  T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                                  int n_tokens, int nq, int nkv, int hd, int page_size) {
-    const int half = hd / 2;
-    const int tokens_per_block = blockDim.x / half;
-    const int t = blockIdx.x * tokens_per_block + threadIdx.x / half;
-    const int i = threadIdx.x % half;
-    if (t >= n_tokens || static_cast<int>(threadIdx.x) >= tokens_per_block * half) return;
-    const int n_heads = nq + 2 * nkv;
-    const size_t base = static_cast<size_t>(t) * n_heads * hd;
+// cos_sin[t][i] = (cos, sin)(float(positions[t]) * inv_freq[i]): the angles of a step are the same in every
+// layer, so they are computed once per step and the layers' kernels read them.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float* __restrict__ cos_sin, int n_tokens, int half) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_tokens * half) return;
     float sn, cs;
-    sincosf(static_cast<float>(positions[t]) * inv_freq[i], &sn, &cs);
-    const long slot = slots ? slots[t] : -1;
-    const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
-    for (int head = 0; head < n_heads; ++head) {
-        const int lo = head * hd + i, hi = lo + half;
-        float a = to_float(qkv_in[base + lo]) + (bias ? to_float(bias[lo]) : 0.f);
-        float b = to_float(qkv_in[base + hi]) + (bias ? to_float(bias[hi]) : 0.f);
-        const bool is_v = head >= nq + nkv;
-        if (!is_v) {
-            const float ra = a * cs - b * sn, rb = a * sn + b * cs;
-            a = ra;
-            b = rb;
+    sincosf(static_cast<float>(positions[idx / half]) * inv_freq[idx % half], &sn, &cs);
+    cos_sin[2 * static_cast<size_t>(idx)] = cs;
+    cos_sin[2 * static_cast<size_t>(idx) + 1] = sn;
+}
+
+__device__ __forceinline__ void load4_as_float(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load4_as_float(const bf16_t* p, float* v) {
+    const uint2 a = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+}
+
+// The same for many tokens (prompt portions) in bfloat16, full rotation (rotary_dim == hd), one tensor in and
+// out, angles from the step's table: a thread owns four neighbouring pairs (i, i + hd/2) of one (token, head).
+template <typename IN>
+__global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const IN* __restrict__ qkv_in, bf16_t* __restrict__ qkv_out,
+                                                                  const bf16_t* __restrict__ bias,
+                                                                  const float* __restrict__ cos_sin,
+                                                                  const int32_t* __restrict__ slots,
+                                                                  bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+                                                                  int n_tokens, int nq, int nkv, int hd, int page_size) {
+    const int half = hd / 2, chunks = half / 4;
+    const int n_heads = nq + 2 * nkv;
+    const long idx = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<long>(n_tokens) * n_heads * chunks) return;
+    const int i = static_cast<int>(idx % chunks) * 4;
+    const int head = static_cast<int>((idx / chunks) % n_heads);
+    const int t = static_cast<int>(idx / (static_cast<long>(chunks) * n_heads));
+    const size_t lo = static_cast<size_t>(t) * n_heads * hd + head * hd + i, hi = lo + half;
+    float a[4], b[4];
+    load4_as_float(qkv_in + lo, a);
+    load4_as_float(qkv_in + hi, b);
+    if (bias) {
+        float ba[4], bb[4];
+        load4_as_float(bias + head * hd + i, ba);
+        load4_as_float(bias + head * hd + i + half, bb);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            a[j] = scale_then_bias(a[j], 1.f, ba[j]);
+            b[j] = scale_then_bias(b[j], 1.f, bb[j]);
         }
-        const T ta = from_float<T>(a), tb = from_float<T>(b);
-        qkv_out[base + lo] = ta;
-        qkv_out[base + hi] = tb;
-        if (slot >= 0 && head >= nq) {
-            if (!is_v) {
-                T* dst = k_cache + ((page * nkv + (head - nq)) * page_size + off) * hd;
-                dst[i] = ta;
-                dst[i + half] = tb;
-            } else {
-                T* dst = v_cache + ((page * nkv + (head - nq - nkv)) * hd) * page_size + off;
-                dst[static_cast<long>(i) * page_size] = ta;
-                dst[static_cast<long>(i + half) * page_size] = tb;
+    }
+    const bool is_v = head >= nq + nkv;
+    if (!is_v) {
+        float cs[8];
+        load4_as_float(cos_sin + (static_cast<size_t>(t) * half + i) * 2, cs);
+        load4_as_float(cos_sin + (static_cast<size_t>(t) * half + i) * 2 + 4, cs + 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float ra, rb;
+            rotate_pair(a[j], b[j], cs[2 * j], cs[2 * j + 1], ra, rb);
+            a[j] = ra;
+            b[j] = rb;
+        }
+    }
+    uint2 pa, pb;
+    pa.x = f32_to_bf16_bits(a[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(a[1])) << 16);
+    pa.y = f32_to_bf16_bits(a[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(a[3])) << 16);
+    pb.x = f32_to_bf16_bits(b[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(b[1])) << 16);
+    pb.y = f32_to_bf16_bits(b[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(b[3])) << 16);
+    *reinterpret_cast<uint2*>(qkv_out + lo) = pa;
+    *reinterpret_cast<uint2*>(qkv_out + hi) = pb;
+    const long slot = (slots && head >= nq) ? slots[t] : -1;
+    if (slot >= 0) {
+        const long page = slot / page_size, off = slot % page_size;
+        if (!is_v) {      // keys: [page][kv head][offset][feature]
+            bf16_t* dst = k_cache + ((page * nkv + (head - nq)) * page_size + off) * hd + i;
+            *reinterpret_cast<uint2*>(dst) = pa;
+            *reinterpret_cast<uint2*>(dst + half) = pb;
+        } else {          // values: [page][kv head][feature][offset]
+            bf16_t* dst = v_cache + ((page * nkv + (head - nq - nkv)) * hd + i) * page_size + off;
+            const uint32_t wa[2] = {pa.x, pa.y}, wb[2] = {pb.x, pb.y};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                dst[static_cast<long>(j) * page_size].bits = static_cast<uint16_t>(wa[j / 2] >> (16 * (j & 1)));
+                dst[static_cast<long>(j + half) * page_size].bits = static_cast<uint16_t>(wb[j / 2] >> (16 * (j & 1)));
             }
         }
     }
@@ -394,13 +443,13 @@ extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_t
 
 extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, int ss_splits, int hidden,
                                    float eps, void* qkv_out, const void* bias,
-                                   const int32_t* positions, const float* inv_freq, int rotary_dim,
-                                   const int32_t* slots, void* k_cache, void* v_cache, int n_tokens, int nq, int nkv,
-                                   int hd, int page_size, int dtype, void* stream) {
+                                   const int32_t* positions, const float* inv_freq, const float* cos_sin,
+                                   int rotary_dim, const int32_t* slots, void* k_cache, void* v_cache, int n_tokens,
+                                   int nq, int nkv, int hd, int page_size, int dtype, void* stream) {
     if (!qkv_in || !qkv_out || !positions || n_tokens < 0 || nq <= 0 || nkv <= 0 || hd <= 0 || page_size <= 0 ||
         n_splits < 0)
         return EGPT_BAD_ARGUMENT;
-    if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim % 2) != 0 || (rotary_dim > 0 && !inv_freq))
+    if (rotary_dim < 0 || rotary_dim > hd || (rotary_dim % 2) != 0 || (rotary_dim > 0 && !inv_freq && !cos_sin))
         return EGPT_BAD_ARGUMENT;
     if (slots && (!k_cache || !v_cache)) return EGPT_BAD_ARGUMENT;
     if (row_ss && (ss_splits < 1 || hidden < 1)) return EGPT_BAD_ARGUMENT;
@@ -408,23 +457,22 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float
     hipStream_t s = static_cast<hipStream_t>(stream);
     const float inv_hidden = row_ss ? 1.0f / static_cast<float>(hidden) : 0.f;
     const size_t stride = static_cast<size_t>(n_tokens) * (nq + 2 * nkv) * hd;
-    if (dtype == 1 && n_splits <= 1 && !row_ss && rotary_dim == hd && n_tokens >= 64 && hd <= 512) {
-        // many tokens: one thread per (token, pair), the angle shared by all heads.  (bfloat16 only: the
-        // float32 path keeps one kernel per operation whatever the batch, so that its results do not depend
-        // on the batch in any bit.)  The input is bfloat16, or one float32 "partial sum".
-        const int half = hd / 2;
-        const int tpb = 256 / half > 0 ? 256 / half : 1;
-        const int blocks = (n_tokens + tpb - 1) / tpb;
+    if (dtype == 1 && n_splits <= 1 && !row_ss && rotary_dim == hd && n_tokens >= 64 && hd % 8 == 0 && cos_sin) {
+        // many tokens: one thread per four pairs of a (token, head).  (bfloat16 only: the float32 path keeps
+        // one kernel per operation whatever the batch, so that its results do not depend on the batch in any
+        // bit.)  The input is bfloat16, or one float32 "partial sum".
+        const long items = static_cast<long>(n_tokens) * (nq + 2 * nkv) * (hd / 8);
+        const unsigned blocks = static_cast<unsigned>((items + 255) / 256);
         if (n_splits == 0)
-            qkv_rope_store_rows_kernel<bf16_t, bf16_t><<<blocks, 256, 0, s>>>(
+            qkv_rope_store_rows_kernel<bf16_t><<<blocks, 256, 0, s>>>(
                 static_cast<const bf16_t*>(qkv_in), static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias),
-                positions, inv_freq, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens,
-                nq, nkv, hd, page_size);
+                cos_sin, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens, nq, nkv, hd,
+                page_size);
         else
-            qkv_rope_store_rows_kernel<bf16_t, float><<<blocks, 256, 0, s>>>(
+            qkv_rope_store_rows_kernel<float><<<blocks, 256, 0, s>>>(
                 static_cast<const float*>(qkv_in), static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias),
-                positions, inv_freq, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens,
-                nq, nkv, hd, page_size);
+                cos_sin, slots, static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), n_tokens, nq, nkv, hd,
+                page_size);
         EGPT_CHECK_LAUNCH();
         return EGPT_OK;
     }
@@ -434,15 +482,28 @@ extern "C" int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float
         qkv_rope_store_kernel<float><<<grid, block, 0, s>>>(
             make_view<float>(qkv_in, n_splits, stride), row_ss, ss_splits, inv_hidden, eps,
             static_cast<float*>(qkv_out), static_cast<const float*>(bias),
-            positions, inv_freq, rotary_dim, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq,
+            positions, inv_freq, cos_sin, rotary_dim, slots, static_cast<float*>(k_cache), static_cast<float*>(v_cache), nq,
             nkv, hd, page_size);
     else if (dtype == 1)
         qkv_rope_store_kernel<bf16_t><<<grid, block, 0, s>>>(
             make_view<bf16_t>(qkv_in, n_splits, stride), row_ss, ss_splits, inv_hidden, eps,
-            static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias), positions, inv_freq, rotary_dim, slots, static_cast<bf16_t*>(k_cache),
+            static_cast<bf16_t*>(qkv_out), static_cast<const bf16_t*>(bias), positions, inv_freq, cos_sin, rotary_dim, slots,
+            static_cast<bf16_t*>(k_cache),
             static_cast<bf16_t*>(v_cache), nq, nkv, hd, page_size);
     else
         return EGPT_BAD_ARGUMENT;
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// cos_sin [n_tokens][half][2] = (cos, sin) of float(positions[t]) * inv_freq[i]
+extern "C" int egpt_rope_table(const int32_t* positions, const float* inv_freq, float* cos_sin, int n_tokens, int half,
+                               void* stream) {
+    if (!positions || !inv_freq || !cos_sin || n_tokens < 0 || half <= 0) return EGPT_BAD_ARGUMENT;
+    if (n_tokens == 0) return EGPT_OK;
+    const long items = static_cast<long>(n_tokens) * half;
+    rope_table_kernel<<<static_cast<unsigned>((items + 255) / 256), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        positions, inv_freq, cos_sin, n_tokens, half);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -457,4 +518,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 6; }
+extern "C" int egpt_abi_version(void) { return 7; }

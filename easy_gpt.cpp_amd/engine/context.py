@@ -46,6 +46,7 @@ class StepContext:
     state_storage: object = None
     cache_location: dict = field(default_factory=dict)
     group_windows: list = field(default_factory=list)
+    shared: dict = field(default_factory=dict)     # what parts of several layers compute once per step and share
 
     def cache_view(self, cache_id: int, writes: bool) -> CacheView:
         g, j = self.cache_location[cache_id]

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 6:
+    if lib.egpt_abi_version() != 7:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -46,14 +46,15 @@ class HipKernels:
             "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
             "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
             "egpt_swiglu": [vp, i, vp, i, i, i, vp],
-            "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
+            "egpt_rope_table": [vp, vp, vp, i, i, vp],
             "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
             "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
-            "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
+            "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
                                             i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
@@ -304,10 +305,21 @@ class HipKernels:
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
         return self.linear(x, w, None, out)
 
+    def rope_table(self, positions, inv_freq):
+        """float32 [T, half, 2]: (cos, sin) of float(positions[t]) * inv_freq[i].  A step's angles are the same in
+        every layer; the kernels that rotate take this table in place of computing the values again."""
+        t, half = positions.shape[0], inv_freq.shape[0]
+        self._need(positions, "positions", _I32, (t,))
+        self._need(inv_freq, "inv_freq", _F32, (half,))
+        out = torch.empty((t, half, 2), dtype=_F32, device=positions.device)
+        self._run("egpt_rope_table", positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), t, half, self._stream())
+        return out
+
     def qkv_rope_store(self, qkv, bias, positions, inv_freq, rotary_dim, slots, k_cache, v_cache, nq, nkv, hd,
-                       page_size, out=None, row_ss=None, hidden=0, eps=0.0):
+                       page_size, out=None, row_ss=None, hidden=0, eps=0.0, cos_sin=None):
         """qkv: act [T, W] or float32 partial sums [S, T, W]; out: act [T, W] (default: qkv itself, in place).
-        row_ss float32 [S2, T]: the product still lacks each row's factor 1/sqrt(sum_s row_ss[s] / hidden + eps)."""
+        row_ss float32 [S2, T]: the product still lacks each row's factor 1/sqrt(sum_s row_ss[s] / hidden + eps).
+        cos_sin: rope_table(positions, inv_freq), if the caller has it."""
         width = (nq + 2 * nkv) * hd
         t = qkv.shape[-2]
         if out is None:
@@ -331,9 +343,12 @@ class HipKernels:
         if row_ss is not None:
             ss_splits = int(row_ss.shape[0])
             self._need(row_ss, "row_ss", _F32, (ss_splits, t))
+        if cos_sin is not None:
+            self._need(cos_sin, "cos_sin", _F32, (t, rotary_dim // 2, 2))
         self._run("egpt_qkv_rope_store", qkv.data_ptr(), splits, self._ptr(row_ss), ss_splits, int(hidden), float(eps),
                   out.data_ptr(), self._ptr(bias), positions.data_ptr(),
-                  self._ptr(inv_freq) if rotary_dim else None, int(rotary_dim), self._ptr(slots),
+                  self._ptr(inv_freq) if rotary_dim else None, self._ptr(cos_sin) if rotary_dim else None,
+                  int(rotary_dim), self._ptr(slots),
                   self._ptr(k_cache), self._ptr(v_cache), t, nq, nkv, hd, page_size, dt, self._stream())
         return out
 
@@ -416,7 +431,7 @@ class HipKernels:
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
                                k_cache, v_cache, block_table, q_start, kv_len, nq, nkv, hd, page_size, scale, window,
-                               max_kv_len, combine=True):
+                               max_kv_len, combine=True, cos_sin=None):
         """Attention for a batch of single decoded tokens (token t belongs to request t) straight from the QKV
         product's float32 partial sums prod [S, T, W]: what qkv_rope_store and paged_attention do together, in
         one kernel.  Returns False if the case is not covered (nothing was done), else what paged_attention
@@ -436,6 +451,9 @@ class HipKernels:
         for name, v in (("q_start", q_start), ("kv_len", kv_len), ("positions", positions), ("slots", slots)):
             self._need(v, name, _I32, (b,))
         self._need(inv_freq, "inv_freq", _F32, (hd // 2,))
+        if cos_sin is None:
+            cos_sin = self.rope_table(positions, inv_freq)
+        self._need(cos_sin, "cos_sin", _F32, (t, hd // 2, 2))
         if bias is not None:
             self._need(bias, "bias", _BF16, (width,))
         ss_splits = 0
@@ -450,7 +468,7 @@ class HipKernels:
             part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=prod.device)
             part_ml = torch.empty((n_splits, t, nq, 2), dtype=_F32, device=prod.device)
         self._run("egpt_attention_decode_fused", prod.data_ptr(), int(in_splits), self._ptr(row_ss), ss_splits, int(hidden),
-                  float(eps), self._ptr(bias), positions.data_ptr(), inv_freq.data_ptr(), slots.data_ptr(), out.data_ptr(),
+                  float(eps), self._ptr(bias), cos_sin.data_ptr(), slots.data_ptr(), out.data_ptr(),
                   self._ptr(part_o), self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
                   table_width, q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale),
                   int(window), n_splits, n_waves, 1 if combine else 0, self._stream())

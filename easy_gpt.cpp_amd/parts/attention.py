@@ -125,14 +125,17 @@ class GQAttention(Mixer):
         # ---- single decoded tokens: bias, rotation, the store of the new key and value and the attention over
         # the cache in one kernel, straight from the product's partial sums
         parts = False
+        cos_sin = self.position.table(ctx) if (rot is not None and hasattr(self.position, "table")) else None
         if (prod.dim() == 3 and rot is not None and slots is not None and ctx.max_q_len == 1
                 and hasattr(k, "attention_decode_fused")):
             parts = k.attention_decode_fused(
                 prod, scale_args.get("row_ss"), scale_args.get("hidden", 0), scale_args.get("eps", 0.0), self.b_qkv,
                 ctx.positions, rot[0], rot[1], slots, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.kv_len,
                 self.n_heads, self.n_kv_heads, self.head_dim, cache.page_size, self.scale, self.window or 0,
-                ctx.max_kv_len, combine=not want_parts)
+                ctx.max_kv_len, combine=not want_parts, cos_sin=cos_sin)
         if parts is False:
+            if cos_sin is not None:
+                scale_args = dict(scale_args, cos_sin=cos_sin)
             parts = self._epilogue_and_attention(k, prod, t, width, dtype, device, rot, slots, common, scale_args, ctx,
                                                  cache, attn, want_parts)
         if parts is not None:

@@ -116,6 +116,8 @@ class Model:
     # ------------------------------------------------------------------ one step
     def forward(self, ctx) -> torch.Tensor | None:
         """Run the step described by `ctx`; returns float32 logits [rows, V] or None if no row is wanted."""
+        if hasattr(ctx, "shared"):
+            ctx.shared.clear()                       # per-step values that layers share are made anew every step
         h = self.embedding.forward(ctx.token_ids)
         delta = None
         for run in self.spec.run_order:

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import torch
 
+from .. import kernels
 from .base import PositionEncoding, register_part
 
 
@@ -40,6 +41,20 @@ class RotaryHalfSplit(PositionEncoding):
         if key not in self._inv_freq:
             self._inv_freq[key] = self.inv_freq_host().to(device)
         return self._inv_freq[key], self.rotary_dim
+
+    def table(self, ctx):
+        """The step's cosines and sines [T, rotary_dim / 2, 2], computed by the first layer that asks and
+        shared by the others (the angles depend on the positions only); None if the backend has no such kernel."""
+        k = kernels.backend()
+        shared = getattr(ctx, "shared", None)
+        if shared is None or not hasattr(k, "rope_table"):
+            return None
+        key = ("rope_table", self.theta, self.rotary_dim)
+        tab = shared.get(key)
+        if tab is None:
+            inv_freq, _ = self.rotary(ctx.positions.device)
+            tab = shared[key] = k.rope_table(ctx.positions, inv_freq)
+        return tab
 
 
 class NoPosition(PositionEncoding):

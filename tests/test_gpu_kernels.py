@@ -278,7 +278,7 @@ def test_consumers_take_a_float32_product_of_many_rows(k):
     kc = torch.zeros(6, nkv, ps, hd, dtype=dtype, device=DEV)
     vc = torch.zeros(6, nkv, hd, ps, dtype=dtype, device=DEV)
     got = torch.empty(t, width, dtype=dtype, device=DEV)
-    k.qkv_rope_store(qp, bias, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=got)
+    k.qkv_rope_store(qp, bias, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=got, cos_sin=k.rope_table(positions, inv))
     x = (qp[0].double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
     refq = x.clone()
     refq[:, : nq + nkv] = plain.rope(x[:, : nq + nkv], positions.cpu(), 1e6)
@@ -287,6 +287,32 @@ def test_consumers_take_a_float32_product_of_many_rows(k):
         pg, off = int(slots[i]) // ps, int(slots[i]) % ps
         assert torch.equal(kc[pg, :, off, :], got.view(t, -1, hd)[i, nq : nq + nkv])
         assert torch.equal(vc[pg, :, :, off], got.view(t, -1, hd)[i, nq + nkv :])
+
+
+def test_rope_table_holds_what_the_kernels_compute(k):
+    # the step's table of cosines and sines against float64, and: a kernel that takes the table leaves the same
+    # bits as one that computes the angles itself
+    hd, nq, nkv, ps, t = 64, 3, 1, 16, 9
+    positions = torch.tensor([0, 1, 2, 17, 255, 4095, 32767, 100000, 5], dtype=torch.int32, device=DEV)
+    inv = plain.rope_inv_freq(hd, 1e6).to(DEV)
+    tab = k.rope_table(positions, inv)
+    ang = (positions.cpu().float()[:, None] * inv.cpu()[None, :]).double()       # the float32 product, as the reference forms it
+    assert tab.shape == (t, hd // 2, 2)
+    assert float((tab[..., 0].double().cpu() - torch.cos(ang)).abs().max()) <= 2e-7
+    assert float((tab[..., 1].double().cpu() - torch.sin(ang)).abs().max()) <= 2e-7
+    width = (nq + 2 * nkv) * hd
+    for dtype in DTYPES:
+        qkv = rnd(t, width, dtype=dtype, seed=1)
+        slots = torch.arange(t, dtype=torch.int32, device=DEV)
+        outs = []
+        for cs in (None, tab):
+            kc = torch.zeros(1, nkv, ps, hd, dtype=dtype, device=DEV)
+            vc = torch.zeros(1, nkv, hd, ps, dtype=dtype, device=DEV)
+            out = torch.empty_like(qkv)
+            k.qkv_rope_store(qkv, None, positions, inv, hd, slots, kc, vc, nq, nkv, hd, ps, out=out, cos_sin=cs)
+            outs.append((out, kc, vc))
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
 
 
 def test_linear_vector_of_the_reference(k):
@@ -317,8 +343,9 @@ def test_swiglu(k, dtype, inter):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("t", [11, 77])
+@pytest.mark.parametrize("table", [False, True])         # angles computed in the kernel, or taken from the step's table
 @pytest.mark.parametrize("nq,nkv,hd,rd,theta", [(6, 3, 48, 48, 1e4), (5, 1, 80, 80, 1e6), (4, 4, 32, 16, 5e5), (14, 2, 64, 64, 1e6)])
-def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta, t):
+def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta, t, table):
     ps, pages = 4, 9 if t == 11 else 30
     qkv = rnd(t, (nq + 2 * nkv) * hd, dtype=dtype, seed=1)
     bias = rnd((nq + 2 * nkv) * hd, dtype=dtype, seed=2)
@@ -330,7 +357,8 @@ def test_qkv_rope_store(k, dtype, nq, nkv, hd, rd, theta, t):
     kc = torch.full((pages, nkv, ps, hd), 77.0, dtype=dtype, device=DEV)
     vc = torch.full((pages, nkv, hd, ps), 77.0, dtype=dtype, device=DEV)
     x = (qkv.double() + bias.double()).cpu().view(t, nq + 2 * nkv, hd)
-    k.qkv_rope_store(qkv, bias, positions, inv, rd, slots, kc, vc, nq, nkv, hd, ps)
+    k.qkv_rope_store(qkv, bias, positions, inv, rd, slots, kc, vc, nq, nkv, hd, ps,
+                     cos_sin=k.rope_table(positions, inv) if table else None)
     ang = (positions.cpu().float()[:, None] * inv.cpu()[None, :]).double()
     cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     ref = x.clone()
@@ -497,7 +525,7 @@ def test_decode_attention_with_the_qkv_epilogue_folded_in(k, nq, nkv, hd, ps, ba
         out2 = torch.zeros(t, nq * hd, dtype=dtype, device=DEV)
         parts2 = k.attention_decode_fused(prod, row_ss, 96, 1e-5, bias, positions, inv_freq, hd, slots, out2, kc2, vc2, table,
                                           q_start, kv_len.to(DEV), nq, nkv, hd, ps, scale, window, int(kv_len.max()),
-                                          combine=combine)
+                                          combine=combine, cos_sin=k.rope_table(positions, inv_freq) if combine else None)
         assert parts2 is not False
         assert torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
         assert (parts1 is None) == (parts2 is None)
