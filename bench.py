@@ -35,13 +35,24 @@ NEW_TOKENS = 128
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 
+# The other layer sizes of the baseline record, for --shape (the default run and its record stay the 0.5B ones):
+# (config changes, layers of the model, prefix length of the decode runs)
+OTHER_SHAPES = {
+    "1.5b": (dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+                  vocab_size=151936, tie_word_embeddings=True), 28, 2048),
+    "7b": (dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
+                vocab_size=152064, tie_word_embeddings=False), 28, 4096),
+}
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=NEW_TOKENS - 16)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--shape", default="0.5b", choices=["0.5b"] + sorted(OTHER_SHAPES),
+                    help="layer sizes: Qwen2.5-0.5B (the record's) or another size of the baseline record")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
@@ -50,6 +61,15 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
         return 2
+    global FULL_LAYERS, PREFIX, CONTEXT
+    base, name = dict(QWEN25_05B), "Qwen2.5-0.5B"
+    if args.shape != "0.5b":
+        changes, FULL_LAYERS, PREFIX = OTHER_SHAPES[args.shape]
+        base.update(changes)
+        CONTEXT = PREFIX + 2048
+        name = f"Qwen2.5-{args.shape.upper()}"
+    if args.layers is None:
+        args.layers = FULL_LAYERS
     if args.warmup + args.steps > CONTEXT - PREFIX:
         print(f"--warmup + --steps must stay within the context of {CONTEXT} after a prefix of {PREFIX}")
         return 2
@@ -60,7 +80,7 @@ def main() -> int:
     from easy_gpt.cpp_amd.sampling import Sampler, SamplingParams
     from easy_gpt.cpp_amd.weights import write_random_model
 
-    cfg = dict(QWEN25_05B, num_hidden_layers=args.layers)
+    cfg = dict(base, num_hidden_layers=args.layers)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     elem = 2 if args.dtype == "bfloat16" else 4
     h, nq, nkv, inter, vocab = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
@@ -116,7 +136,7 @@ def main() -> int:
                    "frac": round(prefill_flops(PREFILL_TOKENS) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     if args.prefill_only:
-        print(json.dumps({"metric": "prefill tok/s at 2,048 tokens (Qwen2.5-0.5B)", "prefill": prefill}), flush=True)
+        print(json.dumps({"metric": f"prefill tok/s at 2,048 tokens ({name})", "prefill": prefill}), flush=True)
         return 0
 
     # ---------------------------------------------------------------- decoding at each batch size
@@ -158,8 +178,7 @@ def main() -> int:
     sec, step_bytes = results[args.batch]
     achieved = step_bytes / (sec / args.steps) / 1e9
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen2.5-0.5B, prefix 2048)" if args.batch == 8
-        else f"decode tok/s at batch {args.batch} (Qwen2.5-0.5B, prefix 2048)",
+        "metric": f"decode tok/s at batch {args.batch} ({name}, prefix {PREFIX})",
         "value": round(args.batch * args.steps / sec, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -172,8 +191,8 @@ def main() -> int:
         "dtype": dtype_key,
         "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
         "config": {
-            "model": "Qwen2.5-0.5B layer sizes", "layers": layers, "layers_of_model": FULL_LAYERS, "hidden": h,
-            "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": True,
+            "model": f"{name} layer sizes", "layers": layers, "layers_of_model": FULL_LAYERS, "hidden": h,
+            "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]),
             "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": NEW_TOKENS,
             "page_size": page_size, "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
             "sampling": "greedy", "parallelism": "single GPU",

@@ -190,7 +190,9 @@ class HipKernels:
         bounded so that the partial sums stay smaller than the weights they came from."""
         steps = -(-k // 128)
         n_blocks = -(-n // 64)
-        s = min(steps, max(1, 1024 // n_blocks), max(1, k // (2 * m)), 20)
+        # a long k range is worth more workgroups: each one's stream is a chain of steps, one load ahead
+        most = 2048 if steps >= 14 else 1024
+        s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20)
         per = -(-steps // s)
         return -(-steps // per)
 
@@ -426,7 +428,11 @@ class HipKernels:
         pairs = b * nkv
         n_waves = 8 if (hd == 64 and pairs * key_blocks <= 8192) else 4
         per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (4 if hd == 64 else 2))
-        n_splits = max(1, min(-(-key_blocks // per_round), 8 if not combine else 16, max(1, 2048 // pairs)))
+        wanted = -(-key_blocks // per_round)
+        # the output projection combines up to 8 parts in registers; more only for few requests with contexts
+        # so long that 8 parts would leave every wavefront four rounds or more
+        most = 16 if (combine or (pairs <= 8 and wanted >= 32)) else 8
+        n_splits = max(1, min(wanted, most, max(1, 2048 // pairs)))
         return n_splits, n_waves
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
