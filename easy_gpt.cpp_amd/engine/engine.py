@@ -265,10 +265,13 @@ class Engine:
             while w < need:
                 w *= 2
             widths.append(w)
-        key = (b, tuple(widths))
+        # The kernels choose their shape (key splits of the attention) by the longest context, and a graph holds
+        # one choice: contexts are bucketed in steps of 512 tokens beside the table widths.
+        kv_bound = -(-(max(rc.num_tokens for rc in rcs) + 1) // 512) * 512
+        key = (b, tuple(widths), kv_bound)
         plan = self._decode_plans.get(key)
         if plan is None:
-            plan = self._decode_plans[key] = _DecodePlan(self, b, widths)
+            plan = self._decode_plans[key] = _DecodePlan(self, b, widths, kv_bound)
         plan.fill(rcs, tokens)
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
@@ -290,7 +293,7 @@ class Engine:
 class _DecodePlan:
     """Static device buffers, a host mirror and the captured graph of one decode batch shape."""
 
-    def __init__(self, engine: Engine, batch: int, widths: list[int]):
+    def __init__(self, engine: Engine, batch: int, widths: list[int], kv_bound: int):
         self.batch, self.widths = batch, list(widths)
         dev = engine.device
         n_groups = len(widths)
@@ -317,7 +320,7 @@ class _DecodePlan:
         ps = engine.page_size
         self.ctx = StepContext(
             num_tokens=b, num_seqs=b, token_ids=v(0), positions=v(1), q_start=v(2), q_len=v(3), kv_len=v(4),
-            want_rows=v(6), max_q_len=1, max_kv_len=min(w * ps for w in widths) if widths else 1,
+            want_rows=v(6), max_q_len=1, max_kv_len=min([kv_bound] + [w * ps for w in widths]),
             q_start_host=list(range(b)), q_len_host=[1] * b, kv_len_host=[0] * b,
             state_slots=v(5), state_slots_host=[0] * b, groups=groups, page_size=ps, kv_storage=engine.kv,
             state_storage=engine.states, cache_location=engine.model.cache_location,
