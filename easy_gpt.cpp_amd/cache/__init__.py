@@ -1,7 +1,5 @@
 from .manager import CacheManager, RequestCache
-from .pages import NoFreeSlot, OutOfPages, PagePool, SlotPool
+from .pages import NoFreeSlot, OutOfPages
 from .storage import KVStorage, StateStorage
 
-__all__ = [
-    "CacheManager", "KVStorage", "NoFreeSlot", "OutOfPages", "PagePool", "RequestCache", "SlotPool", "StateStorage",
-]
+__all__ = ["CacheManager", "KVStorage", "NoFreeSlot", "OutOfPages", "RequestCache", "StateStorage"]

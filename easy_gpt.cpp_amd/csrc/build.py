@@ -1,6 +1,8 @@
-"""Builds the gfx950 kernel library from the .hip sources in this folder with hipcc.
+"""Builds the native libraries: the gfx950 kernel library from the .hip sources in this folder
+with hipcc, and the host library (cache bookkeeping, step metadata) from host/*.cpp with the host
+compiler.
 
-The library is kept beside the sources when that folder is writable (so a built tree can be
+A library is kept beside the sources when that folder is writable (so a built tree can be
 copied to a GPU machine), else in a per-user cache folder.  A stamp file records the hash of
 the sources and flags it was built from; `ensure_built` rebuilds when they differ.
 """
@@ -22,6 +24,12 @@ ARCH = "gfx950"
 # packed-fp32 instructions are kept out of the generated code on purpose
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+HOST_SOURCES = ["host/cache_core.cpp"]
+HOST_HEADERS = ["host/cache_core.h"]
+HOST_LIB_NAME = "libeasygpt_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra"]
 
 
 class BuildError(RuntimeError):
@@ -135,5 +143,59 @@ def ensure_built(verbose: bool = True) -> str:
     return build(verbose)
 
 
+# ---------------------------------------------------------------------------------- the host library
+def _host_compiler() -> str | None:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/llvm/bin/clang++"):
+        if cand and (os.path.isfile(cand) or shutil.which(cand)):
+            return cand
+    return None
+
+
+def host_source_hash() -> str:
+    h = hashlib.sha256()
+    for name in HOST_SOURCES + HOST_HEADERS:
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(name.encode())
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:24]
+
+
+def _host_paths():
+    d = lib_dir()
+    return os.path.join(d, HOST_LIB_NAME), os.path.join(d, "libeasygpt_host.stamp")
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host library.  Always compiles."""
+    cxx = _host_compiler()
+    if cxx is None:
+        raise BuildError("no C++ compiler found (looked at $CXX, g++, c++, clang++)")
+    lib, stamp = _host_paths()
+    tmp_lib = lib + f".tmp{os.getpid()}"
+    t0 = time.time()
+    cmd = [cxx, *HOST_FLAGS, "-I", os.path.join(HERE, "host"), *[os.path.join(HERE, s) for s in HOST_SOURCES], "-o", tmp_lib]
+    _log("compiling " + ", ".join(HOST_SOURCES), verbose)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise BuildError(f"{cxx} failed:\n{r.stdout}")
+    os.replace(tmp_lib, lib)
+    with open(stamp, "w") as f:
+        f.write(host_source_hash())
+    _log(f"built {lib} in {time.time() - t0:.1f} s", verbose)
+    return lib
+
+
+def ensure_host_built(verbose: bool = True) -> str:
+    lib, stamp = _host_paths()
+    if os.path.isfile(lib) and os.path.isfile(stamp):
+        with open(stamp) as f:
+            if f.read().strip() == host_source_hash():
+                return lib
+    return build_host(verbose)
+
+
 if __name__ == "__main__":
+    print(build_host())
     print(build())

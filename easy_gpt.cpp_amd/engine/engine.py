@@ -17,6 +17,7 @@ from typing import Sequence
 import numpy as np
 import torch
 
+from ..cache.manager import _ints
 from ..cache import CacheManager, KVStorage, OutOfPages, RequestCache, StateStorage
 from ..config.registry import load_model_config
 from ..parts.model import Model, build_model
@@ -122,11 +123,11 @@ class Engine:
         if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
             return self._step_decode(entries)
         rcs = self._check(entries)
-        self._reserve_all(rcs, entries)
+        counts = [len(e.tokens) for e in entries]
+        self.cache.reserve_step(rcs, counts)               # all of the step's pages or none
         ctx = self._build_context(rcs, entries)
         logits = self.model.forward(ctx)
-        for rc, e in zip(rcs, entries):
-            self.cache.commit(rc, len(e.tokens))
+        self.cache.commit_step(rcs, counts)
         return logits
 
     def _check(self, entries) -> list[RequestCache]:
@@ -153,20 +154,6 @@ class Engine:
             rcs.append(rc)
         return rcs
 
-    def _reserve_all(self, rcs, entries) -> None:
-        before = [[len(t) for t in rc.tables] for rc in rcs]
-        try:
-            for rc, e in zip(rcs, entries):
-                self.cache.reserve(rc, len(e.tokens))
-        except OutOfPages:
-            for rc, lens in zip(rcs, before):       # give back what this step took
-                for pool, table, n in zip(self.cache.pools, rc.tables, lens):
-                    extra = [p for p in table[n:] if p >= 0]
-                    if extra:
-                        pool.give_back(extra)
-                    del table[n:]
-            raise
-
     def _build_context(self, rcs, entries) -> StepContext:
         ps = self.page_size
         n_groups = len(self.cache.groups)
@@ -177,39 +164,30 @@ class Engine:
             q_start[i] = q_start[i - 1] + q_len[i - 1]
         t = q_start[-1] + q_len[-1]
         kv_len = [rc.num_tokens + n for rc, n in zip(rcs, q_len)]
-        token_ids = np.empty(t, dtype=np.int32)
-        positions = np.empty(t, dtype=np.int32)
-        slots = np.empty((max(n_groups, 1), t), dtype=np.int32)
-        widths = [max((len(rc.tables[g]) for rc in rcs), default=1) or 1 for g in range(n_groups)]
-        tables = [np.full((b, widths[g]), -1, dtype=np.int32) for g in range(n_groups)]
+        widths = [max(max(rc.table_lens[g] for rc in rcs), 1) for g in range(n_groups)]
         want_rows: list[int] = []
-        for i, (rc, e) in enumerate(zip(rcs, entries)):
-            s, n = q_start[i], q_len[i]
-            token_ids[s : s + n] = np.asarray(e.tokens, dtype=np.int64)
-            pos = np.arange(rc.num_tokens, rc.num_tokens + n, dtype=np.int64)
-            positions[s : s + n] = pos
-            for g in range(n_groups):
-                tab = np.asarray(rc.tables[g], dtype=np.int64)
-                tables[g][i, : len(tab)] = tab
-                pages = tab[pos // ps]
-                if (pages < 0).any():
-                    raise RuntimeError("a token of this step would be stored in a page that was given back")
-                slots[g, s : s + n] = pages * ps + pos % ps
-            want_rows.extend(s + int(w) for w in e.want)
-        # one packed upload for everything
-        parts = [token_ids, positions, np.asarray(q_start, np.int32), np.asarray(q_len, np.int32),
-                 np.asarray(kv_len, np.int32), np.asarray([rc.slot for rc in rcs], np.int32),
-                 np.asarray(want_rows, np.int32)]
-        parts += [slots[g] for g in range(n_groups)] + [tables[g].reshape(-1) for g in range(n_groups)]
-        sizes = [p.size for p in parts]
-        packed = torch.from_numpy(np.concatenate([p.reshape(-1) for p in parts]).astype(np.int32, copy=False))
-        if self.device.type == "cuda":
-            packed = packed.pin_memory()
-        dev = packed.to(self.device, non_blocking=True)
-        views, off = [], 0
+        for s0, e in zip(q_start, entries):
+            want_rows.extend(s0 + int(w) for w in e.want)
+        # One packed int32 buffer for everything, filled in place (token ids and wanted rows here, the rest
+        # by the cache manager's library) and uploaded with one copy:
+        # token ids, positions [t each]; q_start, q_len, kv_len, state slots [b each]; wanted rows;
+        # slots [t per group]; block tables [b x width per group]
+        sizes = [t, t, b, b, b, b, len(want_rows)] + [t] * n_groups + [b * widths[g] for g in range(n_groups)]
+        offsets = [0]
         for n in sizes:
-            views.append(dev[off : off + n])
-            off += n
+            offsets.append(offsets[-1] + n)
+        packed = torch.empty(offsets[-1], dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        host = packed.numpy()
+        host[0:t] = np.fromiter((tok for e in entries for tok in e.tokens), dtype=np.int64, count=t)
+        host[offsets[6] : offsets[7]] = want_rows
+        base = packed.data_ptr()
+        ptr = lambda i: base + 4 * offsets[i]
+        self.cache.fill_step(
+            _ints([rc.handle for rc in rcs]), _ints(q_len), _ints(widths),
+            (ptr(1), ptr(2), ptr(3), ptr(4), ptr(5), ptr(7) if n_groups else None, ptr(7 + n_groups) if n_groups else None),
+        )
+        dev = packed.to(self.device, non_blocking=True)
+        views = [dev[offsets[i] : offsets[i + 1]] for i in range(len(sizes))]
         d_tok, d_pos, d_qs, d_ql, d_kv, d_slot, d_want = views[:7]
         groups = []
         for g in range(n_groups):
@@ -254,13 +232,13 @@ class Engine:
             raise ValueError("a request appears twice in one step")
         ps = self.page_size
         # a token needs a new page only when it starts one (tables hold exactly the pages of the tokens so far)
-        starters = [i for i, rc in enumerate(rcs) if rc.num_tokens % ps == 0]
+        starters = [rc for rc in rcs if rc.num_tokens % ps == 0]
         if starters:
-            self._reserve_all([rcs[i] for i in starters], [entries[i] for i in starters])
+            self.cache.reserve_step(starters, [1] * len(starters))
         b = len(rcs)
         widths = []
         for g in range(len(self.cache.groups)):
-            need = max(len(rc.tables[g]) for rc in rcs)
+            need = max(rc.table_lens[g] for rc in rcs)
             w = 4
             while w < need:
                 w *= 2
@@ -281,12 +259,7 @@ class Engine:
         else:
             plan.graph.replay()
             logits = plan.logits
-        if self._has_windows:
-            for rc in rcs:
-                self.cache.commit(rc, 1)
-        else:
-            for rc in rcs:
-                rc.num_tokens += 1
+        self.cache.commit_step(rcs, plan.ones)
         return logits
 
 
@@ -305,17 +278,10 @@ class _DecodePlan:
         self.host_tab = torch.full((max(n_tab, 1),), -1, dtype=torch.int32).pin_memory()
         self.dev_tab = torch.full((max(n_tab, 1),), -1, dtype=torch.int32, device=dev)
         self.np_small = self.host_small.numpy()
-        self.np_tab = self.host_tab.numpy()
-        hs = self.np_small
-        hs[2 * b : 3 * b] = np.arange(b)          # q_start
-        hs[3 * b : 4 * b] = 1                     # q_len
-        hs[6 * b : 7 * b] = np.arange(b)          # wanted rows: all
         v = lambda i: self.dev_small[i * b : (i + 1) * b]
         groups, off = [], 0
-        self.tab_offsets = []
         for g, w in enumerate(widths):
             groups.append(GroupTables(self.dev_tab[off : off + b * w].view(b, w), v(7 + g)))
-            self.tab_offsets.append(off)
             off += b * w
         ps = engine.page_size
         self.ctx = StepContext(
@@ -326,36 +292,24 @@ class _DecodePlan:
             state_storage=engine.states, cache_location=engine.model.cache_location,
             group_windows=[n.window for n in engine.cache.groups],
         )
-        self.row_owner: list = [None] * b
-        self.row_version = [-1] * b
+        self.row_state = np.full(2 * b, -1, dtype=np.int64)     # per row: (handle, table version) last written
+        self.c_widths = _ints(self.widths)
+        self.ones = [1] * b
+        self.cache = engine.cache
         self.copied = None           # event after the last host-to-device copy
         self.graph = None
         self.logits = None
         self.runs = 0
-        self.ps = ps
 
     def fill(self, rcs, tokens) -> None:
         if self.copied is not None:
             self.copied.synchronize()                       # the pinned mirror is free again
-        b, ps, hs = self.batch, self.ps, self.np_small
-        pos = [rc.num_tokens for rc in rcs]
-        hs[0:b] = tokens
-        hs[b : 2 * b] = pos
-        hs[4 * b : 5 * b] = [p + 1 for p in pos]
-        hs[5 * b : 6 * b] = [rc.slot for rc in rcs]
-        tables_changed = False
-        for g, w in enumerate(self.widths):
-            hs[(7 + g) * b : (8 + g) * b] = [rc.tables[g][p // ps] * ps + p % ps for rc, p in zip(rcs, pos)]
-        for i, rc in enumerate(rcs):
-            if self.row_owner[i] is not rc or self.row_version[i] != rc.version:
-                for g, w in enumerate(self.widths):
-                    o = self.tab_offsets[g] + i * w
-                    t = rc.tables[g]
-                    self.np_tab[o : o + len(t)] = t
-                    self.np_tab[o + len(t) : o + w] = -1
-                self.row_owner[i], self.row_version[i] = rc, rc.version
-                tables_changed = True
-        self.ctx.kv_len_host = [p + 1 for p in pos]
+        b = self.batch
+        self.np_small[0:b] = tokens
+        handles = _ints([rc.handle for rc in rcs])
+        tables_changed = self.cache.fill_decode(handles, self.c_widths, self.host_small.data_ptr(),
+                                                self.host_tab.data_ptr(), self.row_state.ctypes.data)
+        self.ctx.kv_len_host = [rc.num_tokens + 1 for rc in rcs]
         self.ctx.state_slots_host = [rc.slot for rc in rcs]
         self.dev_small.copy_(self.host_small, non_blocking=True)
         if tables_changed:

@@ -187,8 +187,8 @@ class Scheduler:
                     # cut the portion down to what the free pages hold
                     rc = self.cache.requests[r.request_id]
                     room = min(
-                        (len(t) + pool.free_count - p) * self.cache.page_size - rc.num_tokens
-                        for t, pool, p in zip(rc.tables, self.cache.pools, promised)
+                        (have + pool.free_count - p) * self.cache.page_size - rc.num_tokens
+                        for have, pool, p in zip(rc.table_lens, self.cache.pools, promised)
                     )
                     count = min(count - 1, max(room, 0))
                 if count > 0:
