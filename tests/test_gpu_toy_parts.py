@@ -3,6 +3,7 @@ toy architecture, loaded from a random-weights folder and stepped, without a cha
 
   * a mixer with per-request state of its own (a decaying running sum: no paged cache, a state slot);
   * a position encoding that is no rotation (a learned table added to queries and keys);
+  * a feed-forward with routing (router logits in float32, every token to its best expert, per-expert token lists);
   * a run order that names a layer twice and lets a layer read another layer's cache.
 The toy parts compute with torch on the GPU; they are test equipment, not a model of anyone's."""
 import json
@@ -17,9 +18,9 @@ import helpers as H
 import plain_qwen2 as plain
 from easy_gpt.cpp_amd.config import Architecture, register_architecture, unregister_architecture
 from easy_gpt.cpp_amd.parts import (
-    LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec, PositionEncoding, RunSpec, StateNeed, register_part,
+    FeedForward, LayerSpec, Mixer, ModelSpec, ParamSpec, PartSpec, PositionEncoding, RunSpec, StateNeed, register_part,
 )
-from easy_gpt.cpp_amd.parts.base import MIXERS, POSITION_ENCODINGS
+from easy_gpt.cpp_amd.parts.base import FEED_FORWARDS, MIXERS, POSITION_ENCODINGS
 
 pytestmark = pytest.mark.gpu
 
@@ -74,6 +75,36 @@ class LearnedOffset(PositionEncoding):
         k.add_(add)
 
 
+class RoutedFFN(FeedForward):
+    """Router logits r = scale * x Wr^T in float32; every token goes to its best expert e and gets
+    softmax(r)_e * relu(x W1_e^T) W2_e^T.  The experts run on the lists of tokens routed to them."""
+
+    def __init__(self, prefix, hidden_size, n_experts, expert_size, router_scale):
+        self.prefix, self.hidden_size = prefix, hidden_size
+        self.n_experts, self.expert_size, self.router_scale = n_experts, expert_size, float(router_scale)
+
+    def param_specs(self):
+        e, h, i = self.n_experts, self.hidden_size, self.expert_size
+        return [ParamSpec(self.prefix + "router.weight", (e, h), dtype="float32"),
+                ParamSpec(self.prefix + "w1.weight", (e, i, h)), ParamSpec(self.prefix + "w2.weight", (e, h, i))]
+
+    def load(self, get, dtype, device):
+        self.router = self._to(get(self.prefix + "router.weight"), "float32", dtype, device)
+        self.w1 = self._to(get(self.prefix + "w1.weight"), "compute", dtype, device)
+        self.w2 = self._to(get(self.prefix + "w2.weight"), "compute", dtype, device)
+
+    def forward(self, x, ctx):
+        logits = (x.float() @ self.router.T) * self.router_scale
+        prob, expert = torch.softmax(logits, -1).max(-1)
+        out = torch.zeros(x.shape[0], self.hidden_size, dtype=torch.float32, device=x.device)
+        for e in range(self.n_experts):
+            rows = (expert == e).nonzero().flatten()                    # this expert's token list
+            if rows.numel():
+                hid = torch.relu(x[rows].float() @ self.w1[e].float().T).to(x.dtype)
+                out[rows] = prob[rows, None] * (hid.float() @ self.w2[e].float().T)
+        return out.to(x.dtype)
+
+
 @dataclass
 class ToyConfig:
     hidden_size: int
@@ -83,6 +114,9 @@ class ToyConfig:
     decay: float
     eps: float
     max_position_embeddings: int
+    n_experts: int
+    expert_size: int
+    router_scale: float
 
     @classmethod
     def from_dict(cls, d, where="config.json"):
@@ -105,10 +139,14 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
         LayerSpec("pre_norm",
                   PartSpec("gq_attention", dict(attn, position=PartSpec("none", {})), "l2.attn."),
                   ff("l2.ff."), norm("l2.n1."), norm("l2.n2.")),
+        LayerSpec("pre_norm", PartSpec("toy_decay", dict(decay=c.decay), "l3.mix."),
+                  PartSpec("toy_routed", dict(n_experts=c.n_experts, expert_size=c.expert_size, router_scale=c.router_scale), "l3.ff."),
+                  norm("l3.n1."), norm("l3.n2.")),
     )
-    # layer 1 runs twice (second time with a cache of its own); layer 2 reads layer 1's first cache and writes none
+    # layer 1 runs twice (second time with a cache of its own); layer 2 reads layer 1's first cache and writes none;
+    # the routed feed-forward comes last, so that a token whose two best experts nearly tie changes only its own logits
     run_order = (RunSpec(0, None, True, state=0), RunSpec(1, cache=0), RunSpec(2, cache=0, writes_cache=False),
-                 RunSpec(1, cache=1))
+                 RunSpec(1, cache=1), RunSpec(3, None, True, state=1))
     return ModelSpec(
         hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
         embedding=PartSpec("token_embedding", {}, "emb."), layers=layers, run_order=run_order,
@@ -117,22 +155,25 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
 
 
 TOY_CONFIG = {"architectures": ["ToyMixForCausalLM"], "hidden_size": 48, "vocab_size": 211, "n_heads": 3, "head_dim": 16,
-              "decay": 0.9, "eps": 1e-5, "max_position_embeddings": 96}
+              "decay": 0.9, "eps": 1e-5, "max_position_embeddings": 96, "n_experts": 4, "expert_size": 40, "router_scale": 300.0}
 
 
 @pytest.fixture()
 def toy_registered():
     register_part("mixer", "toy_decay", DecayMixer)
     register_part("position_encoding", "toy_learned_offset", LearnedOffset)
+    register_part("feed_forward", "toy_routed", RoutedFFN)
     register_architecture(Architecture("ToyMixForCausalLM", ToyConfig, toy_spec, ("toymix",)))
     yield
     unregister_architecture("ToyMixForCausalLM")
     MIXERS.pop("toy_decay")
     POSITION_ENCODINGS.pop("toy_learned_offset")
+    FEED_FORWARDS.pop("toy_routed")
 
 
 def toy_plain(w, cfg, ids):
-    """Whole sequence, no cache, float64: the toy model written out plainly."""
+    """Whole sequence, no cache, float64: the toy model written out plainly.  Returns the logits and, per token,
+    the gap between the two largest router logits of the routed feed-forward."""
     x = w["emb.weight"][torch.tensor(ids)]
     s = len(ids)
     hd, nh = cfg["head_dim"], cfg["n_heads"]
@@ -178,7 +219,24 @@ def toy_plain(w, cfg, ids):
     q, k, v = attn_qkv(xn, "l1.attn.", w["l1.attn.pos.weight"])
     x = x + attn_out(q, k, v, "l1.attn.")
     x = x + ffn(plain.rms_norm(x, w["l1.n2.weight"], cfg["eps"]), "l1.ff.")
-    return plain.linear(plain.rms_norm(x, w["final.weight"], cfg["eps"]), w["head.weight"])
+    # run 4: a second decay mixer (state 1), then the routed feed-forward
+    xn = plain.rms_norm(x, w["l3.n1.weight"], cfg["eps"])
+    u = xn @ w["l3.mix.w.weight"].T
+    st, outs = torch.zeros(cfg["hidden_size"], dtype=torch.float64), []
+    for t in range(s):
+        st = cfg["decay"] * st + u[t]
+        outs.append(st)
+    x = x + torch.stack(outs)
+    xn = plain.rms_norm(x, w["l3.n2.weight"], cfg["eps"])
+    r = (xn @ w["l3.ff.router.weight"].T) * cfg["router_scale"]
+    top2 = r.topk(2, -1).values
+    prob = torch.softmax(r, -1)
+    routed = torch.zeros_like(x)
+    for t in range(s):
+        e = int(r[t].argmax())
+        routed[t] = prob[t, e] * (torch.relu(xn[t] @ w["l3.ff.w1.weight"][e].T) @ w["l3.ff.w2.weight"][e].T)
+    x = x + routed
+    return plain.linear(plain.rms_norm(x, w["final.weight"], cfg["eps"]), w["head.weight"]), top2[:, 0] - top2[:, 1]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -191,15 +249,21 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_registered, tmp_pa
     d = write_random_model(str(tmp_path / "toy"), TOY_CONFIG, seed=3)
     eng = Engine.from_dir(d, dtype=dtype, device="cuda:0", page_size=4, max_tokens=256, max_requests=3)
     assert len(eng.model.cache_groups) == 1 and eng.model.cache_groups[0].cache_ids == (0, 1)
-    assert list(eng.model.state_needs) == [0] and eng.states.data[0].shape == (3, 48)
+    assert list(eng.model.state_needs) == [0, 1] and eng.states.data[0].shape == (3, 48)
     w = plain.read_safetensors(os.path.join(d, "model.safetensors"))
     if dtype == "bfloat16":
         w = {k: v.float().to(torch.bfloat16).double() for k, v in w.items()}
     reqs = H.make_requests(TOY_CONFIG["vocab_size"], [40, 9, 77, 30], seed=5)
-    ref = {rid: toy_plain(w, TOY_CONFIG, ids) for rid, ids in reqs.items()}
+    both = {rid: toy_plain(w, TOY_CONFIG, ids) for rid, ids in reqs.items()}
+    ref = {rid: logits for rid, (logits, _) in both.items()}
+    # a token whose two best experts nearly tie may go to the other one in the engine's precision: such tokens
+    # (few, and only their own logits depend on it) are left out of the comparison
+    near = 1e-3 if dtype == "float32" else 3.0
+    tied = {(rid, t) for rid, (_, gap) in both.items() for t in range(len(gap)) if float(gap[t]) < near}
+    assert len(tied) <= 0.1 * sum(len(v) for v in reqs.values())
     tol = 3e-5 if dtype == "float32" else 3e-2
     for trace in (H.trace_whole(reqs), H.trace_portions(reqs), H.trace_mixed(reqs, seed=2, max_live=3, decode_tail=6)):
         rows = H.replay(eng, trace)
         assert len(rows) == sum(len(v) for v in reqs.values())
-        H.assert_rows_match(rows, ref, tol, f"toy {dtype}")
+        H.assert_rows_match({k: v for k, v in rows.items() if k not in tied}, ref, tol, f"toy {dtype}")
     assert eng.cache.free_pages() == [64]
