@@ -48,7 +48,16 @@ TINY_D = {
     "use_sliding_window": True, "sliding_window": 40, "max_window_layers": 1,
     "bos_token_id": 5, "eos_token_id": 6, "torch_dtype": "bfloat16",
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+# A fifth one with the other head size of the matrix-core attention kernels (128), four query heads on one
+# kv head, a width that is no multiple of the head size, a separate output matrix.
+TINY_E = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 160, "num_attention_heads": 4, "num_key_value_heads": 1,
+    "head_dim": 128, "intermediate_size": 264, "vocab_size": 901, "rope_theta": 300000.0,
+    "rms_norm_eps": 2e-6, "tie_word_embeddings": False, "max_position_embeddings": 384, "hidden_act": "silu",
+    "use_sliding_window": False, "bos_token_id": 8, "eos_token_id": 9, "torch_dtype": "bfloat16",
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4)}
 
 
 @pytest.fixture(scope="session")

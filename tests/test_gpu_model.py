@@ -51,7 +51,7 @@ def lengths_for(name):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_cutting_agrees_with_plain(tiny_models, sharp_models, name, dtype):
     cfg = TINY[name][0]
     reqs = H.make_requests(cfg["vocab_size"], lengths_for(name), seed=21)
@@ -74,7 +74,7 @@ def test_every_cutting_agrees_with_plain(tiny_models, sharp_models, name, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_mixed_batches_with_page_reuse(sharp_models, name, dtype):
     cfg = TINY[name][0]
     cap = cfg["max_position_embeddings"]
