@@ -918,12 +918,13 @@ static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml
     return EGPT_OK;
 }
 
-template <int HD>
+// PF: key blocks per round of loads of a wavefront.  More of them in flight is fewer round trips but more
+// registers; when there are so many workgroups that they must share CUs, fewer registers are worth more.
+template <int HD, int PF>
 static int launch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                          const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size, float scale,
                          int window, int n_splits, int n_waves, int combine, const FusedQkv* fused, hipStream_t s) {
-    constexpr int PF = HD == 64 ? 4 : 2;
     dim3 grid(n_seqs, nkv, n_splits);
     size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
     if (fused) lds += 18 * HD * sizeof(bf16_t);          // 16 query heads, the new key and value
@@ -945,6 +946,20 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
         EGPT_CHECK_LAUNCH();
     }
     return EGPT_OK;
+}
+
+static int dispatch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                           const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
+                           const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
+                           int window, int n_splits, int n_waves, int combine, const FusedQkv* fused, hipStream_t s) {
+    // more workgroups than two per CU: the variant with half the loads in flight and fewer registers
+    const bool lean = static_cast<long>(n_seqs) * nkv * n_splits > 512;
+#define EGPT_LAUNCH_DECODE(HD_, PF_)                                                                             \
+    launch_decode<HD_, PF_>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len, \
+                            n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, fused, s)
+    if (hd == 64) return lean ? EGPT_LAUNCH_DECODE(64, 2) : EGPT_LAUNCH_DECODE(64, 4);
+    return lean ? EGPT_LAUNCH_DECODE(128, 1) : EGPT_LAUNCH_DECODE(128, 2);
+#undef EGPT_LAUNCH_DECODE
 }
 
 }  // namespace egpt
@@ -1023,12 +1038,8 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
         n_waves < 1 || n_waves > 8)
         return EGPT_UNSUPPORTED_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (hd == 64)
-        return launch_decode<64>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start,
-                                 kv_len, n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine,
-                                 nullptr, s);
-    return launch_decode<128>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, nullptr, s);
+    return dispatch_decode(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, nullptr, s);
 }
 
 // The same with the QKV epilogue folded in: the queries, and the new token's key and value, are computed from
@@ -1061,12 +1072,8 @@ extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits,
     f.cos_sin = cos_sin; f.slots = slots;
     f.k_cache_w = static_cast<bf16_t*>(k_cache); f.v_cache_w = static_cast<bf16_t*>(v_cache);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (hd == 64)
-        return launch_decode<64>(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start,
-                                 kv_len, n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine,
-                                 &f, s);
-    return launch_decode<128>(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                              n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, &f, s);
+    return dispatch_decode(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, &f, s);
 }
 
 // bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.
