@@ -416,6 +416,92 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
     }
 }
 
+// The product for 17 to 64 rows and many columns: x stays in LDS for the workgroup's whole k range (up to
+// kResidentSteps steps of 128), staged once, and every load of w for that range is issued before the first
+// product.  With that many rows the step-by-step kernel above pays for its barriers and for float32 partial
+// sums that weigh as much as the weights; here a workgroup is one round of loads, its products and one store,
+// and with a k range of the whole k the output needs no partial sums.
+constexpr int kResidentSteps = 8;
+
+template <int MT, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_resident_kernel(SkinnyArgs a) {
+    constexpr int kThreads = 64 * NW;
+    constexpr int kRow = kResidentSteps * kStep + 8;                       // bf16 elements per staged row
+    __shared__ __attribute__((aligned(16))) bf16_t xs[MT * 16][kRow];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int li = lane % 16, lg = lane / 16;
+    const int split = blockIdx.y;
+    const int m = a.m, n = a.n, k = a.k;
+    const int n0 = (blockIdx.x * NW + wave) * kRowsPerWave;
+    const int total_steps = (k + kStep - 1) / kStep;
+    const int step_begin = split * a.steps_per_split;
+    const int n_steps = min(total_steps, step_begin + a.steps_per_split) - step_begin;       // <= kResidentSteps
+    const int k_begin = step_begin * kStep;
+    const int w_row = min(n0 + li, n - 1);
+    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + k_begin + lg * 32;
+
+    // the whole stream of w for this workgroup
+    uint4 av[kResidentSteps][4];
+#pragma unroll
+    for (int s = 0; s < kResidentSteps; ++s)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            av[s][q] = load16(wp + s * kStep + q * 8, s < n_steps && k_begin + s * kStep + lg * 32 + q * 8 < k);
+    // x: sixteen threads per row take its sixteen chunks of a step; a thread walks the steps of a row (all its
+    // loads in flight together), then the next of its rows.  No division in any index: with a vector
+    // instruction at four cycles, index arithmetic is what such a kernel would otherwise spend its time on.
+    constexpr int kRowsPerPass = kThreads / 16;
+    const int r16 = tid / 16, c16 = (tid % 16) * 8;
+#pragma unroll
+    for (int j = 0; j < (MT * 16 + kRowsPerPass - 1) / kRowsPerPass; ++j) {
+        const int r = r16 + kRowsPerPass * j;
+        if (r >= m) break;                     // rows past m are never read back
+        const bf16_t* xp = a.x + static_cast<size_t>(r) * k + k_begin + c16;
+        uint4 v[kResidentSteps];
+#pragma unroll
+        for (int st = 0; st < kResidentSteps; ++st)
+            v[st] = load16(xp + st * kStep, st < n_steps && k_begin + st * kStep + c16 < k);
+#pragma unroll
+        for (int st = 0; st < kResidentSteps; ++st)
+            if (st < n_steps) *reinterpret_cast<uint4*>(&xs[r][st * kStep + c16]) = v[st];
+    }
+    __syncthreads();
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < kResidentSteps; ++s) {
+        if (s >= n_steps) break;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const bf16x8 wv = __builtin_bit_cast(bf16x8, av[s][q]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const uint4 bv = *reinterpret_cast<const uint4*>(&xs[t * 16 + li][s * kStep + lg * 32 + q * 8]);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
+            }
+        }
+    }
+    // D layout: lane (li, lg) holds rows lg*4 + v of the 16 x 16 tile (an n index) at column li (an m index)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int mm = t * 16 + li;
+        if (mm >= m) continue;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int nn = n0 + lg * 4 + v;
+            if (nn >= n) continue;
+            float val = acc[t][v];
+            if (a.bias) val += to_float(a.bias[nn]);
+            if (a.out_bf16)
+                a.out_bf16[static_cast<size_t>(mm) * n + nn] = from_float<bf16_t>(val);
+            else
+                a.out_f32[(static_cast<size_t>(split) * m + mm) * n + nn] = val;
+        }
+    }
+}
+
 static int check_splits(int k, int n_splits, int* steps_per_split) {
     const int total_steps = (k + kStep - 1) / kStep;
     if (n_splits < 1 || n_splits > total_steps) return EGPT_BAD_ARGUMENT;
@@ -459,6 +545,23 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
     a.out_f32 = out_f32;
     a.out_bf16 = static_cast<bf16_t*>(out_bf16);
     a.m = m; a.n = n; a.k = k;
+    if (waves != 16 && m > 16 && a.steps_per_split <= kResidentSteps && n >= 4096) {
+        // many columns, more than one tile of rows, a k range that fits in LDS: x resident, one round of loads
+        const dim3 grid = skinny_grid(n, n_splits, waves);
+        hipStream_t s_ = static_cast<hipStream_t>(stream);
+        const int mt = (m + 15) / 16;
+        if (waves == 4) {
+            if (mt == 2) gemm_resident_kernel<2, 4><<<grid, 256, 0, s_>>>(a);
+            else if (mt == 3) gemm_resident_kernel<3, 4><<<grid, 256, 0, s_>>>(a);
+            else gemm_resident_kernel<4, 4><<<grid, 256, 0, s_>>>(a);
+        } else {
+            if (mt == 2) gemm_resident_kernel<2, 8><<<grid, 512, 0, s_>>>(a);
+            else if (mt == 3) gemm_resident_kernel<3, 8><<<grid, 512, 0, s_>>>(a);
+            else gemm_resident_kernel<4, 8><<<grid, 512, 0, s_>>>(a);
+        }
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     switch ((m + 15) / 16) {
         case 1: EGPT_SKINNY(1, kPlain, 8); break;
         case 2: EGPT_SKINNY(2, kPlain, 8); break;

@@ -170,9 +170,11 @@ class HipKernels:
                 for r0 in range(0, m, 64):
                     r1 = min(m, r0 + 64)
                     xo, oo = x[r0:r1], out[r0:r1]
+                    # (a very wide output with more than one tile of rows: workgroups of 8 wavefronts stage x half
+                    # as often)
                     self._run("egpt_gemm_skinny", xo.data_ptr(), w.data_ptr(), self._ptr(bias),
                               oo.data_ptr() if to_f32 else None, None if to_f32 else oo.data_ptr(), r1 - r0, n, k, 1,
-                              4, self._stream())
+                              8 if (r1 - r0 > 16 and n >= 65536) else 4, self._stream())
                 return out
             # many rows: the library's matrix product (the reference uses cuBLAS for every linear layer)
             if bias is None:
@@ -292,6 +294,11 @@ class HipKernels:
             self._need(x, "x")
             self._need(w, "w", x.dtype, (n, k))
             s = self._n_splits(m, n, k)
+            if m > 16 and n >= 4096:
+                # more than one tile of rows and many columns: the kernel that keeps x in LDS for a k range of up
+                # to 8 steps; as few splits as that allows (none at all for k <= 1024: no partial sums)
+                steps = -(-k // 128)
+                s = -(-steps // 8)
             out = torch.empty((s, m, n), dtype=_F32, device=x.device)
             self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s, 4,
                       self._stream())
