@@ -33,12 +33,26 @@ def _load_library() -> ctypes.CDLL:
     return lib
 
 
+class _PinnedStream:
+    def __init__(self, kernels):
+        self.kernels = kernels
+
+    def __enter__(self):
+        self.before = self.kernels._pinned
+        self.kernels._pinned = torch.cuda.current_stream().cuda_stream
+
+    def __exit__(self, *exc):
+        self.kernels._pinned = self.before
+        return False
+
+
 class HipKernels:
     name = "hip-gfx950"
 
     def __init__(self):
         lib = _load_library()
         self.lib = lib
+        self._pinned = None
         vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
         lib.egpt_error_string.restype = ctypes.c_char_p
         lib.egpt_error_string.argtypes = [i]
@@ -69,9 +83,16 @@ class HipKernels:
             fn.restype = i
 
     # ------------------------------------------------------------------ helpers
-    @staticmethod
-    def _stream():
-        return torch.cuda.current_stream().cuda_stream
+    def _stream(self):
+        """The stream to launch on: torch's current one.  Asking torch costs several microseconds, and a step
+        launches a couple of hundred kernels, so a model's forward pass asks once (`pinned_stream`)."""
+        return self._pinned if self._pinned is not None else torch.cuda.current_stream().cuda_stream
+
+    def pinned_stream(self):
+        """Context manager: within it every launch goes to the stream that is current on entry.  The caller
+        promises not to change the current stream inside (graph capture changes it before the forward pass
+        is entered, which is fine)."""
+        return _PinnedStream(self)
 
     def _run(self, name: str, *args) -> None:
         code = getattr(self.lib, name)(*args)
