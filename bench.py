@@ -123,7 +123,7 @@ def main() -> int:
     if not args.no_points or args.prefill_only:
         ids = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
         times = []
-        for rep in range(5):
+        for rep in range(11):                                  # the first one warms up; the median of ten counts
             engine.add_request("prefill")
             sync()
             t0 = time.perf_counter()

@@ -140,9 +140,13 @@ class Engine:
                 raise KeyError(f"request {e.request_id!r} is not live (add_request first)")
             rc = self.cache.requests[e.request_id]
             n = len(e.tokens)
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise IndexError(f"token id {t} of request {e.request_id!r} is outside [0, {self.vocab_size})")
+            ids = np.asarray(e.tokens, dtype=np.int64)          # one pass in C instead of a Python loop per token
+            if ids.ndim != 1:
+                raise ValueError(f"the tokens of request {e.request_id!r} must be a flat list of ids")
+            lo, hi = int(ids.min()), int(ids.max())
+            if lo < 0 or hi >= self.vocab_size:
+                bad = lo if lo < 0 else hi
+                raise IndexError(f"token id {bad} of request {e.request_id!r} is outside [0, {self.vocab_size})")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise IndexError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
@@ -178,7 +182,8 @@ class Engine:
             offsets.append(offsets[-1] + n)
         packed = torch.empty(offsets[-1], dtype=torch.int32, pin_memory=self.device.type == "cuda")
         host = packed.numpy()
-        host[0:t] = np.fromiter((tok for e in entries for tok in e.tokens), dtype=np.int64, count=t)
+        for s0, e in zip(q_start, entries):
+            host[s0 : s0 + len(e.tokens)] = e.tokens
         host[offsets[6] : offsets[7]] = want_rows
         base = packed.data_ptr()
         ptr = lambda i: base + 4 * offsets[i]
