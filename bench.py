@@ -54,6 +54,8 @@ def main() -> int:
     ap.add_argument("--shape", default="0.5b", choices=["0.5b"] + sorted(OTHER_SHAPES),
                     help="layer sizes: Qwen2.5-0.5B (the record's) or another size of the baseline record")
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prefix", type=int, default=None,
+                    help="tokens each request holds before decoding starts (default: the record's 2,048)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
@@ -68,6 +70,11 @@ def main() -> int:
         base.update(changes)
         CONTEXT = PREFIX + 2048
         name = f"Qwen2.5-{args.shape.upper()}"
+    if args.prefix is not None:
+        if args.prefix < 1 or args.prefix + NEW_TOKENS > base["max_position_embeddings"]:
+            print(f"--prefix must be between 1 and {base['max_position_embeddings'] - NEW_TOKENS}")
+            return 2
+        PREFIX, CONTEXT = args.prefix, args.prefix + 2048
     if args.layers is None:
         args.layers = FULL_LAYERS
     if args.warmup + args.steps > CONTEXT - PREFIX:
@@ -94,7 +101,8 @@ def main() -> int:
     t_setup = time.time()
     tmp = tempfile.mkdtemp(prefix="egpt_bench_")
     write_random_model(tmp, cfg, seed=0, dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
-    tokens_per_request = -(-(PREFIX + NEW_TOKENS) // page_size) * page_size
+    new_tokens = max(NEW_TOKENS, args.warmup + args.steps)        # a longer run than the record's decodes further
+    tokens_per_request = -(-(PREFIX + new_tokens) // page_size) * page_size
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
                              max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1)
     for f in os.listdir(tmp):
@@ -193,7 +201,7 @@ def main() -> int:
         "config": {
             "model": f"{name} layer sizes", "layers": layers, "layers_of_model": FULL_LAYERS, "hidden": h,
             "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]),
-            "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": NEW_TOKENS,
+            "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": new_tokens,
             "page_size": page_size, "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
             "sampling": "greedy", "parallelism": "single GPU",
         },
