@@ -409,12 +409,14 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
         vv = torch.randn(kv, nkv, hd, generator=g).to(dtype)
         keys.append(kk)
         vals.append(vv)
-        for j in range(kv):
-            if j % ps == 0:
-                table[b, j // ps] = order.pop()
-            pg = int(table[b, j // ps])
-            kc[pg, :, j % ps, :] = kk[j]
-            vc[pg, :, :, j % ps] = vv[j]
+        n = -(-kv // ps)
+        pages = torch.tensor([order.pop() for _ in range(n)], dtype=torch.int64)
+        table[b, :n] = pages.to(torch.int32)
+        kp = torch.full((n * ps, nkv, hd), 1e4, dtype=dtype)
+        vp = torch.full((n * ps, nkv, hd), -1e4, dtype=dtype)
+        kp[:kv], vp[:kv] = kk, vv
+        kc[pages] = kp.view(n, ps, nkv, hd).permute(0, 2, 1, 3)
+        vc[pages] = vp.view(n, ps, nkv, hd).permute(0, 2, 3, 1)
     return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
 
 
@@ -478,6 +480,14 @@ def test_paged_attention_tiled_workgroup_shapes(k, hd, shape, window, ps):
     assert run_paged(k, seqs, 7, 1, hd, ps, torch.bfloat16, window=window, tiled_shape=shape, q_scale=6.0, seed=3) <= 4e-2
 
 
+@pytest.mark.parametrize("hd,shape", [(64, None), (64, 44), (128, None), (128, 41)])
+@pytest.mark.parametrize("window", [0, 4099])
+def test_paged_attention_long_prefixes(k, hd, shape, window):
+    # prompt portions behind thousands of cached keys: many key tiles for each row tile, block tables hundreds of pages wide
+    seqs = [(96, 9000), (1, 5000), (40, 12001), (3, 3)]
+    assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, window=window, tiled_shape=shape, seed=5) <= 1.2e-2
+
+
 def test_paged_attention_tiled_refuses_other_page_sizes(k):
     z = torch.zeros(64, device=DEV)
     p = z.data_ptr()
@@ -487,7 +497,7 @@ def test_paged_attention_tiled_refuses_other_page_sizes(k):
 
 
 @pytest.mark.parametrize("nq,nkv,hd", [(14, 2, 64), (12, 2, 128), (3, 1, 64)])
-@pytest.mark.parametrize("batch,ctx", [(1, 2113), (8, 700), (64, 130), (3, 33)])
+@pytest.mark.parametrize("batch,ctx", [(1, 2113), (8, 700), (64, 130), (3, 33), (1, 20011), (4, 6007), (40, 1500)])
 def test_paged_attention_decode_batches_split_the_key_range(k, nq, nkv, hd, batch, ctx):
     # only decoded tokens, different lengths: the matrix-core kernel splits the keys and combines the parts
     seqs = [(1, max(1, ctx - 37 * i % ctx)) for i in range(batch)]
@@ -497,7 +507,8 @@ def test_paged_attention_decode_batches_split_the_key_range(k, nq, nkv, hd, batc
 
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(14, 2, 64, 16), (12, 2, 128, 16), (3, 3, 64, 32), (16, 1, 64, 16)])
-@pytest.mark.parametrize("batch,ctx,window", [(8, 700, 0), (1, 2113, 0), (64, 130, 0), (3, 33, 0), (5, 1, 0), (8, 300, 100)])
+@pytest.mark.parametrize("batch,ctx,window", [(8, 700, 0), (1, 2113, 0), (64, 130, 0), (3, 33, 0), (5, 1, 0), (8, 300, 100),
+                                              (1, 20011, 0), (4, 6007, 0), (40, 1500, 0), (2, 9000, 4099)])
 @pytest.mark.parametrize("with_scale,with_bias", [(True, True), (False, False)])
 def test_decode_attention_with_the_qkv_epilogue_folded_in(k, nq, nkv, hd, ps, batch, ctx, window, with_scale, with_bias):
     # one kernel for bias + rotation + store + attention must leave the same bits, in its output and in the
