@@ -114,6 +114,26 @@ def test_long_decoding(sharp_models, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_across_the_context_steps_of_the_captured_graphs(sharp_models, dtype):
+    # two requests decoded side by side from 490 and 400 tokens on: the decode graphs are captured per step of the
+    # longest context (512 tokens) and per width of the block tables, and both change on the way
+    name = "D"
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [620, 530], seed=43)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    a, b = reqs["r0"], reqs["r1"]
+    trace = [H.step_record(0, [("r0", a[:490], [489])]), H.step_record(1, [("r1", b[:400], [0, 399])])]
+    for i in range(130):
+        trace.append(H.step_record(2 + i, [("r0", [a[490 + i]], [0]), ("r1", [b[400 + i]], [0])],
+                                   ["r0", "r1"] if i == 129 else []))
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16))
+    rows = H.replay(eng, trace)
+    assert len(rows) == 3 + 260
+    H.assert_rows_match(rows, ref, tol_of(dtype), f"decoding across graph steps {dtype}")
+    assert len({key[2] for key in eng._decode_plans}) >= 2 and len({key[1] for key in eng._decode_plans}) >= 2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens_of_a_sequence(tiny_models, name, dtype):
     cfg = TINY[name][0]
