@@ -11,6 +11,7 @@ the engine's dtype when they take them.
 """
 from __future__ import annotations
 
+import json
 import os
 from typing import Iterable
 
@@ -76,16 +77,57 @@ _STORED_AS = {
 
 
 class CheckedWeights:
-    """A safetensors file whose names and shapes were checked; `get(name)` reads one tensor."""
+    """The safetensors file(s) of a model folder whose names and shapes were checked; `get(name)` reads one tensor.
+
+    A folder holds `model.safetensors` (all the reference reads, /root/reference/src/models/loader.cpp:45-63),
+    or, for checkpoints stored in several files, `model.safetensors.index.json` whose "weight_map" names the
+    file of every tensor."""
+
+    INDEX = "model.safetensors.index.json"
 
     def __init__(self, model_dir: str, specs: Iterable[ParamSpec], ignorable: Iterable[str] = ()):
         self.path = os.path.join(model_dir, "model.safetensors")
-        self.file = SafetensorsFile(self.path)
-        available = {n: self.file.shape(n) for n in self.file.names()}
-        self.ignored = check_names_and_shapes(available, specs, ignorable, where=self.path)
+        self.files: list[SafetensorsFile] = []
+        self._file_of: dict[str, SafetensorsFile] = {}
+        index = os.path.join(model_dir, self.INDEX)
+        try:
+            if not os.path.isfile(self.path) and os.path.isfile(index):
+                self.path = index
+                self._open_shards(model_dir, index)
+            else:
+                f = SafetensorsFile(self.path)
+                self.files.append(f)
+                self._file_of = {n: f for n in f.names()}
+            available = {n: f.shape(n) for n, f in self._file_of.items()}
+            self.ignored = check_names_and_shapes(available, specs, ignorable, where=self.path)
+        except Exception:
+            self.close()
+            raise
+
+    def _open_shards(self, model_dir: str, index: str) -> None:
+        try:
+            with open(index, "r", encoding="utf-8") as fh:
+                weight_map = json.load(fh)["weight_map"]
+            assert isinstance(weight_map, dict) and all(isinstance(v, str) for v in weight_map.values())
+        except (OSError, ValueError, KeyError, TypeError, AssertionError) as e:
+            raise WeightsError(f"{index}: not an index with a 'weight_map' of tensor name -> file ({e})") from e
+        opened: dict[str, SafetensorsFile] = {}
+        for name, rel in weight_map.items():
+            if os.path.basename(rel) != rel:
+                raise WeightsError(f"{index}: file '{rel}' of tensor '{name}' must lie in the model folder")
+            if rel not in opened:
+                opened[rel] = SafetensorsFile(os.path.join(model_dir, rel))
+                self.files.append(opened[rel])
+            if name not in opened[rel].entries:
+                raise WeightsError(f"{index}: tensor '{name}' is not in '{rel}'")
+            self._file_of[name] = opened[rel]
+        # a tensor that a file holds but the index does not name is reported as unexpected by the check
+        for rel, f in opened.items():
+            for name in f.names():
+                self._file_of.setdefault(name, f)
 
     def get(self, name: str) -> torch.Tensor:
-        t = self.file.read(name)
+        t = self._file_of[name].read(name)
         target = _STORED_AS[t.dtype]
         if t.dtype == torch.int64 and t.numel():
             if int(t.max()) > 2**31 - 1 or int(t.min()) < -(2**31):
@@ -93,4 +135,6 @@ class CheckedWeights:
         return t if t.dtype == target else t.to(target)
 
     def close(self) -> None:
-        self.file.close()
+        for f in self.files:
+            f.close()
+        self.files = []

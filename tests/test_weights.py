@@ -76,6 +76,40 @@ def test_complete_set_validates(tmp_path):
     cw.close()
 
 
+def test_checkpoint_in_several_files_with_an_index(tmp_path):
+    model = model_for(FIXTURE)
+    tensors = random_tensors(model.param_specs(), 0, torch.float32)
+    names = list(tensors)
+    parts = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for fname, part in parts.items():
+        write_safetensors(str(tmp_path / fname), {n: tensors[n] for n in part})
+    index = {"metadata": {}, "weight_map": {n: f for f, part in parts.items() for n in part}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    cw = CheckedWeights(str(tmp_path), model.param_specs())
+    for n in names:
+        assert torch.equal(cw.get(n), tensors[n])
+    cw.close()
+    # a tensor that the index sends to the wrong file, a missing file, and a missing tensor
+    bad = dict(index, weight_map=dict(index["weight_map"], **{names[0]: "model-00002-of-00002.safetensors"}))
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(bad))
+    with pytest.raises(WeightsError, match="is not in"):
+        CheckedWeights(str(tmp_path), model.param_specs())
+    bad = dict(index, weight_map=dict(index["weight_map"], **{names[0]: "gone.safetensors"}))
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(bad))
+    with pytest.raises(SafetensorsError, match="not found"):
+        CheckedWeights(str(tmp_path), model.param_specs())
+    os.remove(tmp_path / "model-00002-of-00002.safetensors")
+    write_safetensors(str(tmp_path / "model-00002-of-00002.safetensors"), {n: tensors[n] for n in names[3::2]})
+    short = {n: f for n, f in index["weight_map"].items() if n != names[1]}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": short}))
+    with pytest.raises(WeightsError) as e:
+        CheckedWeights(str(tmp_path), model.param_specs())
+    assert e.value.missing == [names[1]]
+    (tmp_path / "model.safetensors.index.json").write_text("{}")
+    with pytest.raises(WeightsError, match="weight_map"):
+        CheckedWeights(str(tmp_path), model.param_specs())
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     def mutate(t):
         del t["model.layers.0.self_attn.k_proj.weight"]           # missing, as in the reference's test :372
