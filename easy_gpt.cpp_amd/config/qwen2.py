@@ -60,6 +60,10 @@ class Qwen2Config:
                 )
             head_dim = hidden // heads
         layers = r.integer("num_hidden_layers", minimum=1)
+        if data.get("rope_scaling") is not None:
+            # the reference has plain rotary position encoding only (/root/reference/src/ops.cpp:392-458);
+            # running a model that was trained with scaled angles without them would give wrong logits
+            raise ConfigError(f"{where}: 'rope_scaling' ({data['rope_scaling']!r}) is not supported (only plain RoPE)")
         use_window = r.boolean("use_sliding_window", False)
         window = r.integer("sliding_window", None, minimum=1)
         cfg = cls(

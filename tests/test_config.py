@@ -128,3 +128,18 @@ def test_register_another_architecture(tmp_path):
 def test_missing_config_file(tmp_path):
     with pytest.raises(ConfigError, match="not found"):
         load_model_config(str(tmp_path))
+
+
+def test_a_published_config_reads_and_scaled_rotation_is_refused():
+    # the keys a published Qwen2.5 config.json carries (values of the 0.5B model), unknown ones included
+    d = {"architectures": ["Qwen2ForCausalLM"], "attention_dropout": 0.0, "bos_token_id": 151643, "eos_token_id": 151645,
+         "hidden_act": "silu", "hidden_size": 896, "initializer_range": 0.02, "intermediate_size": 4864,
+         "max_position_embeddings": 32768, "max_window_layers": 21, "model_type": "qwen2", "num_attention_heads": 14,
+         "num_hidden_layers": 24, "num_key_value_heads": 2, "rms_norm_eps": 1e-06, "rope_theta": 1000000.0,
+         "sliding_window": 32768, "tie_word_embeddings": True, "torch_dtype": "bfloat16", "use_cache": True,
+         "use_sliding_window": False, "vocab_size": 151936, "rope_scaling": None}
+    cfg = Qwen2Config.from_dict(d)
+    assert cfg.head_dim == 64 and cfg.attention_bias and all(cfg.layer_window(i) is None for i in range(24))
+    d["rope_scaling"] = {"type": "yarn", "factor": 4.0}
+    with pytest.raises(ConfigError, match="rope_scaling"):
+        Qwen2Config.from_dict(d)
