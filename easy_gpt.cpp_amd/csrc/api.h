@@ -19,7 +19,10 @@ int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, 
 // *_splits argument is > 0 and the consumer adds the splits up; 0 means one tensor of the activation type.
 int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
                      const void* weight, float eps, void* out, int n_rows, int hidden, int dtype, void* stream);
-int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype, void* stream);
+// row_ss (may be null) float32 [ss_splits, n_tokens]: gate_up are float32 partial sums that still lack each row's factor
+// 1/sqrt(sum_s row_ss[s][t] / hidden + eps)
+int egpt_swiglu(const void* gate_up, int n_splits, const float* row_ss, int ss_splits, int hidden, float eps, void* out,
+                int n_tokens, int inter, int dtype, void* stream);
 // qkv_out [n_tokens, (nq + 2 nkv) hd] of the activation type; may be qkv_in itself when n_splits == 0.
 // row_ss != null: the product still lacks each row's factor 1 / sqrt(sum_s row_ss[s][row] / hidden + eps).
 // cos_sin != null: the angles' cosines and sines from egpt_rope_table ([n_tokens][rotary_dim / 2][2]) instead of

@@ -154,6 +154,23 @@ __global__ void swiglu_kernel(ProductView<T> gate_up, T* __restrict__ out, int n
     }
 }
 
+// The same from float32 partial sums of a product that still lacks each row's factor 1/rms (a norm folded into
+// the product leaves the factor to its consumer): scale = 1/sqrt(sum_s row_ss[s][t] / hidden + eps) multiplies gate and
+// up before the activation.  One row of workgroups per token.
+template <typename T>
+__global__ void swiglu_scaled_kernel(ProductView<float> gate_up, const float* __restrict__ row_ss, int ss_splits,
+                                     float inv_hidden, float eps, T* __restrict__ out, int n_tokens, int inter) {
+    const size_t t = blockIdx.y;
+    float ss = 0.f;
+    for (int s = 0; s < ss_splits; ++s) ss += row_ss[static_cast<size_t>(s) * n_tokens + t];
+    const float scale = inv_rms(ss, inv_hidden, eps);
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < inter; j += gridDim.x * blockDim.x) {
+        const float g = scale_then_bias(gate_up.at(t * 2 * inter + j), scale, 0.f);
+        const float u = scale_then_bias(gate_up.at(t * 2 * inter + inter + j), scale, 0.f);
+        out[t * inter + j] = from_float<T>(u * (g / (1.0f + expf(-g))));
+    }
+}
+
 // bfloat16, eight features per thread (inter % 8 == 0, one tensor, no partial sums)
 template <typename GT>
 __global__ __launch_bounds__(256) void swiglu_vec8_kernel(const GT* __restrict__ gate_up, bf16_t* __restrict__ out,
@@ -409,14 +426,30 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, i
     return EGPT_OK;
 }
 
-extern "C" int egpt_swiglu(const void* gate_up, int n_splits, void* out, int n_tokens, int inter, int dtype,
-                           void* stream) {
+extern "C" int egpt_swiglu(const void* gate_up, int n_splits, const float* row_ss, int ss_splits, int hidden, float eps,
+                           void* out, int n_tokens, int inter, int dtype, void* stream) {
     if (!gate_up || !out || n_tokens < 0 || inter <= 0 || n_splits < 0) return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t total = static_cast<size_t>(n_tokens) * inter;
     const int blocks = static_cast<int>(total / 256 + 1 > 8192 ? 8192 : total / 256 + 1);
     const size_t stride = total * 2;
+    if (row_ss) {
+        // float32 partial sums with a pending row factor
+        if (n_splits < 1 || ss_splits < 1 || hidden <= 0 || n_tokens > 65535 || (dtype != 0 && dtype != 1))
+            return EGPT_BAD_ARGUMENT;
+        const dim3 grid(static_cast<unsigned>((inter + 255) / 256 > 64 ? 64 : (inter + 255) / 256),
+                        static_cast<unsigned>(n_tokens));
+        const ProductView<float> view = make_view<float>(gate_up, n_splits, stride);
+        if (dtype == 0)
+            swiglu_scaled_kernel<float><<<grid, 256, 0, s>>>(view, row_ss, ss_splits, 1.0f / hidden, eps,
+                                                             static_cast<float*>(out), n_tokens, inter);
+        else
+            swiglu_scaled_kernel<bf16_t><<<grid, 256, 0, s>>>(view, row_ss, ss_splits, 1.0f / hidden, eps,
+                                                              static_cast<bf16_t*>(out), n_tokens, inter);
+        EGPT_CHECK_LAUNCH();
+        return EGPT_OK;
+    }
     if (dtype == 1 && n_splits <= 1 && inter % 8 == 0) {
         const size_t chunks = total / 8;
         const int vblocks = static_cast<int>(chunks / 256 + 1 > 16384 ? 16384 : chunks / 256 + 1);
@@ -518,4 +551,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 7; }
+extern "C" int egpt_abi_version(void) { return 8; }

@@ -135,7 +135,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
     const int step_end = min(total_steps, step_begin + a.steps_per_split);
     const int n_steps = step_end - step_begin;
     const int w_row = min(n0 + li, n - 1);
-    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + lg * 32;
+    // lane group lg takes the lg-th 16 bytes of each 64 of a row: the four groups of a load instruction read 64
+    // contiguous bytes of each of its 16 rows (a memory request is 64 bytes wide; x is read from LDS the same way)
+    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + lg * 8;
 
     f32x4 acc[MT];
 #pragma unroll
@@ -143,9 +145,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
 
     uint4 a_cur[4], a_next[4];
     auto load_w = [&](uint4* av, int step) {
-        const int k0 = step * kStep + lg * 32;
+        const int k0 = step * kStep + lg * 8;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) av[q] = load16(wp + static_cast<size_t>(step) * kStep + q * 8, k0 + q * 8 < k);
+        for (int q = 0; q < 4; ++q) av[q] = load16(wp + static_cast<size_t>(step) * kStep + q * 32, k0 + q * 32 < k);
     };
     // the stream of w starts before anything else
     if (n_steps > 0) load_w(a_cur, step_begin);
@@ -334,7 +336,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
             const bf16x8 av = __builtin_bit_cast(bf16x8, av4[q]);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const uint4 bv = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + li][lg * 32 + q * 8]);
+                const uint4 bv = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + li][q * 32 + lg * 8]);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
             }
         }
@@ -438,7 +440,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_resident_kernel(SkinnyArgs a) {
     const int n_steps = min(total_steps, step_begin + a.steps_per_split) - step_begin;       // <= kResidentSteps
     const int k_begin = step_begin * kStep;
     const int w_row = min(n0 + li, n - 1);
-    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + k_begin + lg * 32;
+    const bf16_t* wp = a.w + static_cast<size_t>(w_row) * k + k_begin + lg * 8;
 
     // the whole stream of w for this workgroup
     uint4 av[kResidentSteps][4];
@@ -446,7 +448,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_resident_kernel(SkinnyArgs a) {
     for (int s = 0; s < kResidentSteps; ++s)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            av[s][q] = load16(wp + s * kStep + q * 8, s < n_steps && k_begin + s * kStep + lg * 32 + q * 8 < k);
+            av[s][q] = load16(wp + s * kStep + q * 32, s < n_steps && k_begin + s * kStep + q * 32 + lg * 8 < k);
     // x: sixteen threads per row take its sixteen chunks of a step; a thread walks the steps of a row (all its
     // loads in flight together), then the next of its rows.  No division in any index: with a vector
     // instruction at four cycles, index arithmetic is what such a kernel would otherwise spend its time on.
@@ -478,7 +480,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_resident_kernel(SkinnyArgs a) {
             const bf16x8 wv = __builtin_bit_cast(bf16x8, av[s][q]);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const uint4 bv = *reinterpret_cast<const uint4*>(&xs[t * 16 + li][s * kStep + lg * 32 + q * 8]);
+                const uint4 bv = *reinterpret_cast<const uint4*>(&xs[t * 16 + li][s * kStep + q * 32 + lg * 8]);
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, __builtin_bit_cast(bf16x8, bv), acc[t], 0, 0, 0);
             }
         }

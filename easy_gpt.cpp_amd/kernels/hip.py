@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 7:
+    if lib.egpt_abi_version() != 8:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -59,7 +59,7 @@ class HipKernels:
         sigs = {
             "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
             "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
-            "egpt_swiglu": [vp, i, vp, i, i, i, vp],
+            "egpt_swiglu": [vp, i, vp, i, i, f, vp, i, i, i, vp],
             "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_rope_table": [vp, vp, vp, i, i, vp],
             "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, vp],
@@ -170,6 +170,20 @@ class HipKernels:
         self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), splits, t, rows.data_ptr(), weight.data_ptr(),
                   float(eps), out.data_ptr(), r, hid, dt, self._stream())
 
+    @staticmethod
+    def _library_rows(m: int, n: int, k: int) -> bool:
+        """Whether a bfloat16 product of m rows goes to the library (the reference uses cuBLAS for every linear
+        layer).  Up to 16 rows never, beyond 64 always.  Between them the own kernels win where the k range
+        has to be split over workgroups (an output narrower than k) and on small matrices, where a step is a
+        chain of round trips to memory; the library wins on large ones, which it streams at 4 to 5 TB/s."""
+        if m <= 16:
+            return False
+        if m > 64:
+            return True
+        if n < k:
+            return False
+        return n * k >= (2 << 20 if m > 32 else 16 << 20)
+
     def linear(self, x, w, bias, out):
         m, k = x.shape
         n = w.shape[0]
@@ -185,20 +199,19 @@ class HipKernels:
             return out
         if x.dtype == _BF16 and k % 8 == 0:
             to_f32 = out.dtype == _F32
-            if m <= 64 or to_f32:
-                # weight-streaming MFMA kernel; more than 64 rows with float32 output (logits at many places)
-                # go through it 64 rows at a time
-                for r0 in range(0, m, 64):
-                    r1 = min(m, r0 + 64)
-                    xo, oo = x[r0:r1], out[r0:r1]
-                    # (a very wide output with more than one tile of rows: workgroups of 8 wavefronts stage x half
-                    # as often)
-                    self._run("egpt_gemm_skinny", xo.data_ptr(), w.data_ptr(), self._ptr(bias),
-                              oo.data_ptr() if to_f32 else None, None if to_f32 else oo.data_ptr(), r1 - r0, n, k, 1,
-                              8 if (r1 - r0 > 16 and n >= 65536) else 4, self._stream())
+            if not self._library_rows(m, n, k):
+                # weight-streaming MFMA kernel (a very wide output with more than one tile of rows: workgroups
+                # of 8 wavefronts stage x half as often)
+                self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), self._ptr(bias),
+                          out.data_ptr() if to_f32 else None, None if to_f32 else out.data_ptr(), m, n, k, 1,
+                          8 if (m > 16 and n >= 65536) else 4, self._stream())
                 return out
-            # many rows: the library's matrix product (the reference uses cuBLAS for every linear layer)
-            if bias is None:
+            # many rows: the library's matrix product; float32 output (logits) unrounded
+            if to_f32:
+                torch.mm(x, w.t(), out_dtype=_F32, out=out)
+                if bias is not None:
+                    out += bias
+            elif bias is None:
                 torch.mm(x, w.t(), out=out)
             else:
                 torch.addmm(bias, x, w.t(), out=out)
@@ -221,13 +234,35 @@ class HipKernels:
 
     fused_rows = 16     # products with a computed x operand take at most this many rows
 
-    def product_normed(self, h, delta, norm_weight, w, waves=4, splits=None):
+    @staticmethod
+    def _normed_shape(n: int, k: int) -> tuple[int, int]:
+        """(splits of the k range, wavefronts per workgroup) of the product with the norm folded in.  Two steps of
+        128 per workgroup are staged at once, which is the kernel's shortest chain of round trips; one step where
+        the matrix is so small that this leaves the GPU short of workgroups.  Every workgroup computes its share
+        of x again, so where the columns allow it workgroups are wide (their wavefronts share the staged x)."""
+        steps = -(-k // 128)
+        per = max(2, -(-steps // 20))
+        if -(-n // 64) * -(-steps // per) < 192:
+            per = max(1, -(-steps // 20))
+        s = -(-steps // per)
+        waves = 4
+        for wide in (16, 8):
+            if -(-n // (16 * wide)) * s >= 400:
+                waves = wide
+                break
+        return s, waves
+
+    def product_normed(self, h, delta, norm_weight, w, waves=None, splits=None):
         """((h + delta) * norm_weight) w^T without the rows' 1/rms factor, for few rows in bfloat16.
         Returns (float32 partial sums [S, T, N], row sums of squares [S, T], h + delta as a new tensor),
-        or None if this case is not covered (the caller then runs the norm by itself)."""
+        or None if this case is not covered or not worth it (the caller then runs the norm by itself)."""
         t, k = h.shape
         n = w.shape[0]
         if w.dtype != _BF16 or not 0 < t <= self.fused_rows or k % 8 or not h.is_cuda:
+            return None
+        if splits is None and waves is None and t * n > 400_000:
+            # every workgroup reads its k range of all rows of h and delta: with this many rows and columns that
+            # is more than a norm kernel of its own costs (measured at 16 rows of a 37,888-column product)
             return None
         if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
             return None
@@ -238,7 +273,8 @@ class HipKernels:
         if delta is not None:
             d_splits = int(delta.shape[0])
             self._need(delta, "delta", _F32, (d_splits, t, k))
-        s = splits or self._n_splits(t, n, k)
+        auto_s, auto_w = self._normed_shape(n, k)
+        s, waves = splits or auto_s, waves or auto_w
         out = torch.empty((s, t, n), dtype=_F32, device=h.device)
         ss = torch.empty((s, t), dtype=_F32, device=h.device)
         h_new = torch.empty_like(h)
@@ -254,6 +290,11 @@ class HipKernels:
         g_splits, t, two_i = gate_up.shape
         n, k = w.shape
         if two_i != 2 * k or not 0 < t <= self.fused_rows or k % 8:
+            return None
+        if waves is None and n >= 3072:
+            # every workgroup computes its share of x from gate_up's partial sums, and with this many columns there
+            # are dozens of workgroups per share: a SwiGLU kernel of its own and the plain product are faster
+            # (measured at 3,584 columns: 35 us against 53)
             return None
         self._need(gate_up, "gate_up", _F32)
         self._need(w, "w", _BF16)
@@ -273,7 +314,7 @@ class HipKernels:
                   float(eps), w.data_ptr(), out.data_ptr(), t, n, k, s, waves, self._stream())
         return out
 
-    def product_attention(self, part_o, part_ml, w, max_splits=4, waves=4):
+    def product_attention(self, part_o, part_ml, w, max_splits=None, waves=None):
         """(combined attention output) w^T from the parts of a split attention: part_o [S, T, nq, hd],
         part_ml [S, T, nq, 2].  Returns float32 partial sums [S2, T, N] or None if not covered."""
         a_splits, t, nq, hd = part_o.shape
@@ -283,6 +324,12 @@ class HipKernels:
         self._need(part_o, "part_o", _F32)
         self._need(part_ml, "part_ml", _F32, (a_splits, t, nq, 2))
         self._need(w, "w", _BF16)
+        # a short k range: few splits, whose partial sums the next product's prologue adds up in registers; a
+        # long one: a step of 128 per workgroup, and workgroups of 8 wavefronts that share the combined x
+        if max_splits is None:
+            max_splits = 4 if k <= 1024 else 14
+        if waves is None:
+            waves = 4 if k <= 1024 else 8
         s = min(self._n_splits(t, n, k), max_splits)
         steps = -(-k // 128)
         per = -(-steps // s)
@@ -311,7 +358,7 @@ class HipKernels:
         in between is the largest single contribution to the bfloat16 error of the logits."""
         m, k = x.shape
         n = w.shape[0]
-        if x.dtype == _BF16 and 0 < m <= 64 and k % 8 == 0:
+        if x.dtype == _BF16 and m > 0 and k % 8 == 0 and not self._library_rows(m, n, k):
             self._need(x, "x")
             self._need(w, "w", x.dtype, (n, k))
             s = self._n_splits(m, n, k)
@@ -324,7 +371,7 @@ class HipKernels:
             self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s, 4,
                       self._stream())
             return out
-        if unrounded and x.dtype == _BF16 and m > 64 and k % 8 == 0:
+        if unrounded and x.dtype == _BF16 and m > 0 and k % 8 == 0:
             # many rows: the library's product (the reference uses cuBLAS for every linear layer), written out in
             # float32; it goes on as a single "partial sum" [1, m, n]
             self._need(x, "x")
@@ -508,12 +555,21 @@ class HipKernels:
                   int(window), n_splits, n_waves, 1 if combine else 0, self._stream())
         return (part_o, part_ml) if (n_splits > 1 and not combine) else None
 
-    def swiglu(self, gate_up, out):
+    def swiglu(self, gate_up, out, row_ss=None, hidden=0, eps=0.0):
+        """out = up * silu(gate) for gate_up act [T, 2I] or float32 partial sums [S, T, 2I].  row_ss float32
+        [S2, T]: the partial sums still lack each row's factor 1/sqrt(sum_s row_ss[s] / hidden + eps)."""
         t, inter = out.shape
         dt = self._act(out, "out")
         splits = self._product(gate_up, "gate_up", out.dtype, t, 2 * inter)
         self._need(out, "out")
-        self._run("egpt_swiglu", gate_up.data_ptr(), splits, out.data_ptr(), t, inter, dt, self._stream())
+        ss_splits = 0
+        if row_ss is not None:
+            if splits < 1:
+                raise ValueError("a pending row factor needs float32 partial sums")
+            ss_splits = int(row_ss.shape[0])
+            self._need(row_ss, "row_ss", _F32, (ss_splits, t))
+        self._run("egpt_swiglu", gate_up.data_ptr(), splits, self._ptr(row_ss), ss_splits, int(hidden), float(eps),
+                  out.data_ptr(), t, inter, dt, self._stream())
 
     def argmax(self, logits, out):
         r, v = logits.shape

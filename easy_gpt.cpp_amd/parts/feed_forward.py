@@ -54,9 +54,12 @@ class SwiGLU(FeedForward):
                 gate_up, row_ss, h_new = fused
                 x.applied(h_new)
                 out = k.product_swiglu(gate_up, row_ss, self.hidden_size, rms[1], self.w_down)
-                if out is None:
-                    raise RuntimeError("the fused SwiGLU product does not cover this size")
-                return out
+                if out is not None:
+                    return out
+                # SwiGLU by itself; it applies the rows' pending 1/rms factor
+                act = torch.empty((h_new.shape[0], self.intermediate_size), dtype=self.w_down.dtype, device=h_new.device)
+                k.swiglu(gate_up, act, row_ss=row_ss, hidden=self.hidden_size, eps=rms[1])
+                return k.product(act, self.w_down)
             x = x.materialize()
         t = x.shape[0]
         gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]

@@ -95,6 +95,10 @@ def test_skinny_product_and_partial_sums(k, m, n, kk):
     ref = plain.linear(x.double().cpu(), w.double().cpu())
     scale = float(ref.abs().max())
     prod = k.product(x, w)
+    if k._library_rows(m, n, kk):        # more than 16 rows of a large matrix without a split k range: the library
+        assert prod.dtype == dtype and prod.shape == (m, n)
+        assert float((prod.double().cpu() - ref).abs().max()) <= 1e-2 * scale
+        prod = k.product(x, w, unrounded=True)
     assert prod.dtype == torch.float32 and prod.dim() == 3 and prod.shape[1:] == (m, n)
     assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale
     for s in sorted({1, 2, min(3, -(-kk // 128)), -(-kk // 128)}):
@@ -113,6 +117,17 @@ def test_skinny_product_and_partial_sums(k, m, n, kk):
     k.linear(x, w, b, out16)
     with_bias = ref + b.double().cpu()
     assert float((out16.double().cpu() - with_bias).abs().max()) <= 1e-2 * float(with_bias.abs().max())   # one bfloat16 rounding
+
+
+def test_which_products_go_to_the_library():
+    from easy_gpt.cpp_amd.kernels.hip import HipKernels
+
+    lib = HipKernels._library_rows
+    assert not lib(16, 151936, 896) and lib(65, 64, 64)                   # up to 16 rows never, beyond 64 always
+    assert lib(64, 9728, 896) and lib(33, 151936, 896) and lib(17, 151936, 896)
+    assert not lib(64, 896, 4864) and not lib(17, 3584, 18944)            # split-k shapes stay with the own kernels
+    assert not lib(32, 9728, 896) and lib(32, 17920, 1536)                # small matrices with up to 32 rows, too
+    assert not lib(64, 1152, 896) and lib(64, 4608, 3584)
 
 
 def test_consumers_add_partial_sums_up(k):
@@ -158,7 +173,8 @@ def test_consumers_add_partial_sums_up(k):
     assert torch.equal(vc[3, :, :, 2], got.view(t, -1, hd)[3, nq + nkv :])
 
 
-@pytest.mark.parametrize("t,hid,n,d_splits", [(1, 896, 1152, 0), (8, 896, 9728, 4), (16, 200, 130, 3), (5, 1536, 2048, 13)])
+@pytest.mark.parametrize("t,hid,n,d_splits", [(1, 896, 1152, 0), (8, 896, 9728, 4), (16, 200, 130, 3), (5, 1536, 2048, 13),
+                                              (8, 3584, 4608, 19), (3, 1536, 17920, 12), (16, 256, 26000, 2)])
 def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
     # ((h + delta) * norm_weight) w^T with the rows' 1/rms applied afterwards equals rmsnorm(h + delta) w^T
     dtype = torch.bfloat16
@@ -175,10 +191,14 @@ def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
     ref = plain.linear(plain.rms_norm(sd, nw.double().cpu(), eps), w.double().cpu())
     # every workgroup width; the k range in as many pieces as the wrapper likes (short ranges, staged at once),
     # in one piece and in two (long ranges, staged step by step)
-    for waves, splits in ((4, None), (8, None), (16, None), (4, 1), (16, 1), (8, 2)):
+    for waves, splits in ((None, None), (4, None), (8, None), (16, None), (4, 1), (16, 1), (8, 2)):
         if splits and splits > -(-hid // 128):
             continue
-        prod, ss, h_new = k.product_normed(h, delta, nw, w, waves=waves, splits=splits)
+        fused = k.product_normed(h, delta, nw, w, waves=waves, splits=splits)
+        if fused is None:                # many rows times many columns: left to a norm kernel of its own
+            assert waves is None and t * n > 400_000
+            continue
+        prod, ss, h_new = fused
         assert torch.equal(h, h0)                                           # the input stream is left alone
         assert torch.equal(h_new, summed)
         assert torch.allclose(ss.double().sum(0).cpu(), (sd * sd).sum(-1), rtol=1e-5)
@@ -197,7 +217,8 @@ def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
         assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())   # position 0: no rotation
 
 
-@pytest.mark.parametrize("t,inter,n,g_splits", [(8, 4864, 896, 4), (3, 200, 120, 1), (16, 328, 192, 2), (7, 640, 100, 6)])
+@pytest.mark.parametrize("t,inter,n,g_splits", [(8, 4864, 896, 4), (3, 200, 120, 1), (16, 328, 192, 2), (7, 640, 100, 6),
+                                                (5, 1000, 3080, 3)])
 def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
     gu = rnd(g_splits, t, 2 * inter, seed=1, scale=1.5)
     ss = torch.rand(3, t, generator=torch.Generator().manual_seed(2)).to(DEV) * 50 + 1
@@ -208,8 +229,16 @@ def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
         z = gu.double().sum(0).cpu() * scale
         g, u = z[:, :inter], z[:, inter:]
         ref = plain.linear(u * g / (1 + torch.exp(-g)), w.double().cpu())
-        for waves, max_splits in ((4, 20), (8, 20), (16, 20), (4, 1), (16, 2)):      # short and long k ranges
+        for waves, max_splits in ((None, 20), (4, 20), (8, 20), (16, 20), (4, 1), (16, 2)):      # short and long k ranges
             prod = k.product_swiglu(gu, row_ss, hidden, eps, w, max_splits=max_splits, waves=waves)
+            if prod is None:             # many columns: SwiGLU by itself, with the rows' factor, then the plain product
+                assert waves is None and n >= 3072
+                act = torch.empty(t, inter, dtype=torch.bfloat16, device=DEV)
+                k.swiglu(gu, act, row_ss=row_ss, hidden=hidden, eps=eps)
+                prod = k.product(act, w)
+                act32 = torch.empty(t, inter, dtype=torch.float32, device=DEV)
+                k.swiglu(gu, act32, row_ss=row_ss, hidden=hidden, eps=eps)
+                assert float((act32.double().cpu() - u * g / (1 + torch.exp(-g))).abs().max()) <= 3e-6 * float((u * g).abs().max())
             assert prod is not None and prod.dim() == 3
             assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, max_splits)
 
@@ -238,10 +267,10 @@ def test_output_projection_combines_attention_parts(k, nq, nkv, hd, batch, ctx):
     assert float((again.float() - out.float()).abs().max()) <= 2e-2      # other splits, other rounding
     w = rnd(200, nq * hd, dtype=dtype, seed=7, scale=0.05)
     ref = plain.linear(again.double().cpu(), w.double().cpu())
-    for waves, max_splits in ((4, 4), (8, 4), (16, 4), (4, 1), (8, 2)):
+    for waves, max_splits in ((None, None), (4, 4), (8, 4), (16, 4), (4, 1), (8, 2), (8, 14)):
         prod = k.product_attention(parts[0], parts[1], w, max_splits=max_splits, waves=waves)
         if prod is None:             # a long k range over too many heads
-            assert max_splits < 4
+            assert max_splits is not None and max_splits < 4
             continue
         assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, max_splits)
 
