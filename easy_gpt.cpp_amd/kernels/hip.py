@@ -260,9 +260,10 @@ class HipKernels:
         n = w.shape[0]
         if w.dtype != _BF16 or not 0 < t <= self.fused_rows or k % 8 or not h.is_cuda:
             return None
-        if splits is None and waves is None and t * n > 400_000:
-            # every workgroup reads its k range of all rows of h and delta: with this many rows and columns that
-            # is more than a norm kernel of its own costs (measured at 16 rows of a 37,888-column product)
+        if splits is None and waves is None and (t * n > 400_000 or n * k >= 64 << 20):
+            # every workgroup reads its k range of all rows of h and of delta's partial sums: on a matrix this large
+            # (or with this many rows and columns) that costs more than a norm kernel of its own (measured on a
+            # 37,888 x 3,584 product behind 14 partial sums: 80 us against 6 + 58)
             return None
         if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
             return None
@@ -291,10 +292,10 @@ class HipKernels:
         n, k = w.shape
         if two_i != 2 * k or not 0 < t <= self.fused_rows or k % 8:
             return None
-        if waves is None and n >= 3072:
+        if waves is None and n >= 1536:
             # every workgroup computes its share of x from gate_up's partial sums, and with this many columns there
             # are dozens of workgroups per share: a SwiGLU kernel of its own and the plain product are faster
-            # (measured at 3,584 columns: 35 us against 53)
+            # (measured inside the model at 8 rows: 15 us against 17 at 1,536 columns, 37 against 54 at 3,584)
             return None
         self._need(gate_up, "gate_up", _F32)
         self._need(w, "w", _BF16)
