@@ -45,6 +45,51 @@ OTHER_SHAPES = {
 }
 
 
+SERVE_REQUESTS, SERVE_NEW_TOKENS, SERVE_CHUNK = 64, 256, 512
+
+
+def serve_workload(engine, name: str, args, vocab: int) -> int:
+    """64 requests, submitted together, prompt lengths uniform in [128, 2048], 256 new tokens each (greedy, end token
+    ignored), through the scheduler with prompts in portions of 512 tokens: total tokens a second."""
+    import random
+
+    import torch
+
+    from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    rnd = random.Random(0)
+    lens = [rnd.randint(128, 2048) for _ in range(SERVE_REQUESTS)]
+    g = torch.Generator().manual_seed(0)
+    results = []
+    for rep in range(2):                                       # the first pass warms up (graphs, library choices)
+        sched = Scheduler(engine, SchedulerConfig(max_active=SERVE_REQUESTS, max_admit_per_step=8, max_tokens_per_step=2048,
+                                                  prefill_chunk=SERVE_CHUNK), eos_token_id=-1)
+        for i, n in enumerate(lens):
+            sched.add(Request(f"s{rep}_{i}", torch.randint(0, vocab, (n,), generator=g).tolist(), SamplingParams(greedy=True),
+                              max_new_tokens=SERVE_NEW_TOKENS, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while sched.has_work():
+            sched.step()
+        torch.cuda.synchronize()
+        results.append((time.perf_counter() - t0, sched.stats))
+        print(f"[bench] serve pass {rep}: {results[-1][0]:.2f} s, {sched.stats.steps} steps", file=sys.stderr, flush=True)
+    sec, st = results[-1]
+    total = sum(lens) + SERVE_REQUESTS * SERVE_NEW_TOKENS
+    print(json.dumps({
+        "metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(total / sec, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(sec / st.steps * 1e3, 3),
+        "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "generated_per_s": round(SERVE_REQUESTS * SERVE_NEW_TOKENS / sec, 1), "seconds": round(sec, 3),
+        "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
+        "config": {"model": f"{name} layer sizes", "requests": SERVE_REQUESTS, "prompt_tokens": sum(lens),
+                   "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": SERVE_CHUNK, "max_tokens_per_step": 2048,
+                   "preemptions": st.preemptions, "sampling": "greedy"},
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -56,9 +101,13 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prefix", type=int, default=None,
                     help="tokens each request holds before decoding starts (default: the record's 2,048)")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--serve", action="store_true",
+                    help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
+                         "each through the scheduler, prompts in portions of 512 (a workload of the baseline record)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
@@ -94,7 +143,7 @@ def main() -> int:
                                 cfg["intermediate_size"], cfg["vocab_size"])
     hd = h // nq
     layers = args.layers
-    page_size = 16
+    page_size = args.page_size
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
 
@@ -103,6 +152,8 @@ def main() -> int:
     write_random_model(tmp, cfg, seed=0, dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
     new_tokens = max(NEW_TOKENS, args.warmup + args.steps)        # a longer run than the record's decodes further
     tokens_per_request = -(-(PREFIX + new_tokens) // page_size) * page_size
+    if args.serve:
+        max_batch, tokens_per_request = SERVE_REQUESTS, -(-(2048 + SERVE_NEW_TOKENS) // page_size) * page_size
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
                              max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1)
     for f in os.listdir(tmp):
@@ -112,6 +163,9 @@ def main() -> int:
     greedy = SamplingParams(greedy=True)
     g = torch.Generator().manual_seed(0)
     print(f"[bench] model ready in {time.time() - t_setup:.1f} s", file=sys.stderr, flush=True)
+
+    if args.serve:
+        return serve_workload(engine, name, args, vocab)
 
     # per-step work of the model, for the rooflines
     layer_weights = (h * (nq + 2 * nkv) * hd + (nq + 2 * nkv) * hd + nq * hd * h + 3 * h * inter + 2 * h) * elem
