@@ -133,6 +133,39 @@ def test_decoding_across_the_context_steps_of_the_captured_graphs(sharp_models, 
     assert len({key[2] for key in eng._decode_plans}) >= 2 and len({key[1] for key in eng._decode_plans}) >= 2
 
 
+def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph(tmp_path):
+    # 40 requests decoded side by side in a model whose gate/up and output matrices are wide enough for the library's
+    # product at this many rows: the captured graph then holds library nodes, is replayed step after step with the
+    # program's own work in between, and every replay is compared with the plain implementation
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    cfg = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 256,
+        "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 4112, "vocab_size": 8300,
+        "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 64,
+    }
+    kernels.use_backend(None)
+    k = kernels.backend()
+    assert k._library_rows(40, 2 * 4112, 256) and k._library_rows(40, 8300, 256) and not k._library_rows(40, 256, 4112)
+    sharp = str(tmp_path)              # plain random weights: this test is about the replays, not about far keys
+    write_random_model(sharp, cfg, seed=9)
+    n_req, prompt, steps = 40, 9, 7
+    reqs = H.make_requests(cfg["vocab_size"], [prompt + steps + i % 3 for i in range(n_req)], seed=61)
+    ref = H.plain_rows(sharp, reqs, bf16_weights=True)
+    ids = list(reqs)
+    trace = [H.step_record(0, [(rid, reqs[rid][:prompt + i % 3], [prompt + i % 3 - 1]) for i, rid in enumerate(ids)])]
+    for s in range(steps):
+        trace.append(H.step_record(1 + s, [(rid, [reqs[rid][prompt + i % 3 + s]], [0]) for i, rid in enumerate(ids)],
+                                   ids if s == steps - 1 else []))
+    eng = engine_for(sharp, "bfloat16", max_tokens=n_req * 64, max_requests=n_req)
+    rows = H.replay(eng, trace)
+    assert len(rows) == n_req * (1 + steps)
+    H.assert_rows_match(rows, ref, H.BF16_TOL, "library products in the decode graph")
+    plans = list(eng._decode_plans.values())
+    assert len(plans) == 1 and plans[0].graph is not None          # two eager visits, then replays
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens_of_a_sequence(tiny_models, name, dtype):
