@@ -366,6 +366,40 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
             if (blockIdx.x == 0 && tid < m)
                 a.ss_out[split * m + tid] = (n_steps > 0 ? ss_part[0][tid] : 0.f) + (n_steps > 1 ? ss_part[1][tid] : 0.f);
         }
+    } else if constexpr (PRO == kPlain) {
+        // A long range of a given x: double-buffered in LDS, and on its way through registers a step before that:
+        // the loads of step + 2 are issued when step + 1 has been written to LDS, so that a step does not wait for
+        // its own x (with 64 rows that wait was a third of the kernel's time).
+        constexpr int kChunks = (MT * 16 * 16 + kThreads - 1) / kThreads;
+        uint4 xr[kChunks];
+        auto x_load = [&](int step) {
+#pragma unroll
+            for (int j = 0; j < kChunks; ++j) {
+                const int c = tid + j * kThreads, r = c / 16, kc = step * kStep + (c % 16) * 8;
+                xr[j] = load16(a.x + static_cast<size_t>(min(r, m - 1)) * k + kc, r < m && kc < k);
+            }
+        };
+        auto x_store = [&](int buf) {
+#pragma unroll
+            for (int j = 0; j < kChunks; ++j) {
+                const int c = tid + j * kThreads;
+                if (c < MT * 16 * 16) *reinterpret_cast<uint4*>(&xs[buf][c / 16][(c % 16) * 8]) = xr[j];
+            }
+        };
+        x_load(step_begin);
+        x_store(0);
+        x_load(step_begin + 1);                   // n_steps > 2 here
+        __syncthreads();
+        for (int step = step_begin; step < step_end; ++step) {
+            const int buf = (step - step_begin) & 1;
+            if (step > step_begin && step + 1 < step_end) load_w(a_next, step + 1);
+            products(buf, a_cur);
+            if (step + 1 < step_end) x_store(buf ^ 1);
+            if (step + 2 < step_end) x_load(step + 2);
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) a_cur[q] = a_next[q];
+        }
     } else {
         // A long range: x double-buffered in LDS, a thread keeps its (row, column) over the steps.
         float ss_acc = 0.f;

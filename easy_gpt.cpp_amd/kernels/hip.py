@@ -228,7 +228,9 @@ class HipKernels:
         n_blocks = -(-n // 64)
         # a long k range is worth more workgroups: each one's stream is a chain of steps, one load ahead
         most = 2048 if steps >= 14 else 1024
-        s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20)
+        # more than one tile of rows: x weighs as much as w in every workgroup and the partial sums more than with
+        # few rows, so fewer, longer ranges (their x travels through registers a step ahead)
+        s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20 if m <= 16 else 10)
         per = -(-steps // s)
         return -(-steps // per)
 
