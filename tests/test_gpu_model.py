@@ -166,6 +166,38 @@ def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph
     assert len(plans) == 1 and plans[0].graph is not None          # two eager visits, then replays
 
 
+def test_a_layer_with_large_matrices_takes_the_kernels_that_are_not_folded(tmp_path):
+    # one layer whose gate/up matrix has 67M elements and whose width is 2,048: with few rows the norm before gate/up
+    # and SwiGLU before down then run as kernels of their own (folded into the products they would be computed again
+    # by hundreds of workgroups), the QKV and output projections keep their folded prologues with wide workgroups
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    cfg = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 1, "hidden_size": 2048,
+        "num_attention_heads": 16, "num_key_value_heads": 2, "intermediate_size": 16384, "vocab_size": 600,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 128,
+    }
+    kernels.use_backend(None)
+    k = kernels.backend()
+    h = torch.zeros(3, 2048, device="cuda")
+    nw = torch.ones(2048, dtype=torch.bfloat16, device="cuda")
+    big = torch.zeros(2 * 16384, 2048, dtype=torch.bfloat16, device="cuda")
+    assert k.product_normed(h, None, nw, big) is None and k.product_normed(h, None, nw, big[:2560]) is not None
+    del big
+    write_random_model(str(tmp_path), cfg, seed=12)
+    reqs = H.make_requests(cfg["vocab_size"], [40, 23, 31], seed=71)
+    ref = H.plain_rows(str(tmp_path), reqs, bf16_weights=True)
+    ids = list(reqs)
+    trace = [H.step_record(0, [(rid, reqs[rid][:-6], [len(reqs[rid]) - 7]) for rid in ids])]
+    for s in range(6):
+        trace.append(H.step_record(1 + s, [(rid, [reqs[rid][len(reqs[rid]) - 6 + s]], [0]) for rid in ids], ids if s == 5 else []))
+    eng = engine_for(str(tmp_path), "bfloat16", max_tokens=256)
+    rows = H.replay(eng, trace)
+    assert len(rows) == 3 * 7
+    H.assert_rows_match(rows, ref, H.BF16_TOL, "large matrices, few rows")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens_of_a_sequence(tiny_models, name, dtype):
