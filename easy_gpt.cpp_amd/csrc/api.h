@@ -37,6 +37,10 @@ int egpt_rope_table(const int32_t* positions, const float* inv_freq, float* cos_
 // waves: wavefronts (of 16 columns of the result each) per workgroup, 4, 8 or 16; here and below.
 int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m, int n,
                      int k, int n_splits, int waves, void* stream);
+// float32 product on the matrix cores (float32 operands and accumulation): out [n_splits][m][n] are partial sums over
+// n_splits ranges of k (bias only with one).  k % 4 == 0.  A row's values do not depend on m or on the other rows.
+int egpt_gemm_f32(const float* x, const float* w, const float* bias, float* out, int m, int n, int k, int n_splits,
+                  void* stream);
 // out = x w^T + bias; x [m,k], w [n,k], out [m,n]; out_f32 != 0 writes float32 whatever dtype is.
 int egpt_linear(const void* x, const void* w, const void* bias, void* out, int m, int n, int k, int dtype,
                 int out_f32, void* stream);

@@ -24,18 +24,25 @@ __device__ __forceinline__ int find_request(const int32_t* q_start, int n_seqs, 
     return lo;
 }
 
-// One wavefront per (token, query head).  Keys are taken 64 at a time: each lane scores one key, the
-// wave agrees on the new maximum, then each lane owns head features lane, lane+64, ... of the output.
+// One workgroup of kGenericWaves wavefronts per (token, query head).  Keys are taken 64 at a time, a chunk of 64
+// by the wavefront whose number is the chunk's number modulo kGenericWaves: each lane scores one key, the wavefront
+// agrees on the new maximum, then each lane owns head features lane, lane+64, ... of the output.  At the end the
+// wavefronts' running (maximum, sum, output) are merged in the order of their numbers.  Which wavefront takes which
+// keys depends on the keys' positions alone, so a token's result is the same bits however the work was cut into
+// steps and whatever else is in the batch.
+constexpr int kGenericWaves = 8;
+
 template <typename T>
-__global__ __launch_bounds__(64) void paged_attention_generic_kernel(
+__global__ __launch_bounds__(64 * kGenericWaves) void paged_attention_generic_kernel(
     const T* __restrict__ qkv, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int nq, int nkv, int hd,
     int page_size, float scale, int window) {
+    constexpr int kMaxOwn = kMaxHeadDim / kWave;
     __shared__ float q_s[kMaxHeadDim];
-    __shared__ float p_s[kWave];
-    __shared__ long v_off_s[kWave];
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    __shared__ float part_ml[kGenericWaves][2];
+    __shared__ float part_o[kGenericWaves][kMaxHeadDim];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int b = find_request(q_start, n_seqs, t);
     const int i = t - q_start[b];
     const int p = kv_len[b] - q_len[b] + i;
@@ -44,13 +51,12 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const int kvh = h / (nq / nkv);
     const int row_width = (nq + 2 * nkv) * hd;
     const T* q = qkv + static_cast<size_t>(t) * row_width + h * hd;
-    for (int d = lane; d < hd; d += kWave) q_s[d] = to_float(q[d]);
+    for (int d = threadIdx.x; d < hd; d += kWave * kGenericWaves) q_s[d] = to_float(q[d]);
     __syncthreads();
     const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
-    constexpr int kMaxOwn = kMaxHeadDim / kWave;
     float acc[kMaxOwn] = {};
     float m_run = -INFINITY, l_run = 0.f;
-    for (int c = lo; c < hi; c += kWave) {
+    for (int c = lo + wave * kWave; c < hi; c += kWave * kGenericWaves) {
         const int j = c + lane;
         float s = -INFINITY;
         long off = 0;
@@ -65,31 +71,51 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
         }
         const float m_new = fmaxf(m_run, wave_max(s));   // finite: key c is always visible
         const float pj = j < hi ? expf(s - m_new) : 0.f;
-        const float alpha = expf(m_run - m_new);          // exp(-inf) = 0 on the first chunk
+        const float alpha = expf(m_run - m_new);          // exp(-inf) = 0 on the wavefront's first chunk
         l_run = l_run * alpha + wave_sum(pj);
         m_run = m_new;
-        p_s[lane] = pj;
-        v_off_s[lane] = off;
-        __syncthreads();
         const int n_valid = min(kWave, hi - c);
 #pragma unroll
-        for (int r = 0; r < kMaxOwn; ++r) {
-            const int d = lane + r * kWave;
-            if (d < hd) {
-                float a = acc[r] * alpha;
-                for (int jj = 0; jj < n_valid; ++jj)
-                    a = fmaf(p_s[jj], to_float(v_cache[v_off_s[jj] + static_cast<long>(d) * page_size]), a);
-                acc[r] = a;
+        for (int r = 0; r < kMaxOwn; ++r) acc[r] *= alpha;
+        // every lane needs every key's weight and place: handed round from the lane that holds them
+        for (int jj = 0; jj < n_valid; ++jj) {
+            const float pw = __shfl(pj, jj, kWave);
+            const long vo = (static_cast<long>(__shfl(static_cast<int>(off >> 32), jj, kWave)) << 32) |
+                            static_cast<unsigned int>(__shfl(static_cast<int>(off), jj, kWave));
+#pragma unroll
+            for (int r = 0; r < kMaxOwn; ++r) {
+                const int d = lane + r * kWave;
+                if (d < hd) acc[r] = fmaf(pw, to_float(v_cache[vo + static_cast<long>(d) * page_size]), acc[r]);
             }
         }
-        __syncthreads();
     }
-    T* o = out + static_cast<size_t>(t) * nq * hd + h * hd;
-    const float inv_l = 1.0f / l_run;
+    // merge: wavefront 0 holds the first chunk, so the overall maximum is finite; a wavefront without keys has
+    // maximum -inf and weight exp(-inf) = 0
+    if (lane == 0) {
+        part_ml[wave][0] = m_run;
+        part_ml[wave][1] = l_run;
+    }
 #pragma unroll
     for (int r = 0; r < kMaxOwn; ++r) {
         const int d = lane + r * kWave;
-        if (d < hd) o[d] = from_float<T>(acc[r] * inv_l);
+        if (d < hd) part_o[wave][d] = acc[r];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float m_all = -INFINITY;
+    for (int w = 0; w < kGenericWaves; ++w) m_all = fmaxf(m_all, part_ml[w][0]);
+    float l_all = 0.f;
+    for (int w = 0; w < kGenericWaves; ++w) l_all = fmaf(part_ml[w][1], expf(part_ml[w][0] - m_all), l_all);
+    const float inv_l = 1.0f / l_all;
+    T* o = out + static_cast<size_t>(t) * nq * hd + h * hd;
+#pragma unroll
+    for (int r = 0; r < kMaxOwn; ++r) {
+        const int d = lane + r * kWave;
+        if (d < hd) {
+            float a = 0.f;
+            for (int w = 0; w < kGenericWaves; ++w) a = fmaf(part_o[w][d], expf(part_ml[w][0] - m_all), a);
+            o[d] = from_float<T>(a * inv_l);
+        }
     }
 }
 
@@ -112,12 +138,12 @@ extern "C" int egpt_paged_attention(const void* qkv, void* out, const void* k_ca
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid(n_tokens, nq);
     if (dtype == 0)
-        paged_attention_generic_kernel<float><<<grid, kWave, 0, s>>>(
+        paged_attention_generic_kernel<float><<<grid, kWave * kGenericWaves, 0, s>>>(
             static_cast<const float*>(qkv), static_cast<float*>(out), static_cast<const float*>(k_cache),
             static_cast<const float*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
             hd, page_size, scale, window);
     else if (dtype == 1)
-        paged_attention_generic_kernel<bf16_t><<<grid, kWave, 0, s>>>(
+        paged_attention_generic_kernel<bf16_t><<<grid, kWave * kGenericWaves, 0, s>>>(
             static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
             hd, page_size, scale, window);

@@ -71,6 +71,7 @@ class HipKernels:
             "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
                                             i, i, f, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_f32": [vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
@@ -216,9 +217,24 @@ class HipKernels:
             else:
                 torch.addmm(bias, x, w.t(), out=out)
             return out
+        if x.dtype == _F32 and k % 4 == 0:
+            # the float32 product on the matrix cores, the whole k range in one piece
+            self._run("egpt_gemm_f32", x.data_ptr(), w.data_ptr(), self._ptr(bias), out.data_ptr(), m, n, k, 1,
+                      self._stream())
+            return out
         self._run("egpt_linear", x.data_ptr(), w.data_ptr(), self._ptr(bias), out.data_ptr(), m, n, k, dt,
                   1 if out.dtype == _F32 else 0, self._stream())
         return out
+
+    @staticmethod
+    def _f32_splits(n: int, k: int) -> int:
+        """Into how many ranges the float32 product splits k: enough workgroups for a narrow result with few rows.
+        The count depends on the matrix alone, never on the rows, so that a row's partial sums, and with them
+        every value of the 32-bit path, are the same bits in whatever batch the row is computed."""
+        steps = -(-k // 64)
+        s = min(steps, max(1, 512 // -(-n // 64)), 8)
+        per = -(-steps // s)
+        return -(-steps // per)
 
     @staticmethod
     def _n_splits(m: int, n: int, k: int) -> int:
@@ -381,6 +397,13 @@ class HipKernels:
             self._need(w, "w", x.dtype, (n, k))
             out = torch.empty((1, m, n), dtype=_F32, device=x.device)
             torch.mm(x, w.t(), out_dtype=_F32, out=out[0])
+            return out
+        if x.dtype == _F32 and m > 0 and k % 4 == 0:
+            self._need(x, "x")
+            self._need(w, "w", _F32, (n, k))
+            s = self._f32_splits(n, k)
+            out = torch.empty((s, m, n), dtype=_F32, device=x.device)
+            self._run("egpt_gemm_f32", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), m, n, k, s, self._stream())
             return out
         out = torch.empty((m, n), dtype=x.dtype, device=x.device)
         return self.linear(x, w, None, out)

@@ -119,6 +119,43 @@ def test_skinny_product_and_partial_sums(k, m, n, kk):
     assert float((out16.double().cpu() - with_bias).abs().max()) <= 1e-2 * float(with_bias.abs().max())   # one bfloat16 rounding
 
 
+@pytest.mark.parametrize("m,n,kk", [(1, 75, 100), (16, 1152, 896), (37, 130, 96), (64, 200, 4864), (130, 1000, 200),
+                                    (300, 64, 68), (5, 777, 120)])
+def test_float32_product_on_the_matrix_cores(k, m, n, kk):
+    x, w, b = rnd(m, kk, seed=1), rnd(n, kk, seed=2, scale=0.1), rnd(n, seed=3)
+    ref = plain.linear(x.double().cpu(), w.double().cpu())
+    scale = float(ref.abs().max())
+
+    def tol(splits):
+        # a float32 sum of kk / splits terms one after the other: roundings of 6e-8 each that add up like a random walk
+        # (the FMA kernel that this one replaced is at the same 3e-6 for 4,864 terms)
+        return max(1e-6, 6e-8 * math.sqrt(kk / splits)) * scale
+
+    prod = k.product(x, w)
+    auto = k._f32_splits(n, kk)
+    assert prod.dtype == torch.float32 and prod.shape == (auto, m, n)
+    assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= tol(auto)
+    steps = -(-kk // 64)
+    for s in sorted({1, 2, 3, steps}):
+        if s > steps or (s - 1) * -(-steps // s) >= steps:
+            continue
+        out = torch.full((s, m, n), 7.0, device=DEV)
+        k._run("egpt_gemm_f32", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), m, n, kk, s, k._stream())
+        assert float((out.double().sum(0).cpu() - ref).abs().max()) <= tol(s), s
+    out = torch.empty(m, n, device=DEV)
+    k.linear(x, w, b, out)
+    assert float((out.double().cpu() - ref - b.double().cpu()).abs().max()) <= tol(1)
+    # a row's values are the same bits alone, among the others, and at another place among them
+    for r in sorted({0, m // 2, m - 1}):
+        alone = k.product(x[r : r + 1].contiguous(), w)
+        assert torch.equal(alone[:, 0], prod[:, r]), r
+    if m > 1:
+        turned = k.product(x.flip(0).contiguous(), w)
+        assert torch.equal(turned.flip(1), prod)
+    with pytest.raises(RuntimeError):
+        k._run("egpt_gemm_f32", x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), m, n, kk, 2, k._stream())   # bias with splits
+
+
 def test_which_products_go_to_the_library():
     from easy_gpt.cpp_amd.kernels.hip import HipKernels
 
