@@ -32,6 +32,20 @@ __device__ __forceinline__ int find_request(const int32_t* q_start, int n_seqs, 
 // steps and whatever else is in the batch.
 constexpr int kGenericWaves = 8;
 
+__device__ __forceinline__ void load4f(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load4f(const bf16_t* p, float* v) {
+    const uint2 a = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(a.x << 16); v[1] = __uint_as_float(a.x & 0xffff0000u);
+    v[2] = __uint_as_float(a.y << 16); v[3] = __uint_as_float(a.y & 0xffff0000u);
+}
+// the value that lane `from` (the same for all lanes) holds
+__device__ __forceinline__ float from_lane(float v, int from) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), from));
+}
+
 template <typename T>
 __global__ __launch_bounds__(64 * kGenericWaves) void paged_attention_generic_kernel(
     const T* __restrict__ qkv, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
@@ -39,7 +53,7 @@ __global__ __launch_bounds__(64 * kGenericWaves) void paged_attention_generic_ke
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len, int n_seqs, int nq, int nkv, int hd,
     int page_size, float scale, int window) {
     constexpr int kMaxOwn = kMaxHeadDim / kWave;
-    __shared__ float q_s[kMaxHeadDim];
+    __shared__ __attribute__((aligned(16))) float q_s[kMaxHeadDim];
     __shared__ float part_ml[kGenericWaves][2];
     __shared__ float part_o[kGenericWaves][kMaxHeadDim];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -54,19 +68,30 @@ __global__ __launch_bounds__(64 * kGenericWaves) void paged_attention_generic_ke
     for (int d = threadIdx.x; d < hd; d += kWave * kGenericWaves) q_s[d] = to_float(q[d]);
     __syncthreads();
     const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+    const bool vec4 = hd % 4 == 0 && page_size % 4 == 0;       // rows of keys and of values start at 16 (8) bytes
     float acc[kMaxOwn] = {};
     float m_run = -INFINITY, l_run = 0.f;
     for (int c = lo + wave * kWave; c < hi; c += kWave * kGenericWaves) {
         const int j = c + lane;
         float s = -INFINITY;
-        long off = 0;
         if (j < hi) {
             const long page = table[j / page_size];
             const long head_base = (page * nkv + kvh) * page_size * hd;   // same for keys and values
-            off = head_base + (j % page_size);                          // values: [feature][offset]
             const T* kr = k_cache + head_base + (j % page_size) * hd;     // keys: [offset][feature]
             float dot = 0.f;
-            for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float(kr[d]), dot);
+            if (vec4) {          // the same sum, its operands loaded four at a time
+                for (int d = 0; d < hd; d += 4) {
+                    float kv[4];
+                    load4f(kr + d, kv);
+                    const float4 qv = *reinterpret_cast<const float4*>(&q_s[d]);
+                    dot = fmaf(qv.x, kv[0], dot);
+                    dot = fmaf(qv.y, kv[1], dot);
+                    dot = fmaf(qv.z, kv[2], dot);
+                    dot = fmaf(qv.w, kv[3], dot);
+                }
+            } else {
+                for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float(kr[d]), dot);
+            }
             s = dot * scale;
         }
         const float m_new = fmaxf(m_run, wave_max(s));   // finite: key c is always visible
@@ -77,11 +102,30 @@ __global__ __launch_bounds__(64 * kGenericWaves) void paged_attention_generic_ke
         const int n_valid = min(kWave, hi - c);
 #pragma unroll
         for (int r = 0; r < kMaxOwn; ++r) acc[r] *= alpha;
-        // every lane needs every key's weight and place: handed round from the lane that holds them
-        for (int jj = 0; jj < n_valid; ++jj) {
-            const float pw = __shfl(pj, jj, kWave);
-            const long vo = (static_cast<long>(__shfl(static_cast<int>(off >> 32), jj, kWave)) << 32) |
-                            static_cast<unsigned int>(__shfl(static_cast<int>(off), jj, kWave));
+        // every lane needs every key's weight and place: taken from the lane that holds them.  Four keys that lie
+        // side by side in a page are one load per feature (the sum goes on key by key as without it).
+        int jj = 0;
+        if (vec4 && c % 4 == 0) {
+            for (; jj + 4 <= n_valid; jj += 4) {
+                const long page = table[(c + jj) / page_size];
+                const long vo = (page * nkv + kvh) * page_size * hd + (c + jj) % page_size;
+                const float pw[4] = {from_lane(pj, jj), from_lane(pj, jj + 1), from_lane(pj, jj + 2), from_lane(pj, jj + 3)};
+#pragma unroll
+                for (int r = 0; r < kMaxOwn; ++r) {
+                    const int d = lane + r * kWave;
+                    if (d < hd) {
+                        float vv[4];
+                        load4f(v_cache + vo + static_cast<long>(d) * page_size, vv);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[r] = fmaf(pw[e], vv[e], acc[r]);
+                    }
+                }
+            }
+        }
+        for (; jj < n_valid; ++jj) {
+            const float pw = from_lane(pj, jj);
+            const long page = table[(c + jj) / page_size];
+            const long vo = (page * nkv + kvh) * page_size * hd + (c + jj) % page_size;
 #pragma unroll
             for (int r = 0; r < kMaxOwn; ++r) {
                 const int d = lane + r * kWave;
