@@ -23,6 +23,9 @@ class StepContext:
     kv_len                 int32 [B]: tokens of the request in the cache once this step's are stored
     want_rows              int32 [R]: flat indices of the tokens whose logits are wanted, or None
     *_host                 the same numbers as Python lists, for parts that plan on the host
+    rows_independent       False when several of the B "requests" are tokens of one request (a portion laid out as
+                           single-token rows that share a block table): a row's keys and values must then be in the
+                           cache before any row's attention reads it
     """
 
     num_tokens: int
@@ -47,6 +50,7 @@ class StepContext:
     cache_location: dict = field(default_factory=dict)
     group_windows: list = field(default_factory=list)
     shared: dict = field(default_factory=dict)     # what parts of several layers compute once per step and share
+    rows_independent: bool = True
 
     def cache_view(self, cache_id: int, writes: bool) -> CacheView:
         g, j = self.cache_location[cache_id]

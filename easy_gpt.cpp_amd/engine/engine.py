@@ -92,6 +92,9 @@ class Engine:
         # steps that hold one token per request are replayed from captured device graphs
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe
         self._decode_plans: dict = {}
+        self._row_plans: dict = {}
+        self.graph_rows = 64        # steps of at most this many tokens in all run as rows of one token each,
+        self.graph_row_reads = 1 << 18      # if the tokens of their portions read at most this many keys in all
         self._graph_pool = None
         self._has_windows = any(g.window is not None for g in groups)
 
@@ -122,6 +125,14 @@ class Engine:
             return None
         if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
             return self._step_decode(entries)
+        if self.use_graphs and not self.model.state_needs and sum(len(e.tokens) for e in entries) <= self.graph_rows:
+            # (as rows of one token, every token of a portion reads its request's keys for itself: not behind a
+            # context so long that this outweighs what the graph saves)
+            requests = self.cache.requests
+            reads = sum(len(e.tokens) * (requests[e.request_id].num_tokens + len(e.tokens))
+                        for e in entries if len(e.tokens) > 1 and e.request_id in requests)
+            if reads <= self.graph_row_reads:
+                return self._step_rows(entries)
         rcs = self._check(entries)
         counts = [len(e.tokens) for e in entries]
         self.cache.reserve_step(rcs, counts)               # all of the step's pages or none
@@ -268,10 +279,56 @@ class Engine:
         return logits
 
 
+    # ------------------------------------------------------------------ few tokens in all, from a graph
+    def _step_rows(self, entries) -> torch.Tensor | None:
+        """A step of few tokens that is not one token per request (a short portion of a prompt, alone or beside
+        decoded tokens): every token becomes a row of its own, a "request" of one token whose context is its
+        position + 1 and whose block table is its request's.  That shape depends on the number of tokens alone,
+        so it is captured and replayed like a decode step, where the same step run kernel by kernel would spend
+        twice its device time on the host.  Keys and values of all rows are stored before attention reads them
+        (`rows_independent` is False).  Logits are computed for every row, the wanted ones are returned.  Not for
+        models with per-request state, whose parts walk a portion token after token."""
+        rcs = self._check(entries)
+        counts = [len(e.tokens) for e in entries]
+        self.cache.reserve_step(rcs, counts)
+        t = sum(counts)
+        widths = []
+        for g in range(len(self.cache.groups)):
+            need = max(rc.table_lens[g] for rc in rcs)
+            w = 4
+            while w < need:
+                w *= 2
+            widths.append(w)
+        kv_bound = -(-max(rc.num_tokens + n for rc, n in zip(rcs, counts)) // 512) * 512
+        key = (t, tuple(widths), kv_bound)
+        plan = self._row_plans.get(key)
+        if plan is None:
+            plan = self._row_plans[key] = _DecodePlan(self, t, widths, kv_bound, rows_independent=False)
+        plan.fill_rows(rcs, entries, counts)
+        if plan.graph is None:
+            logits = self.model.forward(plan.ctx)
+            plan.runs += 1
+            if plan.runs >= 2:
+                plan.capture(self)
+        else:
+            plan.graph.replay()
+            logits = plan.logits
+        self.cache.commit_step(rcs, counts)
+        want, base = [], 0
+        for e, n in zip(entries, counts):
+            want.extend(base + int(w) for w in e.want)
+            base += n
+        if not want:
+            return None
+        if want == list(range(t)):
+            return logits
+        return logits.index_select(0, torch.tensor(want, dtype=torch.int64, device=self.device))
+
+
 class _DecodePlan:
     """Static device buffers, a host mirror and the captured graph of one decode batch shape."""
 
-    def __init__(self, engine: Engine, batch: int, widths: list[int], kv_bound: int):
+    def __init__(self, engine: Engine, batch: int, widths: list[int], kv_bound: int, rows_independent: bool = True):
         self.batch, self.widths = batch, list(widths)
         dev = engine.device
         n_groups = len(widths)
@@ -295,7 +352,7 @@ class _DecodePlan:
             q_start_host=list(range(b)), q_len_host=[1] * b, kv_len_host=[0] * b,
             state_slots=v(5), state_slots_host=[0] * b, groups=groups, page_size=ps, kv_storage=engine.kv,
             state_storage=engine.states, cache_location=engine.model.cache_location,
-            group_windows=[n.window for n in engine.cache.groups],
+            group_windows=[n.window for n in engine.cache.groups], rows_independent=rows_independent,
         )
         self.row_state = np.full(2 * b, -1, dtype=np.int64)     # per row: (handle, table version) last written
         self.c_widths = _ints(self.widths)
@@ -319,6 +376,47 @@ class _DecodePlan:
         self.dev_small.copy_(self.host_small, non_blocking=True)
         if tables_changed:
             self.dev_tab.copy_(self.host_tab, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+
+    def fill_rows(self, rcs, entries, counts) -> None:
+        """The metadata of a step whose tokens are laid out as rows of one token each: the cache manager's library
+        writes the step as it is (positions and slots per token, a table per request), and the per-request parts
+        are repeated for every token of the request."""
+        if self.copied is not None:
+            self.copied.synchronize()
+        t, b = self.batch, len(rcs)
+        n_groups = len(self.widths)
+        small = self.np_small.reshape(7 + n_groups, t)
+        pos = 0
+        for e, n in zip(entries, counts):
+            small[0, pos : pos + n] = e.tokens
+            pos += n
+        per_request = np.empty((4, b), dtype=np.int32)               # q_start, q_len, kv_len, state slots
+        slots = np.empty(max(n_groups * t, 1), dtype=np.int32)
+        tables = np.empty(max(sum(b * w for w in self.widths), 1), dtype=np.int32)
+        self.cache.fill_step(
+            _ints([rc.handle for rc in rcs]), _ints(counts), self.c_widths,
+            (small[1].ctypes.data, per_request[0].ctypes.data, per_request[1].ctypes.data, per_request[2].ctypes.data,
+             per_request[3].ctypes.data, slots.ctypes.data if n_groups else None, tables.ctypes.data if n_groups else None),
+        )
+        rows = np.arange(t, dtype=np.int32)
+        reps = np.asarray(counts)
+        small[2], small[3], small[4] = rows, 1, small[1] + 1
+        small[5] = np.repeat(per_request[3], reps)
+        small[6] = rows
+        tab = self.host_tab.numpy()
+        off_in = off_out = 0
+        for g, w in enumerate(self.widths):
+            small[7 + g] = slots[g * t : (g + 1) * t]
+            tab[off_out : off_out + t * w] = np.repeat(tables[off_in : off_in + b * w].reshape(b, w), reps, axis=0).reshape(-1)
+            off_in += b * w
+            off_out += t * w
+        self.ctx.kv_len_host = (small[4]).tolist()
+        self.ctx.state_slots_host = small[5].tolist()
+        self.dev_small.copy_(self.host_small, non_blocking=True)
+        self.dev_tab.copy_(self.host_tab, non_blocking=True)
         if self.copied is None:
             self.copied = torch.cuda.Event()
         self.copied.record()

@@ -127,7 +127,7 @@ class GQAttention(Mixer):
         parts = False
         cos_sin = self.position.table(ctx) if (rot is not None and hasattr(self.position, "table")) else None
         if (prod.dim() == 3 and rot is not None and slots is not None and ctx.max_q_len == 1
-                and hasattr(k, "attention_decode_fused")):
+                and getattr(ctx, "rows_independent", True) and hasattr(k, "attention_decode_fused")):
             parts = k.attention_decode_fused(
                 prod, scale_args.get("row_ss"), scale_args.get("hidden", 0), scale_args.get("eps", 0.0), self.b_qkv,
                 ctx.positions, rot[0], rot[1], slots, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.kv_len,

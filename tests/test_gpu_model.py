@@ -133,6 +133,42 @@ def test_decoding_across_the_context_steps_of_the_captured_graphs(sharp_models, 
     assert len({key[2] for key in eng._decode_plans}) >= 2 and len({key[1] for key in eng._decode_plans}) >= 2
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_short_portions_run_as_rows_from_a_replayed_graph(sharp_models, name, dtype):
+    # a prompt fed five tokens a step beside another request's decoded tokens: six tokens in every step, laid out as six
+    # rows of one token, captured at the second step and replayed from then on; every step is compared with the plain model
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [90, 96], seed=47)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    a, b = reqs["r0"], reqs["r1"]
+    trace = [H.step_record(0, [("r0", a[:70], [69])])]                       # 70 tokens: the step of many tokens
+    for i in range(19):
+        entries = [("r1", b[5 * i : 5 * i + 5], [0, 4] if i % 2 else [4]), ("r0", [a[70 + i]], [0])]
+        trace.append(H.step_record(1 + i, entries[::-1] if i % 3 == 0 else entries))
+    trace.append(H.step_record(20, [("r1", b[95:], [0]), ("r0", [a[89]], [])], ["r0", "r1"]))
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16))
+    rows = H.replay(eng, trace)
+    H.assert_rows_match(rows, ref, tol_of(dtype), f"rows from a graph {name} {dtype}")
+    plans = eng._row_plans
+    assert any(key[0] == 6 and p.graph is not None for key, p in plans.items())
+    assert not eng._decode_plans                                              # no step was one token per request
+
+
+def test_portions_behind_a_long_context_are_not_laid_out_as_rows(tiny_models):
+    eng = engine_for(tiny_models["D"], "bfloat16", max_tokens=640)
+    eng.graph_row_reads = 2000
+    reqs = H.make_requests(TINY["D"][0]["vocab_size"], [600], seed=48)
+    from easy_gpt.cpp_amd.engine import StepEntry
+    eng.add_request("r")
+    eng.step([StepEntry("r", reqs["r0"][:500], [])])
+    eng.step([StepEntry("r", reqs["r0"][500:510], [9])])                      # 10 tokens x 510 keys > 2000
+    assert not eng._row_plans
+    eng.graph_row_reads = 1 << 18
+    eng.step([StepEntry("r", reqs["r0"][510:520], [9])])
+    assert len(eng._row_plans) == 1
+
+
 def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph(tmp_path):
     # 40 requests decoded side by side in a model whose gate/up and output matrices are wide enough for the library's
     # product at this many rows: the captured graph then holds library nodes, is replayed step after step with the
