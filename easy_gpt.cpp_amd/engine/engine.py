@@ -58,6 +58,8 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> Model:
 
 
 class Engine:
+    PAD_TO = 64          # steps that run from a padded graph are padded to a multiple of this many tokens
+
     def __init__(
         self,
         model: Model,
@@ -82,8 +84,12 @@ class Engine:
             num_pages = -(-int(max_tokens) // self.page_size)
         groups = [g.need for g in model.cache_groups]
         self.cache = CacheManager(groups, self.page_size, int(num_pages), max_requests)
+        # Beyond the pages that the manager hands out, a few that no request ever gets: where the padding tokens of
+        # a step that runs from a padded graph (`_step_padded`) put their keys and values.
+        self._pad_first_page = int(num_pages)
+        self._pad_pages = -(-(self.PAD_TO - 1) // self.page_size)
         self.kv = KVStorage(
-            groups, [len(g.cache_ids) for g in model.cache_groups], [num_pages] * len(groups),
+            groups, [len(g.cache_ids) for g in model.cache_groups], [num_pages + self._pad_pages] * len(groups),
             self.page_size, model.dtype, self.device,
         )
         self.states = StateStorage(model.state_needs, max_requests, self.device)
@@ -93,6 +99,8 @@ class Engine:
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and model.graph_safe
         self._decode_plans: dict = {}
         self._row_plans: dict = {}
+        self._padded_plans: dict = {}
+        self.graph_tokens = 2048    # steps of at most this many tokens run from a graph for their padded size
         self.graph_rows = 64        # steps of at most this many tokens in all run as rows of one token each,
         self.graph_row_reads = 1 << 18      # if the tokens of their portions read at most this many keys in all
         self._graph_pool = None
@@ -133,6 +141,8 @@ class Engine:
                         for e in entries if len(e.tokens) > 1 and e.request_id in requests)
             if reads <= self.graph_row_reads:
                 return self._step_rows(entries)
+        if self.use_graphs and not self.model.state_needs and sum(len(e.tokens) for e in entries) <= self.graph_tokens:
+            return self._step_padded(entries)
         rcs = self._check(entries)
         counts = [len(e.tokens) for e in entries]
         self.cache.reserve_step(rcs, counts)               # all of the step's pages or none
@@ -263,9 +273,7 @@ class Engine:
         # one choice: contexts are bucketed in steps of 512 tokens beside the table widths.
         kv_bound = -(-(max(rc.num_tokens for rc in rcs) + 1) // 512) * 512
         key = (b, tuple(widths), kv_bound)
-        plan = self._decode_plans.get(key)
-        if plan is None:
-            plan = self._decode_plans[key] = _DecodePlan(self, b, widths, kv_bound)
+        plan = self._plan(self._decode_plans, key, lambda: _DecodePlan(self, b, widths, kv_bound))
         plan.fill(rcs, tokens)
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
@@ -278,6 +286,16 @@ class Engine:
         self.cache.commit_step(rcs, plan.ones)
         return logits
 
+
+    MAX_PLANS = 128      # captured graphs kept per kind of step; the oldest goes when one more is needed
+
+    def _plan(self, plans: dict, key, make):
+        plan = plans.get(key)
+        if plan is None:
+            if len(plans) >= self.MAX_PLANS:
+                plans.pop(next(iter(plans)))
+            plan = plans[key] = make()
+        return plan
 
     # ------------------------------------------------------------------ few tokens in all, from a graph
     def _step_rows(self, entries) -> torch.Tensor | None:
@@ -301,9 +319,7 @@ class Engine:
             widths.append(w)
         kv_bound = -(-max(rc.num_tokens + n for rc, n in zip(rcs, counts)) // 512) * 512
         key = (t, tuple(widths), kv_bound)
-        plan = self._row_plans.get(key)
-        if plan is None:
-            plan = self._row_plans[key] = _DecodePlan(self, t, widths, kv_bound, rows_independent=False)
+        plan = self._plan(self._row_plans, key, lambda: _DecodePlan(self, t, widths, kv_bound, rows_independent=False))
         plan.fill_rows(rcs, entries, counts)
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)
@@ -323,6 +339,170 @@ class Engine:
         if want == list(range(t)):
             return logits
         return logits.index_select(0, torch.tensor(want, dtype=torch.int64, device=self.device))
+
+
+    # ------------------------------------------------------------------ any mix, from a graph for its padded size
+    def _step_padded(self, entries) -> torch.Tensor | None:
+        """Any step of up to `graph_tokens` tokens: the same model code as the general step, on static buffers of a
+        padded size, captured once per (tokens rounded up to a multiple of 64, requests rounded up to a power of two,
+        block-table widths) and replayed.  The padding is one more "request" whose tokens have pages of their own
+        that no real request ever gets; the requests after it have no tokens.  Every kernel takes the layout of the
+        step (where each request's tokens start, how many, how long its context is) from device memory, so one graph
+        serves every step of its size.  A step of a few hundred tokens run kernel by kernel takes 4 ms of host time
+        whatever its size; from the graph it takes its device time."""
+        rcs = self._check(entries)
+        counts = [len(e.tokens) for e in entries]
+        self.cache.reserve_step(rcs, counts)
+        t = sum(counts)
+        t_pad = -(-t // self.PAD_TO) * self.PAD_TO
+        b_pad = 2
+        while b_pad < len(rcs) + 1:
+            b_pad *= 2
+        widths = []
+        for g in range(len(self.cache.groups)):
+            need = max(max(rc.table_lens[g] for rc in rcs), self._pad_pages)
+            w = 4
+            while w < need:
+                w *= 2
+            widths.append(w)
+        r_pad = b_pad                           # logits rows: usually one per request or fewer
+        n_wanted = sum(len(e.want) for e in entries)
+        while r_pad < n_wanted:
+            r_pad *= 2
+        key = (t_pad, b_pad, r_pad, tuple(widths))
+        plan = self._plan(self._padded_plans, key, lambda: _PaddedPlan(self, t_pad, b_pad, r_pad, widths))
+        n_want = plan.fill(rcs, entries, counts)
+        if plan.graph is None:
+            logits = self.model.forward(plan.ctx)
+            plan.runs += 1
+            if plan.runs >= 2:
+                plan.capture(self)
+        else:
+            plan.graph.replay()
+            logits = plan.logits
+        self.cache.commit_step(rcs, counts)
+        return logits[:n_want] if n_want else None
+
+
+def _capture(graph, pool, run):
+    """Capture `run` into `graph`.  The collector of reference cycles stays off meanwhile: what it would free (a
+    dead engine's device memory, another graph) must not be freed while a stream is capturing."""
+    import gc
+
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph, pool=pool):
+            return run()
+    finally:
+        if was_enabled:
+            gc.enable()
+
+
+class _PaddedPlan:
+    """Static buffers, a pinned host mirror and the captured graph of one padded step size."""
+
+    def __init__(self, engine: Engine, t_pad: int, b_pad: int, r_pad: int, widths: list[int]):
+        self.t_pad, self.b_pad, self.widths = t_pad, b_pad, list(widths)
+        # (no reference back to the engine: engine and plan would keep each other alive until the collector of
+        # reference cycles runs, which may be in the middle of another engine's graph capture, where memory of
+        # the device must not be freed)
+        self.cache, self.page_size = engine.cache, engine.page_size
+        self.pad_first_page, self.pad_pages = engine._pad_first_page, engine._pad_pages
+        dev = engine.device
+        n_groups = len(widths)
+        ps = engine.page_size
+        # token ids, positions [t_pad each]; q_start, q_len, kv_len, state slots [b_pad each]; wanted rows [r_pad];
+        # slots [t_pad per group]; block tables [b_pad x width per group]
+        sizes = [t_pad, t_pad, b_pad, b_pad, b_pad, b_pad, r_pad] + [t_pad] * n_groups + [b_pad * w for w in widths]
+        self.offsets = [0]
+        for n in sizes:
+            self.offsets.append(self.offsets[-1] + n)
+        self.host = torch.zeros(self.offsets[-1], dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(self.offsets[-1], dtype=torch.int32, device=dev)
+        self.np = self.host.numpy()
+        view = lambda i: self.dev[self.offsets[i] : self.offsets[i + 1]]
+        groups = [GroupTables(view(7 + n_groups + g).view(b_pad, widths[g]), view(7 + g)) for g in range(n_groups)]
+        self.ctx = StepContext(
+            num_tokens=t_pad, num_seqs=b_pad, token_ids=view(0), positions=view(1), q_start=view(2), q_len=view(3),
+            kv_len=view(4), want_rows=view(6), max_q_len=t_pad, max_kv_len=min(w * ps for w in widths) if widths else 0,
+            q_start_host=[0] * b_pad, q_len_host=[0] * b_pad, kv_len_host=[0] * b_pad,
+            state_slots=view(5), state_slots_host=[0] * b_pad, groups=groups, page_size=ps, kv_storage=engine.kv,
+            state_storage=engine.states, cache_location=engine.model.cache_location,
+            group_windows=[n.window for n in engine.cache.groups],
+        )
+        self.c_widths = _ints(self.widths)
+        self.copied = None
+        self.graph = None
+        self.logits = None
+        self.runs = 0
+
+    def part(self, i: int) -> np.ndarray:
+        return self.np[self.offsets[i] : self.offsets[i + 1]]
+
+    def fill(self, rcs, entries, counts) -> int:
+        """Writes the step's metadata; returns how many logits rows are wanted (the first rows of the result)."""
+        if self.copied is not None:
+            self.copied.synchronize()                       # the pinned mirror is free again
+        t_pad, b_pad = self.t_pad, self.b_pad
+        b, t = len(rcs), sum(counts)
+        pad = t_pad - t
+        n_groups = len(self.widths)
+        ps = self.page_size
+        tokens, positions = self.part(0), self.part(1)
+        q_start, q_len, kv_len, state_slots, want_rows = (self.part(i) for i in range(2, 7))
+        pos = 0
+        want: list[int] = []
+        for e, n in zip(entries, counts):
+            tokens[pos : pos + n] = e.tokens
+            want.extend(pos + int(w) for w in e.want)
+            pos += n
+        slots = np.empty(max(n_groups * t, 1), dtype=np.int32)
+        tables = np.empty(max(sum(b * w for w in self.widths), 1), dtype=np.int32)
+        self.cache.fill_step(
+            _ints([rc.handle for rc in rcs]), _ints(counts), self.c_widths,
+            (positions.ctypes.data, q_start.ctypes.data, q_len.ctypes.data, kv_len.ctypes.data, state_slots.ctypes.data,
+             slots.ctypes.data if n_groups else None, tables.ctypes.data if n_groups else None),
+        )
+        # the padding: a request of `pad` tokens at positions 0.. on pages of its own, then requests without tokens
+        tokens[t:] = 0
+        positions[t:] = np.arange(pad, dtype=np.int32)
+        q_start[b:] = t_pad
+        q_len[b:] = 0
+        kv_len[b:] = 0
+        state_slots[b:] = 0
+        q_start[b], q_len[b], kv_len[b] = t, pad, pad
+        want_rows[: len(want)] = want
+        want_rows[len(want) :] = 0
+        pad_slots = (self.pad_first_page + np.arange(pad, dtype=np.int32) // ps) * ps + np.arange(pad, dtype=np.int32) % ps
+        off_in = 0
+        for g, w in enumerate(self.widths):
+            s_out = self.part(7 + g)
+            s_out[:t] = slots[g * t : (g + 1) * t]
+            s_out[t:] = pad_slots
+            tab = self.part(7 + n_groups + g).reshape(b_pad, w)
+            tab[:b] = tables[off_in : off_in + b * w].reshape(b, w)
+            tab[b:] = -1
+            tab[b, : self.pad_pages] = self.pad_first_page + np.arange(self.pad_pages, dtype=np.int32)
+            off_in += b * w
+        ctx = self.ctx
+        ctx.q_start_host = q_start.tolist()
+        ctx.q_len_host = q_len.tolist()
+        ctx.kv_len_host = kv_len.tolist()
+        ctx.state_slots_host = state_slots.tolist()
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+        return len(want)
+
+    def capture(self, engine: Engine) -> None:
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        if engine._graph_pool is None:
+            engine._graph_pool = torch.cuda.graph_pool_handle()
+        self.logits = _capture(graph, engine._graph_pool, lambda: engine.model.forward(self.ctx))
+        self.graph = graph
 
 
 class _DecodePlan:
@@ -426,6 +606,5 @@ class _DecodePlan:
         graph = torch.cuda.CUDAGraph()
         if engine._graph_pool is None:
             engine._graph_pool = torch.cuda.graph_pool_handle()
-        with torch.cuda.graph(graph, pool=engine._graph_pool):
-            self.logits = engine.model.forward(self.ctx)
+        self.logits = _capture(graph, engine._graph_pool, lambda: engine.model.forward(self.ctx))
         self.graph = graph

@@ -155,6 +155,72 @@ def test_short_portions_run_as_rows_from_a_replayed_graph(sharp_models, name, dt
     assert not eng._decode_plans                                              # no step was one token per request
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_steps_of_some_hundred_tokens_replay_the_graph_of_their_padded_size(sharp_models, name, dtype):
+    # steps of 65 to 128 tokens in changing mixes of three requests (portions, single tokens, a request left out, every
+    # row wanted or a few): all of them run from the graph for 128 tokens and four requests, captured at its second visit;
+    # one step of exactly 128 tokens has no padding at all
+    cfg = TINY[name][0]
+    cap = cfg["max_position_embeddings"]
+    reqs = H.make_requests(cfg["vocab_size"], [min(250, cap), 200, 230], seed=49)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    plan = [  # tokens of (r0, r1, r2) in each step
+        (70, 30, 0), (1, 5, 90), (1, 65, 1), (0, 1, 99), (87, 1, 0), (64, 63, 1), (1, 1, 20), (20, 30, 16), (1, 3, 1),
+    ]
+    fed = {rid: 0 for rid in reqs}
+    trace = []
+    for s_i, counts in enumerate(plan):
+        entries = []
+        for rid, n in zip(reqs, counts):
+            n = min(n, len(reqs[rid]) - fed[rid])
+            if n == 0:
+                continue
+            want = list(range(n)) if (s_i + len(entries)) % 2 == 0 else [n - 1]
+            entries.append((rid, reqs[rid][fed[rid] : fed[rid] + n], want))
+            fed[rid] += n
+        trace.append(H.step_record(s_i, entries))
+    rest = {rid: ids[fed[rid]:] for rid, ids in reqs.items() if fed[rid] < len(ids)}
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16) + 3 * 256)
+    rows = H.replay(eng, trace)
+    assert sum(plan[5]) == 128 and len(rows) > 300
+    for rid, ids in rest.items():                                   # what is left, whole
+        out = eng.step([H.StepEntry(rid, ids, list(range(len(ids))))]).float().cpu()
+        for j in range(len(ids)):
+            rows[(rid, fed[rid] + j)] = out[j]
+        eng.finish(rid)
+    H.assert_rows_match(rows, ref, tol_of(dtype), f"padded graphs {name} {dtype}")
+    replayed = [key for key, p in eng._padded_plans.items() if p.graph is not None]
+    assert any(key[0] == 128 and key[1] == 4 for key in replayed), list(eng._padded_plans)
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+def test_an_engine_is_freed_when_its_last_reference_goes(tiny_models):
+    # its plans hold no reference back to it: if they did, its device memory and graphs would be freed whenever the
+    # collector of reference cycles runs, which may be in the middle of another engine's graph capture
+    import gc
+    import weakref
+
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    reqs = H.make_requests(TINY["A"][0]["vocab_size"], [100, 30, 9], seed=50)
+    gc.collect()
+    gc.disable()
+    try:
+        eng = engine_for(tiny_models["A"], "bfloat16", max_tokens=512)
+        for rid, ids in reqs.items():
+            eng.add_request(rid)
+            eng.step([StepEntry(rid, ids[:-3], [])])                      # a padded step and two steps as rows
+        for i in (3, 2, 1):
+            eng.step([StepEntry(rid, [ids[-i]], [0]) for rid, ids in reqs.items()])     # decode steps, captured
+        assert eng._padded_plans and eng._row_plans and eng._decode_plans
+        ref = weakref.ref(eng)
+        del eng
+        assert ref() is None
+    finally:
+        gc.enable()
+
+
 def test_portions_behind_a_long_context_are_not_laid_out_as_rows(tiny_models):
     eng = engine_for(tiny_models["D"], "bfloat16", max_tokens=640)
     eng.graph_row_reads = 2000
