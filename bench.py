@@ -63,8 +63,9 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
     g = torch.Generator().manual_seed(0)
     results = []
     for rep in range(2):                                       # the first pass warms up (graphs, library choices)
-        sched = Scheduler(engine, SchedulerConfig(max_active=SERVE_REQUESTS, max_admit_per_step=8, max_tokens_per_step=2048,
-                                                  prefill_chunk=SERVE_CHUNK), eos_token_id=-1)
+        sched = Scheduler(engine, SchedulerConfig(max_active=SERVE_REQUESTS, max_admit_per_step=8,
+                                                  max_tokens_per_step=args.serve_budget,
+                                                  prefill_chunk=min(SERVE_CHUNK, args.serve_budget)), eos_token_id=-1)
         for i, n in enumerate(lens):
             sched.add(Request(f"s{rep}_{i}", torch.randint(0, vocab, (n,), generator=g).tolist(), SamplingParams(greedy=True),
                               max_new_tokens=SERVE_NEW_TOKENS, ignore_eos=True))
@@ -84,7 +85,8 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
         "generated_per_s": round(SERVE_REQUESTS * SERVE_NEW_TOKENS / sec, 1), "seconds": round(sec, 3),
         "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
         "config": {"model": f"{name} layer sizes", "requests": SERVE_REQUESTS, "prompt_tokens": sum(lens),
-                   "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": SERVE_CHUNK, "max_tokens_per_step": 2048,
+                   "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": min(SERVE_CHUNK, args.serve_budget),
+                   "max_tokens_per_step": args.serve_budget,
                    "preemptions": st.preemptions, "sampling": "greedy"},
     }), flush=True)
     return 0
@@ -105,6 +107,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
     ap.add_argument("--serve", action="store_true",
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
                          "each through the scheduler, prompts in portions of 512 (a workload of the baseline record)")
