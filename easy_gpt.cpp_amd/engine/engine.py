@@ -344,7 +344,7 @@ class Engine:
     # ------------------------------------------------------------------ any mix, from a graph for its padded size
     def _step_padded(self, entries) -> torch.Tensor | None:
         """Any step of up to `graph_tokens` tokens: the same model code as the general step, on static buffers of a
-        padded size, captured once per (tokens rounded up to a multiple of 64, requests rounded up to a power of two,
+        padded size, captured once per (tokens rounded up to a multiple of 64, of 16 up to 256; requests rounded up to a power of two,
         block-table widths) and replayed.  The padding is one more "request" whose tokens have pages of their own
         that no real request ever gets; the requests after it have no tokens.  Every kernel takes the layout of the
         step (where each request's tokens start, how many, how long its context is) from device memory, so one graph
@@ -354,7 +354,8 @@ class Engine:
         counts = [len(e.tokens) for e in entries]
         self.cache.reserve_step(rcs, counts)
         t = sum(counts)
-        t_pad = -(-t // self.PAD_TO) * self.PAD_TO
+        step = 16 if t <= 256 else self.PAD_TO          # small steps are padded less: their time grows with their rows
+        t_pad = -(-t // step) * step
         b_pad = 2
         while b_pad < len(rcs) + 1:
             b_pad *= 2

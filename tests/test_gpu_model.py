@@ -158,15 +158,15 @@ def test_short_portions_run_as_rows_from_a_replayed_graph(sharp_models, name, dt
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["B", "D"])
 def test_steps_of_some_hundred_tokens_replay_the_graph_of_their_padded_size(sharp_models, name, dtype):
-    # steps of 65 to 128 tokens in changing mixes of three requests (portions, single tokens, a request left out, every
-    # row wanted or a few): all of them run from the graph for 128 tokens and four requests, captured at its second visit;
-    # one step of exactly 128 tokens has no padding at all
+    # steps of 97 to 112 tokens in changing mixes of three requests (portions, single tokens, a request left out): all of
+    # them run from the graph for 112 tokens and four requests, captured at its second visit and replayed after; one of
+    # them has exactly 112 tokens and so no padding at all; one step wants every row and has a graph of its own
     cfg = TINY[name][0]
     cap = cfg["max_position_embeddings"]
-    reqs = H.make_requests(cfg["vocab_size"], [min(250, cap), 200, 230], seed=49)
+    reqs = H.make_requests(cfg["vocab_size"], [min(250, cap), 230, 240], seed=49)
     ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
     plan = [  # tokens of (r0, r1, r2) in each step
-        (70, 30, 0), (1, 5, 90), (1, 65, 1), (0, 1, 99), (87, 1, 0), (64, 63, 1), (1, 1, 20), (20, 30, 16), (1, 3, 1),
+        (70, 30, 0), (1, 5, 95), (1, 100, 1), (0, 1, 99), (97, 1, 0), (1, 1, 110), (60, 50, 1), (20, 30, 16), (1, 3, 1),
     ]
     fed = {rid: 0 for rid in reqs}
     trace = []
@@ -176,22 +176,23 @@ def test_steps_of_some_hundred_tokens_replay_the_graph_of_their_padded_size(shar
             n = min(n, len(reqs[rid]) - fed[rid])
             if n == 0:
                 continue
-            want = list(range(n)) if (s_i + len(entries)) % 2 == 0 else [n - 1]
+            want = list(range(n)) if s_i == 3 else ([n - 1] if (s_i + len(entries)) % 2 else [0, n - 1])
             entries.append((rid, reqs[rid][fed[rid] : fed[rid] + n], want))
             fed[rid] += n
         trace.append(H.step_record(s_i, entries))
     rest = {rid: ids[fed[rid]:] for rid, ids in reqs.items() if fed[rid] < len(ids)}
     eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16) + 3 * 256)
     rows = H.replay(eng, trace)
-    assert sum(plan[5]) == 128 and len(rows) > 300
+    assert sum(plan[5]) == 112 and len(rows) > 110
     for rid, ids in rest.items():                                   # what is left, whole
         out = eng.step([H.StepEntry(rid, ids, list(range(len(ids))))]).float().cpu()
         for j in range(len(ids)):
             rows[(rid, fed[rid] + j)] = out[j]
+    for rid in reqs:
         eng.finish(rid)
     H.assert_rows_match(rows, ref, tol_of(dtype), f"padded graphs {name} {dtype}")
-    replayed = [key for key, p in eng._padded_plans.items() if p.graph is not None]
-    assert any(key[0] == 128 and key[1] == 4 for key in replayed), list(eng._padded_plans)
+    visits = {key: (p.runs, p.graph is not None) for key, p in eng._padded_plans.items()}
+    assert any(key[0] == 112 and key[1] == 4 and captured for key, (runs, captured) in visits.items()), visits
     assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
 
 
