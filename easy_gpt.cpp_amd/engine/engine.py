@@ -101,6 +101,7 @@ class Engine:
         self._row_plans: dict = {}
         self._padded_plans: dict = {}
         self.graph_tokens = 2048    # steps of at most this many tokens run from a graph for their padded size
+        self.capture_after = 2      # a shape's graph is captured at this visit (None: never, the same kernels one by one)
         self.graph_rows = 64        # steps of at most this many tokens in all run as rows of one token each,
         self.graph_row_reads = 1 << 18      # if the tokens of their portions read at most this many keys in all
         self._graph_pool = None
@@ -278,7 +279,7 @@ class Engine:
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
             plan.runs += 1
-            if plan.runs >= 2:                              # captured from the second visit on
+            if self.capture_after is not None and plan.runs >= self.capture_after:                              # captured from the second visit on
                 plan.capture(self)
         else:
             plan.graph.replay()
@@ -324,7 +325,7 @@ class Engine:
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)
             plan.runs += 1
-            if plan.runs >= 2:
+            if self.capture_after is not None and plan.runs >= self.capture_after:
                 plan.capture(self)
         else:
             plan.graph.replay()
@@ -376,7 +377,7 @@ class Engine:
         if plan.graph is None:
             logits = self.model.forward(plan.ctx)
             plan.runs += 1
-            if plan.runs >= 2:
+            if self.capture_after is not None and plan.runs >= self.capture_after:
                 plan.capture(self)
         else:
             plan.graph.replay()

@@ -196,6 +196,40 @@ def test_steps_of_some_hundred_tokens_replay_the_graph_of_their_padded_size(shar
     assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
 
 
+def test_graph_replays_of_large_steps_equal_the_steps_run_kernel_by_kernel(tmp_path):
+    # layer sizes of the 0.5B model (the library's products at their real shapes), two layers: steps of 2,048 and of 300
+    # tokens replayed from their graphs several times, with other work between the replays, against the same steps of an
+    # engine that runs the same padded steps kernel by kernel: the same kernels, so the same bits
+    from easy_gpt.cpp_amd.engine import StepEntry
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    cfg = {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 896,
+        "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 9001,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 4096,
+    }
+    write_random_model(str(tmp_path), cfg, seed=13, dtype=torch.bfloat16)
+    graphs = engine_for(str(tmp_path), "bfloat16", max_tokens=4096 + 1024)
+    plain_steps = engine_for(str(tmp_path), "bfloat16", max_tokens=4096 + 1024)
+    plain_steps.capture_after = None                     # the same steps on the same padded shapes, never captured
+    g = torch.Generator().manual_seed(5)
+    for rep in range(5):
+        big = torch.randint(0, 9001, (2048,), generator=g).tolist()
+        small = torch.randint(0, 9001, (300,), generator=g).tolist()
+        outs = []
+        for eng in (graphs, plain_steps):
+            eng.add_request("big"), eng.add_request("small")
+            a = eng.step([StepEntry("big", big, [0, 1000, 2047])]).clone()
+            b = eng.step([StepEntry("small", small[:290], [289]), StepEntry("big", [7], [0])]).clone()
+            c = eng.step([StepEntry("small", small[290:], [9])]).clone()              # rows of one token
+            eng.finish("big"), eng.finish("small")
+            outs.append((a, b, c))
+        for x, y in zip(*outs):
+            assert torch.equal(x, y), rep
+    assert all(p.graph is not None for p in graphs._padded_plans.values()) and len(graphs._padded_plans) == 2
+    assert all(p.graph is None for p in plain_steps._padded_plans.values()) and len(plain_steps._padded_plans) == 2
+
+
 def test_an_engine_is_freed_when_its_last_reference_goes(tiny_models):
     # its plans hold no reference back to it: if they did, its device memory and graphs would be freed whenever the
     # collector of reference cycles runs, which may be in the middle of another engine's graph capture
