@@ -230,6 +230,32 @@ def test_graph_replays_of_large_steps_equal_the_steps_run_kernel_by_kernel(tmp_p
     assert all(p.graph is None for p in plain_steps._padded_plans.values()) and len(plain_steps._padded_plans) == 2
 
 
+def test_plans_are_dropped_and_made_again_when_there_are_too_many(sharp_by_dtype):
+    # at most two graphs of a kind are kept here: steps of five sizes in turn drop and re-capture them all the time
+    name, dtype = "D", "bfloat16"
+    cfg = TINY[name][0]
+    model_dir = sharp_by_dtype[dtype][name]
+    reqs = H.make_requests(cfg["vocab_size"], [400, 360], seed=52)
+    ref = H.plain_rows(model_dir, reqs, bf16_weights=True)
+    eng = engine_for(model_dir, dtype, max_tokens=1280)
+    eng.MAX_PLANS = 2
+    sizes = [70, 20, 100, 3, 130]
+    fed = {"r0": 0, "r1": 0}
+    trace, s_i = [], 0
+    while any(fed[r] < len(reqs[r]) for r in reqs):
+        entries = []
+        for j, rid in enumerate(reqs):
+            n = min(sizes[(s_i + 2 * j) % len(sizes)], len(reqs[rid]) - fed[rid])
+            if n:
+                entries.append((rid, reqs[rid][fed[rid] : fed[rid] + n], [0, n - 1]))
+                fed[rid] += n
+        trace.append(H.step_record(s_i, entries))
+        s_i += 1
+    rows = H.replay(eng, trace)
+    H.assert_rows_match(rows, ref, H.BF16_TOL, "plans dropped and made again")
+    assert len(eng._padded_plans) <= 2 and len(eng._row_plans) <= 2 and s_i >= 6
+
+
 def test_an_engine_is_freed_when_its_last_reference_goes(tiny_models):
     # its plans hold no reference back to it: if they did, its device memory and graphs would be freed whenever the
     # collector of reference cycles runs, which may be in the middle of another engine's graph capture
