@@ -263,32 +263,47 @@ class Engine:
         if starters:
             self.cache.reserve_step(starters, [1] * len(starters))
         b = len(rcs)
-        widths = []
-        for g in range(len(self.cache.groups)):
-            need = max(rc.table_lens[g] for rc in rcs)
-            w = 4
-            while w < need:
-                w *= 2
-            widths.append(w)
+        widths = self._table_widths(rcs)
         # The kernels choose their shape (key splits of the attention) by the longest context, and a graph holds
         # one choice: contexts are bucketed in steps of 512 tokens beside the table widths.
         kv_bound = -(-(max(rc.num_tokens for rc in rcs) + 1) // 512) * 512
         key = (b, tuple(widths), kv_bound)
         plan = self._plan(self._decode_plans, key, lambda: _DecodePlan(self, b, widths, kv_bound))
         plan.fill(rcs, tokens)
-        if plan.graph is None:
-            logits = self.model.forward(plan.ctx)           # eager once: the result, and the warm-up
-            plan.runs += 1
-            if self.capture_after is not None and plan.runs >= self.capture_after:                              # captured from the second visit on
-                plan.capture(self)
-        else:
-            plan.graph.replay()
-            logits = plan.logits
+        logits = self._run(plan)
         self.cache.commit_step(rcs, plan.ones)
         return logits
 
-
+    # ------------------------------------------------------------------ what the steps from graphs share
     MAX_PLANS = 128      # captured graphs kept per kind of step; the oldest goes when one more is needed
+
+    def _table_widths(self, rcs, at_least: int = 0) -> list[int]:
+        """Block-table widths of a plan: for each group the next power of two (from 4) that holds the longest table."""
+        widths = []
+        for g in range(len(self.cache.groups)):
+            need = max(max(rc.table_lens[g] for rc in rcs), at_least)
+            w = 4
+            while w < need:
+                w *= 2
+            widths.append(w)
+        return widths
+
+    def _run(self, plan) -> torch.Tensor:
+        """The model on the plan's buffers: kernel by kernel on its first visits (the result, and the warm-up), the
+        graph captured at visit `capture_after` and replayed from then on."""
+        if plan.graph is not None:
+            plan.graph.replay()
+            return plan.logits
+        logits = self.model.forward(plan.ctx)
+        plan.runs += 1
+        if self.capture_after is not None and plan.runs >= self.capture_after:
+            graph = torch.cuda.CUDAGraph()
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            torch.cuda.synchronize()
+            plan.logits = _capture(graph, self._graph_pool, lambda: self.model.forward(plan.ctx))
+            plan.graph = graph
+        return logits
 
     def _plan(self, plans: dict, key, make):
         plan = plans.get(key)
@@ -311,25 +326,12 @@ class Engine:
         counts = [len(e.tokens) for e in entries]
         self.cache.reserve_step(rcs, counts)
         t = sum(counts)
-        widths = []
-        for g in range(len(self.cache.groups)):
-            need = max(rc.table_lens[g] for rc in rcs)
-            w = 4
-            while w < need:
-                w *= 2
-            widths.append(w)
+        widths = self._table_widths(rcs)
         kv_bound = -(-max(rc.num_tokens + n for rc, n in zip(rcs, counts)) // 512) * 512
         key = (t, tuple(widths), kv_bound)
         plan = self._plan(self._row_plans, key, lambda: _DecodePlan(self, t, widths, kv_bound, rows_independent=False))
         plan.fill_rows(rcs, entries, counts)
-        if plan.graph is None:
-            logits = self.model.forward(plan.ctx)
-            plan.runs += 1
-            if self.capture_after is not None and plan.runs >= self.capture_after:
-                plan.capture(self)
-        else:
-            plan.graph.replay()
-            logits = plan.logits
+        logits = self._run(plan)
         self.cache.commit_step(rcs, counts)
         want, base = [], 0
         for e, n in zip(entries, counts):
@@ -360,13 +362,7 @@ class Engine:
         b_pad = 2
         while b_pad < len(rcs) + 1:
             b_pad *= 2
-        widths = []
-        for g in range(len(self.cache.groups)):
-            need = max(max(rc.table_lens[g] for rc in rcs), self._pad_pages)
-            w = 4
-            while w < need:
-                w *= 2
-            widths.append(w)
+        widths = self._table_widths(rcs, at_least=self._pad_pages)
         r_pad = b_pad                           # logits rows: usually one per request or fewer
         n_wanted = sum(len(e.want) for e in entries)
         while r_pad < n_wanted:
@@ -374,14 +370,7 @@ class Engine:
         key = (t_pad, b_pad, r_pad, tuple(widths))
         plan = self._plan(self._padded_plans, key, lambda: _PaddedPlan(self, t_pad, b_pad, r_pad, widths))
         n_want = plan.fill(rcs, entries, counts)
-        if plan.graph is None:
-            logits = self.model.forward(plan.ctx)
-            plan.runs += 1
-            if self.capture_after is not None and plan.runs >= self.capture_after:
-                plan.capture(self)
-        else:
-            plan.graph.replay()
-            logits = plan.logits
+        logits = self._run(plan)
         self.cache.commit_step(rcs, counts)
         return logits[:n_want] if n_want else None
 
@@ -498,13 +487,6 @@ class _PaddedPlan:
         self.copied.record()
         return len(want)
 
-    def capture(self, engine: Engine) -> None:
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        if engine._graph_pool is None:
-            engine._graph_pool = torch.cuda.graph_pool_handle()
-        self.logits = _capture(graph, engine._graph_pool, lambda: engine.model.forward(self.ctx))
-        self.graph = graph
 
 
 class _DecodePlan:
@@ -603,10 +585,3 @@ class _DecodePlan:
             self.copied = torch.cuda.Event()
         self.copied.record()
 
-    def capture(self, engine: Engine) -> None:
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        if engine._graph_pool is None:
-            engine._graph_pool = torch.cuda.graph_pool_handle()
-        self.logits = _capture(graph, engine._graph_pool, lambda: engine.model.forward(self.ctx))
-        self.graph = graph
