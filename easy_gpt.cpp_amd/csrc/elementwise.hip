@@ -101,6 +101,9 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
     float* hrow = h + src * hidden;
     const DT* drow = delta ? delta + src * hidden : nullptr;
     const bool write_back = (rows == nullptr) && (delta != nullptr);
+    // a row that the workgroup covers in one pass stays in registers for the second pass (one round trip less)
+    const bool one_pass = hidden <= static_cast<int>(blockDim.x) * 8;
+    float kept[8] = {};
     float ss = 0.f;
     for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
         float v[8];
@@ -116,19 +119,27 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
             }
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+        for (int i = 0; i < 8; ++i) {
+            ss += v[i] * v[i];
+            kept[i] = v[i];
+        }
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
     bf16_t* orow = out + static_cast<size_t>(r) * hidden;
     for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
         float v[8], w[8];
-        load8_as_float(hrow + j, v);
-        if (drow && !write_back) {
-            float d[8];
-            load8_as_float(drow + j, d);
+        if (one_pass) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] += d[i];
+            for (int i = 0; i < 8; ++i) v[i] = kept[i];
+        } else {
+            load8_as_float(hrow + j, v);
+            if (drow && !write_back) {
+                float d[8];
+                load8_as_float(drow + j, d);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] += d[i];
+            }
         }
         load8_as_float(weight + j, w);
         uint4 o;
