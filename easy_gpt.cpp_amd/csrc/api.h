@@ -92,6 +92,11 @@ int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, in
 // weights: scratch for n_rows * vocab floats.
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                 const float* uniform, int32_t* out, float* weights, int n_rows, int vocab, void* stream);
+// The same in stages for wide vocabularies (several workgroups per row, then the selection on the tokens that can still
+// be kept); workspace: egpt_sample_workspace(n_rows, vocab) bytes of device memory.
+size_t egpt_sample_workspace(int n_rows, int vocab);
+int egpt_sample_wide(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
+                     const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab, void* stream);
 
 #ifdef __cplusplus
 }

@@ -14,7 +14,7 @@ namespace egpt {
 constexpr int kSampleThreads = 1024;
 
 // Calls f(index, value) for every element of p[0..n) once, spread over the workgroup's threads (thread `tid` of
-// `n_threads`).  The body reads 16 bytes per thread and keeps four such loads in flight: a pass over a row is a
+// `n_threads`).  The body reads 16 bytes per thread and keeps eight such loads in flight: a pass over a row is a
 // chain of dependent loads otherwise, and its time is their latency, not the row's size.
 template <typename F>
 __device__ __forceinline__ void for_each_in_row(const float* __restrict__ p, int n, int tid, int n_threads, F f) {
@@ -22,8 +22,24 @@ __device__ __forceinline__ void for_each_in_row(const float* __restrict__ p, int
     for (int j = tid; j < head; j += n_threads) f(j, p[j]);
     const float4* p4 = reinterpret_cast<const float4*>(p + head);
     const int n4 = (n - head) / 4;
-#pragma unroll 4
-    for (int i = tid; i < n4; i += n_threads) {
+    // eight loads issued before the first value is used (the compiler does not do this by itself across calls of f
+    // that hold ballots or atomic additions)
+    constexpr int kAhead = 8;
+    int i = tid;
+    for (; i + (kAhead - 1) * n_threads < n4; i += kAhead * n_threads) {
+        float4 v[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) v[u] = p4[i + u * n_threads];
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int j = head + 4 * (i + u * n_threads);
+            f(j, v[u].x);
+            f(j + 1, v[u].y);
+            f(j + 2, v[u].z);
+            f(j + 3, v[u].w);
+        }
+    }
+    for (; i < n4; i += n_threads) {
         const float4 v = p4[i];
         const int j = head + 4 * i;
         f(j, v.x);
@@ -283,12 +299,206 @@ __device__ uint32_t select_by_mass(const float* __restrict__ w, int vocab, uint3
     return lo;
 }
 
+// ---- wide vocabularies: the row-wide work spread over many workgroups, the selection on what is left of the row
+//
+// The selection below walks its row a dozen times with one workgroup, which for 150,000 tokens is 300 us whatever the
+// number of rows.  For a wide vocabulary three small kernels with kSamplePieces workgroups per row come first: they
+// count the weights by exponent (those within 2^-16 of the largest, which hold the top-k tokens and the top-p mass of
+// any distribution that is not nearly flat), decide below which exponent no token can be kept, and write the tokens at
+// or above it, in index order, into a list of candidates.  The selection then runs on that list, unchanged.
+constexpr int kSamplePieces = 32;
+constexpr int kTopBins = 16;            // exponents 127 (weight 1.0) down to 112, one bin each; bin kTopBins: the rest
+
+__device__ __forceinline__ int top_bin_of(uint32_t bits) {           // bits of a weight in [0, 1]
+    const int e = static_cast<int>(bits >> 23);
+    return e >= 128 - kTopBins ? 127 - e : kTopBins;
+}
+
+// piece_count / piece_mass [rows][kSamplePieces][kTopBins + 1]: per piece of the row, how many weights each bin holds
+// and their mass in fixed point
+__global__ __launch_bounds__(256) void sample_hist_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                          const int32_t* __restrict__ best, unsigned int* __restrict__ piece_count,
+                                                          unsigned long long* __restrict__ piece_mass, int vocab) {
+    __shared__ unsigned int s_count[kTopBins + 1];
+    __shared__ unsigned long long s_mass[kTopBins + 1];
+    const int r = blockIdx.x, c = blockIdx.y;
+    const float temp = temperature[r];
+    if (!(temp > 0.f)) return;
+    const float* row = logits + static_cast<size_t>(r) * vocab;
+    const float mx = row[best[r]];
+    const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+    const int piece = (vocab + kSamplePieces - 1) / kSamplePieces;
+    const int begin = min(vocab, c * piece), n = min(vocab, begin + piece) - begin;
+    unsigned int cnt[kTopBins + 1];
+    unsigned long long mass[kTopBins + 1];
+#pragma unroll
+    for (int i = 0; i <= kTopBins; ++i) {
+        cnt[i] = 0u;
+        mass[i] = 0ull;
+    }
+    for_each_in_row(row + begin, n, threadIdx.x, blockDim.x, [&](int, float x) {
+        const float w = weight_of(x, mx, inv_t);
+        const int bin = top_bin_of(__float_as_uint(w));
+        const unsigned long long f = fixed_of(w);
+#pragma unroll
+        for (int i = 0; i <= kTopBins; ++i) {
+            cnt[i] += bin == i ? 1u : 0u;
+            mass[i] += bin == i ? f : 0ull;
+        }
+    });
+    for (int i = threadIdx.x; i <= kTopBins; i += blockDim.x) {
+        s_count[i] = 0u;
+        s_mass[i] = 0ull;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x % kWave;
+#pragma unroll
+    for (int i = 0; i <= kTopBins; ++i) {
+        unsigned int cv = cnt[i];
+        unsigned long long mv = mass[i];
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) {
+            cv += __shfl_xor(cv, o, kWave);
+            mv += __shfl_xor(mv, o, kWave);
+        }
+        if (lane == 0 && cv) {                       // integer sums: the order does not matter
+            atomicAdd(&s_count[i], cv);
+            atomicAdd(&s_mass[i], mv);
+        }
+    }
+    __syncthreads();
+    const size_t base = (static_cast<size_t>(r) * kSamplePieces + c) * (kTopBins + 1);
+    for (int i = threadIdx.x; i <= kTopBins; i += blockDim.x) {
+        piece_count[base + i] = s_count[i];
+        piece_mass[base + i] = s_mass[i];
+    }
+}
+
+// cutoff[r]: bit pattern below which no weight of row r can be kept; offsets[r][0..kSamplePieces]: where each piece's
+// candidates start in the row's list (the last entry is their number)
+__global__ __launch_bounds__(64) void sample_plan_kernel(const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
+                                                         const float* __restrict__ top_p,
+                                                         const unsigned int* __restrict__ piece_count,
+                                                         const unsigned long long* __restrict__ piece_mass,
+                                                         uint32_t* __restrict__ cutoff, int32_t* __restrict__ offsets,
+                                                         unsigned long long* __restrict__ row_mass, int vocab) {
+    __shared__ unsigned int s_count[kTopBins + 1];
+    __shared__ unsigned long long s_mass[kTopBins + 1];
+    __shared__ int s_bin;
+    const int r = blockIdx.x, t = threadIdx.x;
+    if (!(temperature[r] > 0.f)) return;
+    const size_t base = static_cast<size_t>(r) * kSamplePieces * (kTopBins + 1);
+    if (t <= kTopBins) {
+        unsigned int cv = 0u;
+        unsigned long long mv = 0ull;
+        for (int c = 0; c < kSamplePieces; ++c) {
+            cv += piece_count[base + c * (kTopBins + 1) + t];
+            mv += piece_mass[base + c * (kTopBins + 1) + t];
+        }
+        s_count[t] = cv;
+        s_mass[t] = mv;
+    }
+    __syncthreads();
+    if (t == 0) {
+        // the last bin whose tokens can be kept (kTopBins: every token can)
+        const int k = top_k[r];
+        const float p = top_p[r];
+        int last = kTopBins;
+        if (k > 0 && k < vocab) {                    // the k-th largest weight lies in this bin; top-p only removes more
+            unsigned int cum = 0u;
+            for (int i = 0; i <= kTopBins; ++i) {
+                cum += s_count[i];
+                if (cum >= static_cast<unsigned int>(k)) {
+                    last = i;
+                    break;
+                }
+            }
+        } else if (p > 0.f && p < 1.f) {             // the mass p of the whole row is reached within this bin
+            unsigned long long total = 0ull;
+            for (int i = 0; i <= kTopBins; ++i) total += s_mass[i];
+            unsigned long long need = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(total));
+            if (need == 0ull) need = 1ull;
+            unsigned long long cum = 0ull;
+            for (int i = 0; i <= kTopBins; ++i) {
+                cum += s_mass[i];
+                if (cum >= need) {
+                    last = i;
+                    break;
+                }
+            }
+        }
+        s_bin = last;
+        cutoff[r] = last >= kTopBins ? 0u : static_cast<uint32_t>(127 - last) << 23;
+        unsigned long long all = 0ull;
+        for (int i = 0; i <= kTopBins; ++i) all += s_mass[i];
+        row_mass[r] = all;                           // the mass of the whole row: what top-p without top-k refers to
+    }
+    __syncthreads();
+    if (t == 0) {
+        const int last = s_bin;
+        int at = 0;
+        for (int c = 0; c < kSamplePieces; ++c) {
+            offsets[r * (kSamplePieces + 1) + c] = at;
+            for (int i = 0; i <= last; ++i) at += static_cast<int>(piece_count[base + c * (kTopBins + 1) + i]);
+        }
+        offsets[r * (kSamplePieces + 1) + kSamplePieces] = at;
+    }
+}
+
+// the candidates of a piece, in index order: cand_w / cand_idx [rows][vocab]
+__global__ __launch_bounds__(256) void sample_compact_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                             const int32_t* __restrict__ best, const uint32_t* __restrict__ cutoff,
+                                                             const int32_t* __restrict__ offsets, float* __restrict__ cand_w,
+                                                             int32_t* __restrict__ cand_idx, int vocab) {
+    __shared__ int s_wave[4];
+    const int r = blockIdx.x, c = blockIdx.y;
+    const float temp = temperature[r];
+    if (!(temp > 0.f)) return;
+    const float* row = logits + static_cast<size_t>(r) * vocab;
+    const float mx = row[best[r]];
+    const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+    const uint32_t cut = cutoff[r];
+    const int piece = (vocab + kSamplePieces - 1) / kSamplePieces;
+    const int begin = min(vocab, c * piece), end = min(vocab, begin + piece);
+    float* ow = cand_w + static_cast<size_t>(r) * vocab;
+    int32_t* oi = cand_idx + static_cast<size_t>(r) * vocab;
+    int at = offsets[r * (kSamplePieces + 1) + c];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    // 256 tokens at a time, token j by thread j: the order of the list is the order of the tokens
+    for (int j0 = begin; j0 < end; j0 += 256) {
+        const int j = j0 + threadIdx.x;
+        float w = 0.f;
+        bool keep = false;
+        if (j < end) {
+            w = weight_of(row[j], mx, inv_t);
+            keep = __float_as_uint(w) >= cut;
+        }
+        const unsigned long long mask = __ballot(keep);
+        const int before = __popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) s_wave[wave] = __popcll(mask);
+        __syncthreads();
+        int wave_base = 0, total = 0;
+        for (int i = 0; i < 4; ++i) {
+            wave_base += i < wave ? s_wave[i] : 0;
+            total += s_wave[i];
+        }
+        if (keep) {
+            ow[at + wave_base + before] = w;
+            oi[at + wave_base + before] = j;
+        }
+        at += total;
+        __syncthreads();
+    }
+}
+
 // One workgroup per row.  `weights` is scratch [rows][vocab] float32: the weights are computed once and the
-// selection passes read them back (from cache).
+// selection passes read them back (from cache).  With a list of candidates (cand_idx != null) `weights` holds the
+// candidates' weights, cand_count[r * cand_stride] their number, and `best` the row's argmax.
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
     const float* __restrict__ top_p, const float* __restrict__ uniform, int32_t* __restrict__ out,
-    float* __restrict__ weights, int vocab) {
+    float* __restrict__ weights, int vocab, const int32_t* __restrict__ cand_idx, const int32_t* __restrict__ cand_count,
+    int cand_stride, const int32_t* __restrict__ best_in, const unsigned long long* __restrict__ row_mass) {
     __shared__ float s_val[16];
     __shared__ int s_idx[16];
     __shared__ unsigned int hist[256];
@@ -303,20 +513,28 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
     const float* row = logits + static_cast<size_t>(r) * vocab;
     float* w = weights + static_cast<size_t>(r) * vocab;
+    const int32_t* idx_of = cand_idx ? cand_idx + static_cast<size_t>(r) * vocab : nullptr;
     const float temp = temperature[r];
-    const int best = block_argmax(row, vocab, s_val, s_idx);
+    const int best = cand_idx ? best_in[r] : block_argmax(row, vocab, s_val, s_idx);
     if (!(temp > 0.f)) {  // greedy, as the reference for temperature <= 0 (sampler.cpp:46-49)
         if (threadIdx.x == 0) out[r] = best;
         return;
     }
-    const float mx = row[best];
-    const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
-    for_each_in_row(row, vocab, threadIdx.x, blockDim.x, [&](int j, float x) { w[j] = weight_of(x, mx, inv_t); });
-    __syncthreads();   // each thread reads back what others wrote: same workgroup, so a barrier suffices
+    const int full_vocab = vocab;
+    if (cand_idx) {
+        vocab = cand_count[r * cand_stride];         // from here on the row is the list of candidates
+    } else {
+        const float mx = row[best];
+        const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
+        for_each_in_row(row, vocab, threadIdx.x, blockDim.x, [&](int j, float x) { w[j] = weight_of(x, mx, inv_t); });
+        __syncthreads();   // each thread reads back what others wrote: same workgroup, so a barrier suffices
+    }
     // kept set = { j : w_j >= threshold }; the threshold starts at 0 (everything)
     uint32_t threshold = 0u;
     const int k = top_k[r];
-    if (k > 0 && k < vocab) threshold = select_by_count(w, vocab, static_cast<unsigned int>(k), hist, &s_a, &s_need);
+    const bool k_active = k > 0 && k < full_vocab;
+    if (k_active && k < vocab)        // (a list of exactly k candidates is the top k)
+        threshold = select_by_count(w, vocab, static_cast<unsigned int>(k), hist, &s_a, &s_need);
     const float p = top_p[r];
     if (p > 0.f && p < 1.f) {
         // mass of what top-k kept, in fixed point: per-thread sums, then over the wavefronts in order
@@ -331,6 +549,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
         unsigned long long kept = 0ull;
         for (int i = 0; i < n_waves; ++i) kept += s_wave[i];
         __syncthreads();
+        // (a list of candidates without top-k holds only the upper part of the row: the mass p refers to the whole row)
+        if (cand_idx && !k_active) kept = row_mass[r];
         unsigned long long need = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(kept));
         if (need == 0ull) need = 1ull;
         threshold = select_by_mass(w, vocab, threshold, need, s_wave, &s_a, &s_b, &s_above);
@@ -390,7 +610,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
             if (hit) pick = base + __ffsll(static_cast<long long>(hit)) - 1;
             cum += __shfl(incl, kWave - 1, kWave);
         }
-        if (lane == 0) out[r] = pick >= 0 ? pick : (last_kept >= 0 ? last_kept : best);
+        if (lane == 0) {
+            const int at = pick >= 0 ? pick : last_kept;
+            out[r] = at < 0 ? best : (idx_of ? idx_of[at] : at);
+        }
     }
 }
 
@@ -422,8 +645,59 @@ extern "C" int egpt_sample(const float* logits, const float* temperature, const 
     if (!logits || !temperature || !top_k || !top_p || !uniform || !out || !weights || n_rows < 0 || vocab <= 0)
         return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
-    sample_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, top_k,
-                                                                                   top_p, uniform, out, weights, vocab);
+    sample_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(
+        logits, temperature, top_k, top_p, uniform, out, weights, vocab, nullptr, nullptr, 0, nullptr, nullptr);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
+// The same for wide vocabularies, in stages (argmax, counts by exponent, the plan, the list of candidates, the
+// selection on the list).  workspace: egpt_sample_workspace(n_rows, vocab) bytes of device memory.
+static size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+extern "C" size_t egpt_sample_workspace(int n_rows, int vocab) {
+    const size_t r = static_cast<size_t>(n_rows > 0 ? n_rows : 0), v = static_cast<size_t>(vocab > 0 ? vocab : 0);
+    return align256(r * v * 4) * 2                                         // candidates: weights, indices
+           + align256(r * kSamplePieces * (kTopBins + 1) * 8)            // masses
+           + align256(r * kSamplePieces * (kTopBins + 1) * 4)            // counts
+           + align256(r * (kSamplePieces + 1) * 4) + align256(r * 4) * 2   // offsets, cutoff, best
+           + align256(r * 8)                                               // mass of the row
+           + align256(r * kArgmaxPieces * 8);                              // argmax pieces
+}
+
+extern "C" int egpt_sample_wide(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
+                                const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab, void* stream) {
+    if (!logits || !temperature || !top_k || !top_p || !uniform || !out || !workspace || n_rows < 0 || vocab <= 0)
+        return EGPT_BAD_ARGUMENT;
+    if (n_rows == 0) return EGPT_OK;
+    if (n_rows > 65535) return EGPT_UNSUPPORTED_SIZE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t r = static_cast<size_t>(n_rows), v = static_cast<size_t>(vocab);
+    char* p = static_cast<char*>(workspace);
+    float* cand_w = reinterpret_cast<float*>(p);                               p += align256(r * v * 4);
+    int32_t* cand_idx = reinterpret_cast<int32_t*>(p);                         p += align256(r * v * 4);
+    unsigned long long* piece_mass = reinterpret_cast<unsigned long long*>(p); p += align256(r * kSamplePieces * (kTopBins + 1) * 8);
+    unsigned int* piece_count = reinterpret_cast<unsigned int*>(p);            p += align256(r * kSamplePieces * (kTopBins + 1) * 4);
+    int32_t* offsets = reinterpret_cast<int32_t*>(p);                          p += align256(r * (kSamplePieces + 1) * 4);
+    uint32_t* cutoff = reinterpret_cast<uint32_t*>(p);                         p += align256(r * 4);
+    int32_t* best = reinterpret_cast<int32_t*>(p);                             p += align256(r * 4);
+    unsigned long long* row_mass = reinterpret_cast<unsigned long long*>(p);   p += align256(r * 8);
+    float* pv = reinterpret_cast<float*>(p);
+    int32_t* pi = reinterpret_cast<int32_t*>(pv + r * kArgmaxPieces);
+    argmax_pieces_kernel<<<dim3(n_rows, kArgmaxPieces), 256, 0, s>>>(logits, pv, pi, vocab);
+    EGPT_CHECK_LAUNCH();
+    argmax_pick_kernel<<<n_rows, kWave, 0, s>>>(pv, pi, best);
+    EGPT_CHECK_LAUNCH();
+    sample_hist_kernel<<<dim3(n_rows, kSamplePieces), 256, 0, s>>>(logits, temperature, best, piece_count, piece_mass, vocab);
+    EGPT_CHECK_LAUNCH();
+    sample_plan_kernel<<<n_rows, 64, 0, s>>>(temperature, top_k, top_p, piece_count, piece_mass, cutoff, offsets, row_mass,
+                                             vocab);
+    EGPT_CHECK_LAUNCH();
+    sample_compact_kernel<<<dim3(n_rows, kSamplePieces), 256, 0, s>>>(logits, temperature, best, cutoff, offsets, cand_w,
+                                                                      cand_idx, vocab);
+    EGPT_CHECK_LAUNCH();
+    sample_kernel<<<n_rows, kSampleThreads, 0, s>>>(logits, temperature, top_k, top_p, uniform, out, cand_w, vocab, cand_idx,
+                                                    offsets + kSamplePieces, kSamplePieces + 1, best, row_mass);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -77,7 +77,10 @@ class HipKernels:
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
+            "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
         }
+        lib.egpt_sample_workspace.restype = ctypes.c_size_t
+        lib.egpt_sample_workspace.argtypes = [i, i]
         for name, argtypes in sigs.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
@@ -612,6 +615,12 @@ class HipKernels:
         self._need(top_p, "top_p", _F32, (r,))
         self._need(uniform, "uniform", _F32, (r,))
         self._need(out, "out", _I32, (r,))
+        if v >= 8192:
+            # a wide vocabulary: the row-wide passes by many workgroups, the selection on the tokens that are left
+            space = torch.empty(int(self.lib.egpt_sample_workspace(r, v)), dtype=torch.uint8, device=logits.device)
+            self._run("egpt_sample_wide", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
+                      uniform.data_ptr(), out.data_ptr(), space.data_ptr(), r, v, self._stream())
+            return
         weights = torch.empty((r, v), dtype=_F32, device=logits.device)
         self._run("egpt_sample", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(),
                   uniform.data_ptr(), out.data_ptr(), weights.data_ptr(), r, v, self._stream())

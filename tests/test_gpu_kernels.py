@@ -689,15 +689,34 @@ def test_argmax_lowest_index_wins(k):
     assert out2.tolist() == wide.argmax(-1).tolist()
 
 
-@pytest.mark.parametrize("vocab", [777, 5000])
-def test_sample_follows_the_reference_s_distribution(k, vocab):
+@pytest.mark.parametrize("vocab,scale", [(777, 2.5), (5000, 2.5), (9001, 2.5), (151936, 2.5), (40003, 0.02), (151936, 9.0),
+                                         (8192, 0.0)])
+def test_sample_follows_the_reference_s_distribution(k, vocab, scale):
+    # narrow vocabularies go through one kernel, wide ones (from 8,192 tokens) through the staged one; logits nearly
+    # flat (every token in one exponent of the weights: nothing can be cut before the selection), all equal, and peaked
     rows = 64
-    logits = rnd(rows, vocab, seed=6, scale=2.5)
-    cases = [(0.8, 20, 0.95), (1.0, 0, 1.0), (0.5, 5, 0.5), (2.0, 0, 0.9), (1.3, 50, 1.0), (0.0, 0, 1.0)]
+    logits = rnd(rows, vocab, seed=6, scale=scale)
+    cases = [(0.8, 20, 0.95), (1.0, 0, 1.0), (0.5, 5, 0.5), (2.0, 0, 0.9), (1.3, 50, 1.0), (0.0, 0, 1.0), (0.7, 0, 0.3),
+             (1.0, 3000, 0.99)]
     g = torch.Generator().manual_seed(9)
     temp = torch.tensor([cases[i % len(cases)][0] for i in range(rows)])
     topk = torch.tensor([cases[i % len(cases)][1] for i in range(rows)], dtype=torch.int32)
     topp = torch.tensor([cases[i % len(cases)][2] for i in range(rows)])
+    if scale == 0.0:
+        # all tokens tie: a cut by count or by mass has no boundary to fall on (the kernel keeps ties whole, the
+        # reference's sort keeps the lowest indices); what is compared is the draw from the whole row
+        topk.zero_()
+        topp.fill_(1.0)
+    # The kernel selects on float32 weights and keeps the tokens that tie with the k-th whole.  Where the k-th and the
+    # next weight of a row are closer than float32 tells apart (it happens among thousands of nearly equal ones), the
+    # float64 reference still separates them: such a row takes the next k whose boundary float32 resolves.
+    for r in range(rows):
+        kk = int(topk[r])
+        if temp[r] > 0 and 0 < kk < vocab:
+            srt = torch.sort(logits[r].cpu().double(), descending=True).values / float(temp[r])
+            while kk < vocab and float(srt[kk - 1] - srt[kk]) < 1e-6:
+                kk += 1
+            topk[r] = kk
     u = torch.rand(rows, generator=g)
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
     k.sample(logits, temp.to(DEV), topk.to(DEV), topp.to(DEV), u.to(DEV), out)
