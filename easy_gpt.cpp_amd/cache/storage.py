@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from ..parts.base import CacheNeed, StateNeed
+from ..parts.base import StateNeed
 
 
 class KVStorage:

@@ -11,7 +11,7 @@ from __future__ import annotations
 import os
 import sys
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 USAGE = """Usage: easy_llm [--model <dir>] [--prompt-file <path>] [--max-steps <n>]
                 [--temperature <float>] [--top-p <float>] [--top-k <int>] [--seed <int>] [--greedy]

@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import _ints
-from ..cache import CacheManager, KVStorage, OutOfPages, RequestCache, StateStorage
+from ..cache import CacheManager, KVStorage, RequestCache, StateStorage
 from ..config.registry import load_model_config
 from ..parts.model import Model, build_model
 from ..weights.loader import CheckedWeights

@@ -7,7 +7,6 @@ rounded to the output tensor's dtype.
 """
 from __future__ import annotations
 
-import math
 
 import torch
 

@@ -6,7 +6,6 @@ import json
 import os
 import random
 
-import numpy as np
 import torch
 
 import plain_qwen2 as plain

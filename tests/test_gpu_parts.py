@@ -1,5 +1,4 @@
 """Each part of a layer alone on the GPU against the plain implementation's function for it."""
-import math
 from types import SimpleNamespace
 
 import pytest

@@ -6,8 +6,6 @@ toy architecture, loaded from a random-weights folder and stepped, without a cha
   * a feed-forward with routing (router logits in float32, every token to its best expert, per-expert token lists);
   * a run order that names a layer twice and lets a layer read another layer's cache.
 The toy parts compute with torch on the GPU; they are test equipment, not a model of anyone's."""
-import json
-import math
 import os
 from dataclasses import dataclass
 

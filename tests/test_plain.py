@@ -2,7 +2,6 @@
 reduce to a library routine, and invariants, each chosen so that a plausible mistake fails it."""
 import math
 
-import pytest
 import torch
 import torch.nn.functional as F
 
