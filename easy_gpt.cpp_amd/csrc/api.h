@@ -87,6 +87,9 @@ int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss
                             void* stream);
 int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd, const void* w,
                           float* out, int m, int n, int n_splits, int waves, void* stream);
+// Gate/up product with SwiGLU for up to 64 rows (see gemm_gate_up.hip): out bfloat16 [m][inter] from x bfloat16 [m][k]
+// and w bfloat16 [2 * inter][k] (gate rows, then up rows); k % 8 == 0.
+int egpt_gemm_gate_up_swiglu(const void* x, const void* w, void* out, int m, int inter, int k, int groups, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
 // weights: scratch for n_rows * vocab floats.

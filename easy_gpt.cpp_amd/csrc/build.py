@@ -17,7 +17,7 @@ import tempfile
 import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "attention.hip", "attention_mfma.hip", "sampling.hip"]
+SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_gate_up.hip", "attention.hip", "attention_mfma.hip", "sampling.hip"]
 HEADERS = ["api.h", "common.h"]
 LIB_NAME = "libeasygpt_hip.so"
 ARCH = "gfx950"

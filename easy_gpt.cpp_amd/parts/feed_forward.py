@@ -62,6 +62,10 @@ class SwiGLU(FeedForward):
                 return k.product(act, self.w_down)
             x = x.materialize()
         t = x.shape[0]
+        if hasattr(k, "gate_up_swiglu"):
+            act = k.gate_up_swiglu(x, self.w_gate_up)    # a few dozen tokens: product and activation in one kernel
+            if act is not None:
+                return k.product(act, self.w_down)
         gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]
         if gate_up.dim() == 3 and hasattr(k, "product_swiglu"):
             out = k.product_swiglu(gate_up, None, self.hidden_size, 0.0, self.w_down)

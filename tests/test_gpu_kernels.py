@@ -280,6 +280,28 @@ def test_product_with_swiglu_folded_in(k, t, inter, n, g_splits):
             assert float((prod.double().sum(0).cpu() - ref).abs().max()) <= 1.2e-2 * float(ref.abs().max()), (waves, max_splits)
 
 
+@pytest.mark.parametrize("t,inter,hid", [(64, 4864, 896), (17, 176, 64), (33, 250, 96), (48, 1000, 1544), (20, 23, 8),
+                                          (64, 8960, 1536), (31, 40, 2056)])
+def test_gate_up_product_with_swiglu(k, t, inter, hid):
+    # one kernel for [gate | up] = x w^T and up * silu(gate); widths that are no multiple of a tile, of a chunk of 32 or
+    # of the wavefronts' share of k; a k range of several rounds; one and two column groups per workgroup
+    x = rnd(t, hid, dtype=torch.bfloat16, seed=1)
+    w = rnd(2 * inter, hid, dtype=torch.bfloat16, seed=2, scale=1.5 / math.sqrt(hid))
+    gu = plain.linear(x.double().cpu(), w.double().cpu())
+    g, u = gu[:, :inter], gu[:, inter:]
+    ref = u * (g / (1.0 + torch.exp(-g)))
+    for groups in (1, 2, None):
+        act = k.gate_up_swiglu(x, w, groups=groups)
+        if act is None:                  # a large matrix: the wrapper leaves it to the product and the SwiGLU kernel
+            assert groups is None and 2 * inter * hid >= 16 << 20
+            continue
+        assert act.dtype == torch.bfloat16 and tuple(act.shape) == (t, inter)
+        assert float((act.double().cpu() - ref).abs().max()) <= 6e-3 * float(ref.abs().max()), groups
+    # rows outside the kernel's range are refused by the wrapper, not computed wrongly
+    assert k.gate_up_swiglu(x[:16].contiguous(), w) is None
+    assert k.gate_up_swiglu(torch.cat([x, x, x, x, x])[:65].contiguous(), w) is None
+
+
 @pytest.mark.parametrize("nq,nkv,hd,batch,ctx", [(14, 2, 64, 8, 700), (12, 2, 128, 3, 300), (14, 2, 64, 1, 2113), (3, 1, 64, 16, 90)])
 def test_output_projection_combines_attention_parts(k, nq, nkv, hd, batch, ctx):
     # split attention left uncombined, then combined by the output projection: equals combine + plain product
