@@ -329,42 +329,35 @@ __global__ __launch_bounds__(256) void sample_hist_kernel(const float* __restric
     const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
     const int piece = (vocab + kSamplePieces - 1) / kSamplePieces;
     const int begin = min(vocab, c * piece), n = min(vocab, begin + piece) - begin;
-    unsigned int cnt[kTopBins + 1];
-    unsigned long long mass[kTopBins + 1];
-#pragma unroll
-    for (int i = 0; i <= kTopBins; ++i) {
-        cnt[i] = 0u;
-        mass[i] = 0ull;
-    }
-    for_each_in_row(row + begin, n, threadIdx.x, blockDim.x, [&](int, float x) {
-        const float w = weight_of(x, mx, inv_t);
-        const int bin = top_bin_of(__float_as_uint(w));
-        const unsigned long long f = fixed_of(w);
-#pragma unroll
-        for (int i = 0; i <= kTopBins; ++i) {
-            cnt[i] += bin == i ? 1u : 0u;
-            mass[i] += bin == i ? f : 0ull;
-        }
-    });
     for (int i = threadIdx.x; i <= kTopBins; i += blockDim.x) {
         s_count[i] = 0u;
         s_mass[i] = 0ull;
     }
     __syncthreads();
-    const int lane = threadIdx.x % kWave;
-#pragma unroll
-    for (int i = 0; i <= kTopBins; ++i) {
-        unsigned int cv = cnt[i];
-        unsigned long long mv = mass[i];
-#pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) {
-            cv += __shfl_xor(cv, o, kWave);
-            mv += __shfl_xor(mv, o, kWave);
+    // Nearly every weight lies below the top bins and is summed in registers; the few above go to the bins in LDS
+    // (integer additions: the order does not matter).
+    unsigned int rest_count = 0u;
+    unsigned long long rest_mass = 0ull;
+    for_each_in_row(row + begin, n, threadIdx.x, blockDim.x, [&](int, float x) {
+        const float w = weight_of(x, mx, inv_t);
+        const int bin = top_bin_of(__float_as_uint(w));
+        const unsigned long long f = fixed_of(w);
+        if (bin == kTopBins) {
+            rest_count += 1u;
+            rest_mass += f;
+        } else {
+            atomicAdd(&s_count[bin], 1u);
+            atomicAdd(&s_mass[bin], f);
         }
-        if (lane == 0 && cv) {                       // integer sums: the order does not matter
-            atomicAdd(&s_count[i], cv);
-            atomicAdd(&s_mass[i], mv);
-        }
+    });
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+        rest_count += __shfl_xor(rest_count, o, kWave);
+        rest_mass += __shfl_xor(rest_mass, o, kWave);
+    }
+    if (threadIdx.x % kWave == 0 && rest_count) {
+        atomicAdd(&s_count[kTopBins], rest_count);
+        atomicAdd(&s_mass[kTopBins], rest_mass);
     }
     __syncthreads();
     const size_t base = (static_cast<size_t>(r) * kSamplePieces + c) * (kTopBins + 1);
@@ -434,15 +427,24 @@ __global__ __launch_bounds__(64) void sample_plan_kernel(const float* __restrict
         row_mass[r] = all;                           // the mass of the whole row: what top-p without top-k refers to
     }
     __syncthreads();
-    if (t == 0) {
-        const int last = s_bin;
-        int at = 0;
-        for (int c = 0; c < kSamplePieces; ++c) {
-            offsets[r * (kSamplePieces + 1) + c] = at;
-            for (int i = 0; i <= last; ++i) at += static_cast<int>(piece_count[base + c * (kTopBins + 1) + i]);
-        }
-        offsets[r * (kSamplePieces + 1) + kSamplePieces] = at;
+    // where each piece's candidates start: thread c counts piece c, a prefix sum over the wavefront does the rest
+    const int last = s_bin;
+    int mine = 0;
+    if (t < kSamplePieces) {
+        unsigned int v[kTopBins + 1];
+#pragma unroll
+        for (int i = 0; i <= kTopBins; ++i) v[i] = piece_count[base + t * (kTopBins + 1) + i];
+#pragma unroll
+        for (int i = 0; i <= kTopBins; ++i) mine += i <= last ? static_cast<int>(v[i]) : 0;
     }
+    int incl = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const int up = __shfl_up(incl, o, kWave);
+        if (t >= o) incl += up;
+    }
+    if (t < kSamplePieces) offsets[r * (kSamplePieces + 1) + t] = incl - mine;
+    if (t == kSamplePieces - 1) offsets[r * (kSamplePieces + 1) + kSamplePieces] = incl;
 }
 
 // the candidates of a piece, in index order: cand_w / cand_idx [rows][vocab]
@@ -491,6 +493,65 @@ __global__ __launch_bounds__(256) void sample_compact_kernel(const float* __rest
     }
 }
 
+// The selection and the draw for a list of at most kSampleThreads weights, one thread each (a list of candidates is
+// usually a few dozen tokens, and the passes of the general selection cost their barriers, not their data).
+// Token j is among the k most likely iff fewer than k weights are greater than its own, and within the mass `need`
+// iff the mass of the greater weights is below it: the same sets as the thresholds of select_by_count and
+// select_by_mass (ties whole).  Counts and fixed-point masses are integers, so nothing depends on an order; the
+// draw walks the kept weights in index order.  Returns the picked position in the list or -1 (every thread).
+__device__ int pick_from_short_list(const float* __restrict__ w, int n, bool cut_by_count, unsigned int k, float p,
+                                    bool mass_of_row, unsigned long long row_mass, float u, float* s_list /* [kSampleThreads] */,
+                                    unsigned long long* s_wave /* [16] */, float* s_piece /* [16] */, int* s_pick /* [2] */) {
+    const int j = threadIdx.x, lane = j % kWave, wave = j / kWave, n_waves = blockDim.x / kWave;
+    const float wj = j < n ? w[j] : 0.f;
+    s_list[j] = wj;                                   // slots past n hold 0: never greater than a weight
+    if (j < 2) s_pick[j] = j == 0 ? 0x7fffffff : -1;
+    __syncthreads();
+    unsigned int above = 0u;
+    unsigned long long mass_above = 0ull;
+    const int n4 = (n + 3) / 4;
+    for (int i = 0; i < n4; ++i) {                    // every thread reads the same address: a broadcast
+        const float4 v = reinterpret_cast<const float4*>(s_list)[i];
+        above += (v.x > wj) + (v.y > wj) + (v.z > wj) + (v.w > wj);
+        mass_above += (v.x > wj ? fixed_of(v.x) : 0ull) + (v.y > wj ? fixed_of(v.y) : 0ull) +
+                      (v.z > wj ? fixed_of(v.z) : 0ull) + (v.w > wj ? fixed_of(v.w) : 0ull);
+    }
+    bool keep = j < n && (!cut_by_count || above < k);
+    if (p > 0.f && p < 1.f) {
+        unsigned long long mine = keep ? fixed_of(wj) : 0ull;
+#pragma unroll
+        for (int o = kWave / 2; o > 0; o >>= 1) mine += __shfl_xor(mine, o, kWave);
+        if (lane == 0) s_wave[wave] = mine;
+        __syncthreads();
+        unsigned long long kept = 0ull;
+        for (int i = 0; i < n_waves; ++i) kept += s_wave[i];
+        if (mass_of_row) kept = row_mass;
+        unsigned long long need = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(kept));
+        if (need == 0ull) need = 1ull;
+        keep = keep && mass_above < need;
+    }
+    // inverse CDF in index order: prefix sums inside the wavefronts, then over them
+    const float mine = keep ? wj : 0.f;
+    float incl = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const float up = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += up;
+    }
+    if (lane == kWave - 1) s_piece[wave] = incl;
+    __syncthreads();
+    float before = 0.f, total = 0.f;
+    for (int i = 0; i < n_waves; ++i) {
+        before += i < wave ? s_piece[i] : 0.f;
+        total += s_piece[i];
+    }
+    const float target = fminf(fmaxf(u, 0.f), 0.99999994f) * total;
+    if (keep && before + incl > target) atomicMin(&s_pick[0], j);
+    if (keep) atomicMax(&s_pick[1], j);               // the last kept token catches rounding at the end
+    __syncthreads();
+    return s_pick[0] != 0x7fffffff ? s_pick[0] : s_pick[1];
+}
+
 // One workgroup per row.  `weights` is scratch [rows][vocab] float32: the weights are computed once and the
 // selection passes read them back (from cache).  With a list of candidates (cand_idx != null) `weights` holds the
 // candidates' weights, cand_count[r * cand_stride] their number, and `best` the row's argmax.
@@ -509,6 +570,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     __shared__ float s_piece[16];
     __shared__ int s_owner;
     __shared__ float s_before;
+    __shared__ __attribute__((aligned(16))) float s_list[kSampleThreads];
+    __shared__ int s_pick[2];
     const int r = blockIdx.x;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, n_waves = blockDim.x / kWave;
     const float* row = logits + static_cast<size_t>(r) * vocab;
@@ -529,10 +592,17 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
         for_each_in_row(row, vocab, threadIdx.x, blockDim.x, [&](int j, float x) { w[j] = weight_of(x, mx, inv_t); });
         __syncthreads();   // each thread reads back what others wrote: same workgroup, so a barrier suffices
     }
-    // kept set = { j : w_j >= threshold }; the threshold starts at 0 (everything)
-    uint32_t threshold = 0u;
     const int k = top_k[r];
     const bool k_active = k > 0 && k < full_vocab;
+    if (vocab <= kSampleThreads) {                   // a short row or list: one thread per token
+        const int at = pick_from_short_list(w, vocab, k_active && k < vocab, static_cast<unsigned int>(k), top_p[r],
+                                            cand_idx && !k_active, cand_idx ? row_mass[r] : 0ull, uniform[r], s_list,
+                                            s_wave, s_piece, s_pick);
+        if (threadIdx.x == 0) out[r] = at < 0 ? best : (idx_of ? idx_of[at] : at);
+        return;
+    }
+    // kept set = { j : w_j >= threshold }; the threshold starts at 0 (everything)
+    uint32_t threshold = 0u;
     if (k_active && k < vocab)        // (a list of exactly k candidates is the top k)
         threshold = select_by_count(w, vocab, static_cast<unsigned int>(k), hist, &s_a, &s_need);
     const float p = top_p[r];
