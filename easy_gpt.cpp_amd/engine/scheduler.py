@@ -61,6 +61,15 @@ class Request:
     def all_tokens(self) -> list[int]:
         return self.prompt + self.output
 
+    def tokens(self, start: int, count: int) -> list[int]:
+        """all_tokens()[start : start + count] without building the whole list (a decoding request asks for one)."""
+        n = len(self.prompt)
+        if start >= n:
+            return self.output[start - n : start - n + count]
+        if start + count <= n:
+            return self.prompt[start : start + count]
+        return self.prompt[start:] + self.output[: start + count - n]
+
     def pending(self) -> int:
         """Tokens not yet in the cache: the rest of the prompt, or the one last sampled token."""
         return len(self.prompt) + len(self.output) - self.computed
@@ -179,8 +188,9 @@ class Scheduler:
             if restart:
                 continue
             # 2. prompt portions of running requests, in order of admission
+            planned = {id(e.request) for e in entries}
             for r in self.running:
-                if (r.pending() == 1 and r.output) or budget < 1 or any(e.request is r for e in entries):
+                if (r.pending() == 1 and r.output) or budget < 1 or id(r) in planned:
                     continue
                 count = min(r.pending(), cfg.prefill_chunk, budget)
                 while count > 0 and not take(r, count):
@@ -242,7 +252,7 @@ class Scheduler:
         t0 = time.perf_counter()
         batch = []
         for e in entries:
-            toks = e.request.all_tokens()[e.start : e.start + e.count]
+            toks = e.request.tokens(e.start, e.count)
             batch.append(StepEntry(e.request.request_id, toks, [e.count - 1] if e.samples else []))
         logits = self.engine.step(batch)
         finished: list[Request] = []
