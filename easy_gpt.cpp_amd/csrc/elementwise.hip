@@ -58,16 +58,26 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
     const bool has_delta = delta.present();
     const size_t dbase = src * hidden;
     const bool write_back = (rows == nullptr) && has_delta;
+    // a row that the workgroup covers in one pass stays in registers, with its norm weight, for the second pass:
+    // the sum over the workgroup is then the only wait between the loads and the store
+    const bool one_pass = hidden <= static_cast<int>(blockDim.x);
+    float kept = 0.f, kept_w = 0.f;
     float ss = 0.f;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = hrow[j];
+        if (one_pass) kept_w = to_float(weight[j]);
         if (has_delta) v += delta.at(dbase + j);
         if (write_back) hrow[j] = v;
         ss += v * v;
+        kept = v;
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
     T* orow = out + static_cast<size_t>(r) * hidden;
+    if (one_pass) {
+        if (static_cast<int>(threadIdx.x) < hidden) orow[threadIdx.x] = from_float<T>(kept * inv * kept_w);
+        return;
+    }
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
         float v = hrow[j];                       // already updated when written back
         if (has_delta && !write_back) v += delta.at(dbase + j);
