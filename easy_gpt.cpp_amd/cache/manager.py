@@ -43,7 +43,7 @@ def _library():
         from ..csrc import build
 
         lib = ctypes.CDLL(build.ensure_host_built())
-        if lib.egh_abi_version() != 1:
+        if lib.egh_abi_version() != 2:
             raise RuntimeError("the host library has an unexpected ABI version")
         vp, i = ctypes.c_void_p, ctypes.c_int
         sigs = {
@@ -55,6 +55,7 @@ def _library():
             "egh_reserve": ([vp, i, vp, vp, vp], i), "egh_commit": ([vp, i, vp, vp], i),
             "egh_slot_index": ([vp, i, i, i], i), "egh_check": ([vp, vp, i], i),
             "egh_fill_decode": ([vp, i, vp, vp, vp, vp, vp], i),
+            "egh_fill_decode_rows": ([vp, i, i, vp, vp, vp, vp, vp], i),
             "egh_fill_step": ([vp, i, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp], i),
         }
         for name, (args, res) in sigs.items():
@@ -262,10 +263,13 @@ class CacheManager:
             assert rc.table_lens == [self._lib.egh_table_len(self._core, rc.handle, g) for g in range(len(self.groups))]
 
     # ------------------------------------------------------------------ a step's metadata, written by the library
-    def fill_decode(self, handles, widths, small_ptr: int, tab_ptr: int, row_state_ptr: int) -> bool:
+    def fill_decode(self, handles, widths, small_ptr: int, tab_ptr: int, row_state_ptr: int, rows: int | None = None) -> bool:
         """One token per request: positions, lengths, slots and (where they changed) block-table rows, written
-        into the caller's int32 buffers (layout in csrc/host/cache_core.h).  True if a table row was rewritten."""
-        code = self._lib.egh_fill_decode(self._core, len(handles), handles, widths, small_ptr, tab_ptr, row_state_ptr)
+        into the caller's int32 buffers (layout in csrc/host/cache_core.h), which are laid out for `rows` requests
+        (default: as many as there are handles).  True if a table row was rewritten."""
+        n = len(handles)
+        code = self._lib.egh_fill_decode_rows(self._core, n, n if rows is None else rows, handles, widths, small_ptr,
+                                              tab_ptr, row_state_ptr)
         if code == EGH_NO_PAGE:
             raise RuntimeError("a token of this step would be stored in a page that was given back")
         if code < 0:

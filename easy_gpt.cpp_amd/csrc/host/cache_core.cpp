@@ -66,7 +66,7 @@ struct EghCore {
 
 extern "C" {
 
-int egh_abi_version(void) { return 1; }
+int egh_abi_version(void) { return 2; }
 
 EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pages, int page_size, int max_requests) {
     if (n_groups < 0 || page_size < 1 || max_requests < 0 || (n_groups > 0 && (!windows || !num_pages))) return nullptr;
@@ -278,9 +278,9 @@ int egh_check(const EghCore* c, char* message, int cap) {
     return EGH_OK;
 }
 
-int egh_fill_decode(const EghCore* c, int b, const int32_t* handles, const int32_t* widths, int32_t* small,
-                    int32_t* tab, int64_t* row_state) {
-    if (!c || b <= 0 || !handles || !small || !row_state || (c->n_groups() > 0 && (!widths || !tab)))
+int egh_fill_decode_rows(const EghCore* c, int b, int rows, const int32_t* handles, const int32_t* widths,
+                         int32_t* small, int32_t* tab, int64_t* row_state) {
+    if (!c || b <= 0 || rows < b || !handles || !small || !row_state || (c->n_groups() > 0 && (!widths || !tab)))
         return EGH_BAD_ARGUMENT;
     const int ng = c->n_groups(), ps = c->page_size;
     int changed = 0;
@@ -289,18 +289,18 @@ int egh_fill_decode(const EghCore* c, int b, const int32_t* handles, const int32
         const Request* r = c->get(handles[i]);
         if (!r) return EGH_BAD_HANDLE;
         const int pos = r->num_tokens;
-        small[1 * b + i] = pos;
-        small[2 * b + i] = i;
-        small[3 * b + i] = 1;
-        small[4 * b + i] = pos + 1;
-        small[5 * b + i] = r->slot;
-        small[6 * b + i] = i;
+        small[1 * rows + i] = pos;
+        small[2 * rows + i] = i;
+        small[3 * rows + i] = 1;
+        small[4 * rows + i] = pos + 1;
+        small[5 * rows + i] = r->slot;
+        small[6 * rows + i] = i;
         for (int g = 0; g < ng; ++g) {
             const std::vector<int32_t>& t = r->tables[g];
             const int idx = pos / ps;
             if (idx >= static_cast<int>(t.size()) || t[idx] < 0) return EGH_NO_PAGE;
             if (static_cast<int>(t.size()) > widths[g]) return EGH_BAD_ARGUMENT;
-            small[(7 + g) * b + i] = t[idx] * ps + pos % ps;
+            small[(7 + g) * rows + i] = t[idx] * ps + pos % ps;
         }
     }
     for (int g = 0; g < ng; ++g) {
@@ -314,13 +314,18 @@ int egh_fill_decode(const EghCore* c, int b, const int32_t* handles, const int32
                 changed = 1;
             }
         }
-        tab_off += static_cast<size_t>(b) * widths[g];
+        tab_off += static_cast<size_t>(rows) * widths[g];
     }
     for (int i = 0; i < b; ++i) {
         row_state[2 * i] = handles[i];
         row_state[2 * i + 1] = c->get(handles[i])->version;
     }
     return changed;
+}
+
+int egh_fill_decode(const EghCore* c, int b, const int32_t* handles, const int32_t* widths, int32_t* small,
+                    int32_t* tab, int64_t* row_state) {
+    return egh_fill_decode_rows(c, b, b, handles, widths, small, tab, row_state);
 }
 
 int egh_fill_step(const EghCore* c, int b, const int32_t* handles, const int32_t* counts, const int32_t* widths,

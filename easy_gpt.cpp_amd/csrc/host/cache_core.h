@@ -55,6 +55,11 @@ int egh_check(const EghCore* c, char* message, int cap);
 // says they changed.  Returns 1 if a table row was rewritten, 0 if not, < 0 on error.
 int egh_fill_decode(const EghCore* c, int b, const int32_t* handles, const int32_t* widths, int32_t* small,
                     int32_t* tab, int64_t* row_state);
+// The same into buffers laid out for `rows` >= b requests (a batch padded to a size that a graph exists for): the
+// first b entries of every row of `small` and the first b table rows of every group are written, the rest is the
+// caller's.
+int egh_fill_decode_rows(const EghCore* c, int b, int rows, const int32_t* handles, const int32_t* widths,
+                         int32_t* small, int32_t* tab, int64_t* row_state);
 // Any mix: counts[i] tokens per request, token-major outputs of T = sum counts entries (positions, slots per
 // group [n_groups][T]), per-request outputs of b entries, tables per group [b][widths[g]] concatenated.
 int egh_fill_step(const EghCore* c, int b, const int32_t* handles, const int32_t* counts, const int32_t* widths,

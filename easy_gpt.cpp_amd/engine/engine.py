@@ -263,16 +263,20 @@ class Engine:
         if starters:
             self.cache.reserve_step(starters, [1] * len(starters))
         b = len(rcs)
+        # Beyond 16 requests the batch is padded to a multiple of 8 with rows of one token at position 0 on a page
+        # that no request owns: requests finish one by one, and every batch size would otherwise be a graph of its
+        # own, run kernel by kernel on its first visits (up to 16 the kernels' shapes follow the batch size).
+        rows = b if b <= 16 else -(-b // 8) * 8
         widths = self._table_widths(rcs)
         # The kernels choose their shape (key splits of the attention) by the longest context, and a graph holds
         # one choice: contexts are bucketed in steps of 512 tokens beside the table widths.
         kv_bound = -(-(max(rc.num_tokens for rc in rcs) + 1) // 512) * 512
-        key = (b, tuple(widths), kv_bound)
-        plan = self._plan(self._decode_plans, key, lambda: _DecodePlan(self, b, widths, kv_bound))
+        key = (rows, tuple(widths), kv_bound)
+        plan = self._plan(self._decode_plans, key, lambda: _DecodePlan(self, rows, widths, kv_bound))
         plan.fill(rcs, tokens)
         logits = self._run(plan)
-        self.cache.commit_step(rcs, plan.ones)
-        return logits
+        self.cache.commit_step(rcs, [1] * b)
+        return logits[:b]
 
     # ------------------------------------------------------------------ what the steps from graphs share
     MAX_PLANS = 128      # captured graphs kept per kind of step; the oldest goes when one more is needed
@@ -520,8 +524,8 @@ class _DecodePlan:
         )
         self.row_state = np.full(2 * b, -1, dtype=np.int64)     # per row: (handle, table version) last written
         self.c_widths = _ints(self.widths)
-        self.ones = [1] * b
         self.cache = engine.cache
+        self.pad_page, self.page_size = engine._pad_first_page, ps
         self.copied = None           # event after the last host-to-device copy
         self.graph = None
         self.logits = None
@@ -530,13 +534,36 @@ class _DecodePlan:
     def fill(self, rcs, tokens) -> None:
         if self.copied is not None:
             self.copied.synchronize()                       # the pinned mirror is free again
-        b = self.batch
+        rows, b = self.batch, len(rcs)
         self.np_small[0:b] = tokens
         handles = _ints([rc.handle for rc in rcs])
         tables_changed = self.cache.fill_decode(handles, self.c_widths, self.host_small.data_ptr(),
-                                                self.host_tab.data_ptr(), self.row_state.ctypes.data)
-        self.ctx.kv_len_host = [rc.num_tokens + 1 for rc in rcs]
-        self.ctx.state_slots_host = [rc.slot for rc in rcs]
+                                                self.host_tab.data_ptr(), self.row_state.ctypes.data, rows=rows)
+        self.ctx.kv_len_host = [rc.num_tokens + 1 for rc in rcs] + [1] * (rows - b)
+        self.ctx.state_slots_host = [rc.slot for rc in rcs] + [0] * (rows - b)
+        if b < rows:
+            # the padding: token 0 at position 0, alone in its context, all on the first slot of the padding's page
+            # (the same key and value from every such row)
+            n_groups = len(self.widths)
+            small = self.np_small.reshape(7 + n_groups, rows)
+            small[0, b:] = 0
+            small[1, b:] = 0
+            small[2, b:] = np.arange(b, rows, dtype=np.int32)
+            small[3, b:] = 1
+            small[4, b:] = 1
+            small[5, b:] = 0
+            small[6, b:] = np.arange(b, rows, dtype=np.int32)
+            small[7:, b:] = self.pad_page * self.page_size
+            tab = self.host_tab.numpy()
+            off = 0
+            for w in self.widths:
+                for i in range(b, rows):
+                    if self.row_state[2 * i] != -2:          # the row held a request's table (or nothing yet)
+                        tab[off + i * w : off + (i + 1) * w] = -1
+                        tab[off + i * w] = self.pad_page
+                        tables_changed = True
+                off += rows * w
+            self.row_state[2 * b : 2 * rows : 2] = -2
         self.dev_small.copy_(self.host_small, non_blocking=True)
         if tables_changed:
             self.dev_tab.copy_(self.host_tab, non_blocking=True)

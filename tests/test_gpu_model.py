@@ -329,6 +329,42 @@ def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph
     assert len(plans) == 1 and plans[0].graph is not None          # two eager visits, then replays
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_batches_that_shrink_share_the_graph_of_their_padded_size(sharp_models, dtype):
+    # 23 requests decode side by side and end one by one: batches of 23 down to 17 run from one graph of 24 rows
+    # (rows that were a request become padding and the other way round), 16 and fewer from graphs of their own size;
+    # every step is compared with the plain implementation
+    m = sharp_models["D"]
+    n_req, prompt = 23, 6
+    lens = [prompt + 4 + i for i in range(n_req)]                    # request i decodes 4 + i tokens after its prompt
+    reqs = H.make_requests(TINY["D"][0]["vocab_size"], lens, seed=71)
+    ref = H.plain_rows(m, reqs, bf16_weights=(dtype == "bfloat16"))
+    ids = list(reqs)
+    trace = [H.step_record(0, [(rid, reqs[rid][:prompt], [prompt - 1]) for rid in ids])]
+    fed = {rid: prompt for rid in ids}
+    live = list(ids)
+    step = 1
+    while live:
+        # a request that is put in front of the others now and then: rows change their owners
+        order = live[step % 3:] + live[:step % 3]
+        entries = [(rid, [reqs[rid][fed[rid]]], [0]) for rid in order]
+        for rid in order:
+            fed[rid] += 1
+        ended = [rid for rid in order if fed[rid] == len(reqs[rid])]
+        trace.append(H.step_record(step, entries, ended))
+        live = [rid for rid in live if rid not in ended]
+        step += 1
+    eng = engine_for(m, dtype, max_tokens=n_req * 64, max_requests=n_req)
+    rows = H.replay(eng, trace)
+    assert len(rows) == n_req + sum(n - prompt for n in lens)
+    H.assert_rows_match(rows, ref, tol_of(dtype), "decode batches padded to the size of a graph")
+    sizes = sorted({key[0] for key in eng._decode_plans})
+    assert 24 in sizes and not any(16 < b < 24 for b in sizes), sizes
+    padded = [p for key, p in eng._decode_plans.items() if key[0] == 24]
+    assert all(p.graph is not None for p in padded)                  # visited often enough to be captured and replayed
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
 def test_a_layer_with_large_matrices_takes_the_kernels_that_are_not_folded(tmp_path):
     # one layer whose gate/up matrix has 67M elements and whose width is 2,048: with few rows the norm before gate/up
     # and SwiGLU before down then run as kernels of their own (folded into the products they would be computed again
