@@ -101,7 +101,7 @@ class Engine:
         self._row_plans: dict = {}
         self._padded_plans: dict = {}
         self.graph_tokens = 2048    # steps of at most this many tokens run from a graph for their padded size
-        self.capture_after = 2      # a shape's graph is captured at this visit (None: never, the same kernels one by one)
+        self.capture_after = 1      # a shape's graph is captured right after this visit (None: never, the same kernels one by one)
         self.graph_rows = 64        # steps of at most this many tokens in all run as rows of one token each,
         self.graph_row_reads = 1 << 18      # if the tokens of their portions read at most this many keys in all
         self._graph_pool = None

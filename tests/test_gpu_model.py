@@ -326,7 +326,7 @@ def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph
     assert len(rows) == n_req * (1 + steps)
     H.assert_rows_match(rows, ref, H.BF16_TOL, "library products in the decode graph")
     plans = list(eng._decode_plans.values())
-    assert len(plans) == 1 and plans[0].graph is not None          # two eager visits, then replays
+    assert len(plans) == 1 and plans[0].graph is not None          # an eager visit, then replays
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
