@@ -553,14 +553,23 @@ class HipKernels:
         output projection combines are read by every column of workgroups there, so they stay few."""
         key_blocks = -(-max_kv_len // 32)
         pairs = b * nkv
-        n_waves = 8 if (hd == 64 and pairs * key_blocks <= 8192) else 4
-        per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (4 if hd == 64 else 2))
-        wanted = -(-key_blocks // per_round)
-        # the output projection combines up to 8 parts in registers; more only for few requests with contexts
-        # so long that 8 parts would leave every wavefront four rounds or more
-        most = 16 if (combine or (pairs <= 8 and wanted >= 32)) else 8
-        n_splits = max(1, min(wanted, most, max(1, 2048 // pairs)))
-        return n_splits, n_waves
+
+        def splits_for(n_waves):
+            per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (4 if hd == 64 else 2))
+            wanted = -(-key_blocks // per_round)
+            # the output projection combines up to 8 parts in registers; more only for few requests with contexts
+            # so long that 8 parts would leave every wavefront four rounds or more
+            most = 16 if (combine or (pairs <= 8 and wanted >= 32)) else 8
+            return max(1, min(wanted, most, max(1, 2048 // pairs)))
+
+        if hd == 64 and pairs * key_blocks <= 8192:
+            n_splits = splits_for(8)
+            # wide workgroups as long as each has a CU of its own: a few more than CUs, and those that share one set
+            # the kernel's time (measured at 2,048-token contexts: 1.84 ms a step at batch 44 and 48 with 264 and 288
+            # workgroups of eight wavefronts, 1.66 with 440 and 480 of four; 1.57 either way at batch 40)
+            if pairs * n_splits <= 256:
+                return n_splits, 8
+        return splits_for(4), 4
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
                                k_cache, v_cache, block_table, q_start, kv_len, nq, nkv, hd, page_size, scale, window,
