@@ -560,7 +560,11 @@ class HipKernels:
             # the output projection combines up to 8 parts in registers; more only for few requests with contexts
             # so long that 8 parts would leave every wavefront four rounds or more
             most = 16 if (combine or (pairs <= 8 and wanted >= 32)) else 8
-            return max(1, min(wanted, most, max(1, 2048 // pairs)))
+            # head size 128: at most two workgroups per CU, beyond which the kernel's variant with fewer loads in
+            # flight runs (measured at the 1.5B sizes, 2,048-token contexts: 2.42 ms a step with 512 workgroups at
+            # batch 32 against 2.63 with 576, 3.20 with 512 at batch 64 against 3.48 with 1,152)
+            room = 2048 if hd == 64 else 512
+            return max(1, min(wanted, most, max(1, room // pairs)))
 
         if hd == 64 and pairs * key_blocks <= 8192:
             n_splits = splits_for(8)
