@@ -255,6 +255,7 @@ class HipKernels:
         return -(-steps // per)
 
     fused_rows = 16     # products with a computed x operand take at most this many rows
+    normed_rows_cols = 400_000   # rows x columns beyond which the norm is not folded into a product
 
     @staticmethod
     def _normed_shape(n: int, k: int) -> tuple[int, int]:
@@ -282,10 +283,12 @@ class HipKernels:
         n = w.shape[0]
         if w.dtype != _BF16 or not 0 < t <= self.fused_rows or k % 8 or not h.is_cuda:
             return None
-        if splits is None and waves is None and (t * n > 400_000 or n * k >= 64 << 20):
+        if splits is None and waves is None and (t * n > self.normed_rows_cols or n * k >= 64 << 20
+                                                 or (n * k >= 16 << 20 and t * n > 100_000)):
             # every workgroup reads its k range of all rows of h and of delta's partial sums: on a matrix this large
             # (or with this many rows and columns) that costs more than a norm kernel of its own (measured on a
-            # 37,888 x 3,584 product behind 14 partial sums: 80 us against 6 + 58)
+            # 37,888 x 3,584 product behind 14 partial sums: 80 us against 6 + 58; on a 17,920 x 1,536 one with 16 rows
+            # 26 us against 5 + 13, and from 6 rows on the separate kernels win there, which they never do on 9,728 x 896)
             return None
         if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
             return None
