@@ -279,7 +279,7 @@ class Engine:
         return logits[:b]
 
     # ------------------------------------------------------------------ what the steps from graphs share
-    MAX_PLANS = 128      # captured graphs kept per kind of step; the oldest goes when one more is needed
+    MAX_PLANS = 128      # captured graphs kept per kind of step; the least recently used goes when one more is needed
 
     def _table_widths(self, rcs, at_least: int = 0) -> list[int]:
         """Block-table widths of a plan: for each group the next power of two (from 4) that holds the longest table."""
@@ -310,11 +310,12 @@ class Engine:
         return logits
 
     def _plan(self, plans: dict, key, make):
-        plan = plans.get(key)
+        plan = plans.pop(key, None)
         if plan is None:
             if len(plans) >= self.MAX_PLANS:
-                plans.pop(next(iter(plans)))
-            plan = plans[key] = make()
+                plans.pop(next(iter(plans)))               # the one that was used longest ago
+            plan = make()
+        plans[key] = plan                                  # most recently used last
         return plan
 
     # ------------------------------------------------------------------ few tokens in all, from a graph
