@@ -153,9 +153,35 @@ class Scheduler:
         self.stats.preemptions += 1
         self.waiting.appendleft(r)
 
+    def _plan_decode_only(self) -> list[PlannedEntry] | None:
+        """The common step of a busy engine, decided in one pass: nobody waits, every running request decodes, and
+        the pages that their next tokens start are free.  The same entries as the general rules give; None if any
+        of this does not hold (the general rules then decide, and may preempt)."""
+        running = self.running
+        if self.waiting or not running or len(running) > self.config.max_tokens_per_step:
+            return None
+        cache = self.cache
+        requests, ps = cache.requests, cache.page_size
+        need = [0] * len(cache.pools)
+        for r in running:
+            if not r.output or len(r.prompt) + len(r.output) - r.computed != 1:
+                return None
+            rc = requests[r.request_id]
+            want = (rc.num_tokens + ps) // ps                   # pages that hold num_tokens + 1 tokens
+            for g, have in enumerate(rc.table_lens):
+                if want > have:
+                    need[g] += want - have
+        for n, pool in zip(need, cache.pools):
+            if n > pool.free_count:
+                return None
+        return [PlannedEntry(r, r.computed, 1, True) for r in running]
+
     def plan(self) -> list[PlannedEntry]:
         """Decide the next step.  May admit, preempt or fail requests; returns what to run."""
         cfg = self.config
+        entries = self._plan_decode_only()
+        if entries is not None:
+            return entries
         while True:
             budget = cfg.max_tokens_per_step
             promised = [0] * len(self.cache.pools)

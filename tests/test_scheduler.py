@@ -202,6 +202,37 @@ def test_random_workloads_finish_with_the_right_tokens(seed):
     assert eng.cache.free_pages() == [eng.cache.pools[0].num_pages]
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_the_one_pass_decision_for_decoding_requests_is_the_general_one(seed):
+    # while every running request decodes and nobody waits, the step is decided in one pass: whenever that pass
+    # decides at all, it names the same entries as the general rules; when pages run short it leaves the decision
+    # (and the preemption) to them
+    rng = random.Random(seed)
+    eng = FakeEngine(num_pages=rng.choice([14, 30, 200]), page_size=4, max_requests=6)
+    s = Scheduler(eng, SchedulerConfig(max_active=6, max_admit_per_step=6, max_tokens_per_step=64, prefill_chunk=16))
+    for i in range(6):
+        s.add(Request(i, [rng.randrange(1, VOCAB) for _ in range(rng.randint(1, 9))], GREEDY, max_new_tokens=rng.randint(2, 12)))
+    decided = 0
+    for _ in range(400):
+        if not s.has_work():
+            break
+        fast = s._plan_decode_only()
+        if fast is not None:
+            decided += 1
+            s._plan_decode_only = lambda: None                    # the general rules alone
+            try:
+                general = s.plan()
+            finally:
+                del s._plan_decode_only
+            assert [(e.request.request_id, e.start, e.count, e.samples) for e in fast] == \
+                   [(e.request.request_id, e.start, e.count, e.samples) for e in general]
+        s.step()
+    assert not s.has_work() and decided > 0
+    for r in s.done:
+        if r.status == "finished":
+            assert r.output == expected_output(r.prompt, len(r.output))
+
+
 def test_temperature_sampling_does_not_depend_on_neighbours():
     outs = []
     for others in (0, 3):
