@@ -105,6 +105,8 @@ def main() -> int:
                     help="tokens each request holds before decoding starts (default: the record's 2,048)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-tune", action="store_true",
+                    help="take the library's first choice for its matrix products instead of the measured one")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
     ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
@@ -158,7 +160,8 @@ def main() -> int:
     if args.serve:
         max_batch, tokens_per_request = SERVE_REQUESTS, -(-(2048 + SERVE_NEW_TOKENS) // page_size) * page_size
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
-                             max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1)
+                             max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1,
+                             tune_products=not args.no_tune)
     for f in os.listdir(tmp):
         os.remove(os.path.join(tmp, f))
     os.rmdir(tmp)
@@ -260,7 +263,7 @@ def main() -> int:
             "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]),
             "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": new_tokens,
             "page_size": page_size, "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "sampling": "greedy", "parallelism": "single GPU",
+            "sampling": "greedy", "parallelism": "single GPU", "library_products": "first choice" if args.no_tune else "measured",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 5)},

@@ -37,6 +37,7 @@ USAGE = """Usage: easy_llm [--model <dir>] [--prompt-file <path>] [--max-steps <
       --prefill-chunk <n>    Largest prompt portion in one step (default: 512)
       --cache-tokens <n>     Tokens the paged cache holds (default: 65536)
       --page-size <n>        Tokens per cache page (default: 16)
+      --tune-products        Choose the library's matrix products by measurement (about a second per new shape)
   -h, --help                Show this help message
 Examples:
   bin/easy_llm --model data/model --max-steps 128 "1 2 3"
@@ -71,6 +72,7 @@ class CliOptions:
     prefill_chunk: int = 512
     cache_tokens: int = 65536
     page_size: int = 16
+    tune_products: bool = False
 
 
 class CliError(ValueError):
@@ -162,6 +164,8 @@ def parse_args(argv: list[str]) -> CliOptions:
                 raise CliError("max-new-tokens must be greater than 0")
         elif arg == "--ignore-eos":
             o.ignore_eos = True
+        elif arg == "--tune-products":
+            o.tune_products = True
         elif arg in ("--max-tokens-per-step", "--prefill-chunk", "--cache-tokens", "--page-size"):
             name = arg[2:].replace("-", "_")
             v = _number(int, value(arg), arg[2:].replace("-", " "))
@@ -238,7 +242,7 @@ def main(argv: list[str] | None = None) -> int:
 
     llm = LLM(o.model, dtype=o.dtype, cache_tokens=o.cache_tokens, page_size=o.page_size,
               max_active=o.serve_max_active, max_admit_per_step=o.serve_prefill_batch,
-              max_tokens_per_step=o.max_tokens_per_step, prefill_chunk=o.prefill_chunk)
+              max_tokens_per_step=o.max_tokens_per_step, prefill_chunk=o.prefill_chunk, tune_products=o.tune_products)
     last = [time.perf_counter()]
 
     def on_step(sched):

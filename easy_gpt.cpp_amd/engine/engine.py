@@ -69,14 +69,20 @@ class Engine:
         num_pages: int | None = None,
         max_requests: int = 64,
         use_graphs: bool = True,
+        tune_products: bool = False,
     ):
         """max_tokens: the most tokens live requests hold at any time (each request's count
         rounded up to a page); the pools are made for that many.  num_pages sets the page
-        count directly."""
+        count directly.  tune_products: the library's many-row products are chosen by measurement at a shape's
+        first visit (`kernels.tune_library_products`: process-wide, about a second per new shape)."""
         if model.device is None:
             raise RuntimeError("the model has no weights yet (Model.load)")
         self.model = model
         self.device = model.device
+        if tune_products and self.device.type == "cuda":
+            from .. import kernels
+
+            kernels.tune_library_products(True)
         self.page_size = int(page_size)
         if num_pages is None:
             if max_tokens is None:

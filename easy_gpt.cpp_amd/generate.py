@@ -29,9 +29,10 @@ class LLM:
         max_admit_per_step: int = 4,
         max_tokens_per_step: int = 2048,
         prefill_chunk: int = 512,
+        tune_products: bool = False,
     ):
         self.engine = Engine.from_dir(model_dir, dtype=dtype, device=device, page_size=page_size,
-                                      max_tokens=cache_tokens, max_requests=max_active)
+                                      max_tokens=cache_tokens, max_requests=max_active, tune_products=tune_products)
         self.config = SchedulerConfig(max_active=max_active, max_admit_per_step=max_admit_per_step,
                                       max_tokens_per_step=max_tokens_per_step, prefill_chunk=prefill_chunk)
         self.eos_token_id = self.engine.model.spec.eos_token_id

@@ -52,3 +52,30 @@ def use_backend(obj) -> None:
     """Install `obj` as the backend (None restores the default).  For tests."""
     global _backend
     _backend = obj
+
+
+_tuning_dir = None
+library_tuning = False      # whether the library's bfloat16 products are chosen by measurement (tune_library_products)
+
+
+def tune_library_products(enable: bool = True) -> None:
+    """Let the library's matrix products (the many-row bfloat16 products, torch.mm) be chosen by measurement: the
+    first time a shape is multiplied outside a graph capture, torch's TunableOp times the library's candidates for
+    it (about a second per shape with the limits set here) and keeps the fastest for the life of the process; the
+    library's own first choice is up to a third slower on some shapes (the 2,048 x 9,728 x 896 product: 53 us
+    against 40).  Process-wide, off unless asked for: a step with new shapes waits for the measurement, and which
+    candidate wins may differ from run to run, and with it the last bits of a result."""
+    global _tuning_dir, library_tuning
+    import torch.cuda.tunable as tunable
+
+    if enable and _tuning_dir is None:
+        import os
+        import tempfile
+
+        _tuning_dir = tempfile.TemporaryDirectory(prefix="egpt_tuning_")      # TunableOp writes its picks to a file
+        tunable.set_filename(os.path.join(_tuning_dir.name, "picks.csv"))
+        tunable.set_max_tuning_duration(30)
+        tunable.set_max_tuning_iterations(20)
+    tunable.enable(bool(enable))
+    tunable.tuning_enable(bool(enable))
+    library_tuning = bool(enable)

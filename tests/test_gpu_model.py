@@ -397,6 +397,29 @@ def test_a_layer_with_large_matrices_takes_the_kernels_that_are_not_folded(tmp_p
     H.assert_rows_match(rows, ref, H.BF16_TOL, "large matrices, few rows")
 
 
+def test_library_products_chosen_by_measurement(sharp_by_dtype):
+    # with tune_products the library's many-row products are measured at their first visit and the fastest candidate
+    # kept; the products with float32 output stay with the library's first choice.  Whatever is chosen, the logits
+    # are the plain implementation's, on the first visit (kernel by kernel) and from the replayed graph
+    from easy_gpt.cpp_amd import kernels
+
+    m = sharp_by_dtype["bfloat16"]["D"]
+    reqs = H.make_requests(TINY["D"][0]["vocab_size"], [200, 150], seed=81)
+    ref = H.plain_rows(m, reqs, bf16_weights=True)
+    try:
+        eng = engine_for(m, "bfloat16", max_tokens=1024, tune_products=True)
+        assert kernels.library_tuning and torch.cuda.tunable.is_enabled()
+        for visit in range(3):                               # the same shapes again: the graph of the first visit
+            trace = [H.step_record(0, [(rid, ids, list(range(len(ids)))) for rid, ids in reqs.items()], list(reqs))]
+            rows = H.replay(eng, trace)
+            H.assert_rows_match(rows, ref, H.BF16_TOL, f"tuned library products, visit {visit}")
+        assert any(p.graph is not None for p in eng._padded_plans.values())
+        assert torch.cuda.tunable.is_enabled()               # switched back on after every float32-output product
+    finally:
+        kernels.tune_library_products(False)
+    assert not kernels.library_tuning and not torch.cuda.tunable.is_enabled()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens_of_a_sequence(tiny_models, name, dtype):
