@@ -308,7 +308,9 @@ class Engine:
         plan.runs += 1
         if self.capture_after is not None and plan.runs >= self.capture_after:
             graph = torch.cuda.CUDAGraph()
-            if self._graph_pool is None:
+            plans = (self._decode_plans, self._row_plans, self._padded_plans)
+            if self._graph_pool is None or not any(p.graph is not None for d in plans for p in d.values()):
+                # the first graph, or the first after every earlier one was dropped (their pool went with the last)
                 self._graph_pool = torch.cuda.graph_pool_handle()
             torch.cuda.synchronize()
             plan.logits = _capture(graph, self._graph_pool, lambda: self.model.forward(plan.ctx))
