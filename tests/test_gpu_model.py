@@ -256,6 +256,25 @@ def test_plans_are_dropped_and_made_again_when_there_are_too_many(sharp_by_dtype
     assert len(eng._padded_plans) <= 2 and len(eng._row_plans) <= 2 and s_i >= 6
 
 
+def test_a_graph_is_captured_after_every_earlier_one_was_dropped(sharp_by_dtype):
+    # one graph kept per kind of step: every new shape drops the only graph there is, and the next capture starts
+    # from nothing again (the pool that the dropped graphs shared went with the last of them)
+    cfg = TINY["D"][0]
+    model_dir = sharp_by_dtype["bfloat16"]["D"]
+    reqs = H.make_requests(cfg["vocab_size"], [300], seed=53)
+    ref = H.plain_rows(model_dir, reqs, bf16_weights=True)
+    eng = engine_for(model_dir, "bfloat16", max_tokens=640)
+    eng.MAX_PLANS = 1
+    sizes, fed, trace = [70, 130, 70, 30], 0, []
+    while fed < 300:
+        n = min(sizes[len(trace) % len(sizes)], 300 - fed)
+        trace.append(H.step_record(len(trace), [("r0", reqs["r0"][fed : fed + n], [0, n - 1])]))
+        fed += n
+    rows = H.replay(eng, trace)
+    H.assert_rows_match(rows, ref, H.BF16_TOL, "one graph kept")
+    assert len(eng._padded_plans) == 1 and len(trace) >= 4
+
+
 def test_an_engine_is_freed_when_its_last_reference_goes(tiny_models):
     # its plans hold no reference back to it: if they did, its device memory and graphs would be freed whenever the
     # collector of reference cycles runs, which may be in the middle of another engine's graph capture
