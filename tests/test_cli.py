@@ -49,6 +49,7 @@ def test_short_and_long_options():
                     "-f", "p.txt", "--model", "dir", "--dtype", "float32", "--max-new-tokens", "5", "--ignore-eos"])
     assert (o.max_steps, o.temperature, o.top_p, o.top_k, o.seed, o.use_greedy) == (64, 0.7, 0.9, 40, 7, True)
     assert (o.prompt_file, o.model, o.dtype, o.max_new_tokens, o.ignore_eos) == ("p.txt", "dir", "float32", 5, True)
+    assert parse_args(["--tune-products", "1 2"]).tune_products and not parse_args(["1 2"]).tune_products
     assert parse_args(["-h", "--bogus"]).show_help
 
 
