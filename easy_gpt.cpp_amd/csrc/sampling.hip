@@ -374,13 +374,53 @@ __global__ __launch_bounds__(64) void sample_plan_kernel(const float* __restrict
                                                          const unsigned int* __restrict__ piece_count,
                                                          const unsigned long long* __restrict__ piece_mass,
                                                          uint32_t* __restrict__ cutoff, int32_t* __restrict__ offsets,
-                                                         unsigned long long* __restrict__ row_mass, int vocab) {
+                                                         unsigned long long* __restrict__ row_mass,
+                                                         const float* __restrict__ uniform, int32_t* __restrict__ direct_piece,
+                                                         unsigned long long* __restrict__ direct_target, int vocab) {
     __shared__ unsigned int s_count[kTopBins + 1];
     __shared__ unsigned long long s_mass[kTopBins + 1];
     __shared__ int s_bin;
     const int r = blockIdx.x, t = threadIdx.x;
-    if (!(temperature[r] > 0.f)) return;
+    if (!(temperature[r] > 0.f)) {
+        if (t == 0) direct_piece[r] = -1;
+        return;
+    }
     const size_t base = static_cast<size_t>(r) * kSamplePieces * (kTopBins + 1);
+    {
+        // Neither cut is asked for: the draw needs no selection.  The pieces' masses are known, so the drawn point
+        // (in fixed point, of the whole row's mass) names its piece and what is left of it inside that piece; the
+        // last kernel walks that piece alone.  No list of candidates is made for such a row.
+        const int k = top_k[r];
+        const float p = top_p[r];
+        if (!(k > 0 && k < vocab) && !(p > 0.f && p < 1.f)) {
+            unsigned long long mine = 0ull;
+            if (t < kSamplePieces)
+                for (int i = 0; i <= kTopBins; ++i) mine += piece_mass[base + t * (kTopBins + 1) + i];
+            unsigned long long incl = mine;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const unsigned long long up = __shfl_up(incl, o, kWave);
+                if (t >= o) incl += up;
+            }
+            const unsigned long long total = __shfl(incl, kSamplePieces - 1, kWave);
+            const float u = fminf(fmaxf(uniform[r], 0.f), 0.99999994f);
+            unsigned long long target = static_cast<unsigned long long>(static_cast<double>(u) * static_cast<double>(total));
+            if (total > 0ull && target >= total) target = total - 1ull;
+            const bool here = t < kSamplePieces && incl > target && incl - mine <= target;   // at most one piece
+            const unsigned long long holders = __ballot(here);
+            const int piece = holders ? __ffsll(static_cast<long long>(holders)) - 1 : 0;      // (an empty row: piece 0)
+            const unsigned long long inside = __shfl(target - (incl - mine), piece, kWave);
+            if (t < kSamplePieces) offsets[r * (kSamplePieces + 1) + t] = 0;
+            if (t == 0) {
+                direct_piece[r] = piece;
+                direct_target[r] = holders ? inside : 0ull;
+                offsets[r * (kSamplePieces + 1) + kSamplePieces] = 0;
+                cutoff[r] = 0xffffffffu;
+                row_mass[r] = total;
+            }
+            return;
+        }
+    }
     if (t <= kTopBins) {
         unsigned int cv = 0u;
         unsigned long long mv = 0ull;
@@ -421,6 +461,7 @@ __global__ __launch_bounds__(64) void sample_plan_kernel(const float* __restrict
             }
         }
         s_bin = last;
+        direct_piece[r] = -1;
         cutoff[r] = last >= kTopBins ? 0u : static_cast<uint32_t>(127 - last) << 23;
         unsigned long long all = 0ull;
         for (int i = 0; i <= kTopBins; ++i) all += s_mass[i];
@@ -451,11 +492,12 @@ __global__ __launch_bounds__(64) void sample_plan_kernel(const float* __restrict
 __global__ __launch_bounds__(256) void sample_compact_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
                                                              const int32_t* __restrict__ best, const uint32_t* __restrict__ cutoff,
                                                              const int32_t* __restrict__ offsets, float* __restrict__ cand_w,
-                                                             int32_t* __restrict__ cand_idx, int vocab) {
+                                                             int32_t* __restrict__ cand_idx,
+                                                             const int32_t* __restrict__ direct_piece, int vocab) {
     __shared__ int s_wave[4];
     const int r = blockIdx.x, c = blockIdx.y;
     const float temp = temperature[r];
-    if (!(temp > 0.f)) return;
+    if (!(temp > 0.f) || direct_piece[r] >= 0) return;
     const float* row = logits + static_cast<size_t>(r) * vocab;
     const float mx = row[best[r]];
     const float inv_t = 1.0f / fmaxf(temp, 1e-6f);
@@ -552,6 +594,44 @@ __device__ int pick_from_short_list(const float* __restrict__ w, int n, bool cut
     return s_pick[0] != 0x7fffffff ? s_pick[0] : s_pick[1];
 }
 
+// The draw inside one piece of a row (tokens [begin, begin + n)) for a row without cuts: `target` is the drawn point
+// in the fixed-point mass of the piece.  Every thread takes a run of consecutive tokens, the runs' masses are summed
+// up over the workgroup in index order, and the thread whose run holds the point finds the token.  The weights
+// are computed as the counting kernel computed them, so the masses are the same integers.  Returns the token or
+// -1 (every thread).
+__device__ int pick_in_piece(const float* __restrict__ row, int begin, int n, float mx, float inv_t, unsigned long long target,
+                             unsigned long long* s_wave /* [16] */, int* s_pick /* [1] */) {
+    const int j = threadIdx.x, lane = j % kWave, wave = j / kWave, n_waves = blockDim.x / kWave;
+    const int run = (n + static_cast<int>(blockDim.x) - 1) / static_cast<int>(blockDim.x);
+    const int r_begin = min(n, j * run), r_end = min(n, r_begin + run);
+    unsigned long long mine = 0ull;
+    for (int i = r_begin; i < r_end; ++i) mine += fixed_of(weight_of(row[begin + i], mx, inv_t));
+    unsigned long long incl = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const unsigned long long up = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += up;
+    }
+    if (lane == kWave - 1) s_wave[wave] = incl;
+    if (j == 0) s_pick[0] = -1;
+    __syncthreads();
+    unsigned long long before = 0ull;
+    for (int i = 0; i < wave; ++i) before += s_wave[i];
+    const unsigned long long excl = before + incl - mine;
+    if (mine > 0ull && excl <= target && target < excl + mine) {
+        unsigned long long cum = excl;
+        for (int i = r_begin; i < r_end; ++i) {
+            cum += fixed_of(weight_of(row[begin + i], mx, inv_t));
+            if (cum > target) {
+                s_pick[0] = begin + i;
+                break;
+            }
+        }
+    }
+    __syncthreads();
+    return s_pick[0];
+}
+
 // One workgroup per row.  `weights` is scratch [rows][vocab] float32: the weights are computed once and the
 // selection passes read them back (from cache).  With a list of candidates (cand_idx != null) `weights` holds the
 // candidates' weights, cand_count[r * cand_stride] their number, and `best` the row's argmax.
@@ -559,7 +639,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
     const float* __restrict__ top_p, const float* __restrict__ uniform, int32_t* __restrict__ out,
     float* __restrict__ weights, int vocab, const int32_t* __restrict__ cand_idx, const int32_t* __restrict__ cand_count,
-    int cand_stride, const int32_t* __restrict__ best_in, const unsigned long long* __restrict__ row_mass) {
+    int cand_stride, const int32_t* __restrict__ best_in, const unsigned long long* __restrict__ row_mass,
+    const int32_t* __restrict__ direct_piece, const unsigned long long* __restrict__ direct_target) {
     __shared__ float s_val[16];
     __shared__ int s_idx[16];
     __shared__ unsigned int hist[256];
@@ -584,6 +665,13 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
         return;
     }
     const int full_vocab = vocab;
+    if (cand_idx && direct_piece[r] >= 0) {          // no cuts: the drawn point's piece is known, walk it
+        const int piece = (vocab + kSamplePieces - 1) / kSamplePieces;
+        const int begin = min(vocab, direct_piece[r] * piece), n = min(vocab, begin + piece) - begin;
+        const int at = pick_in_piece(row, begin, n, row[best], 1.0f / fmaxf(temp, 1e-6f), direct_target[r], s_wave, s_pick);
+        if (threadIdx.x == 0) out[r] = at < 0 ? best : at;
+        return;
+    }
     if (cand_idx) {
         vocab = cand_count[r * cand_stride];         // from here on the row is the list of candidates
     } else {
@@ -716,7 +804,7 @@ extern "C" int egpt_sample(const float* logits, const float* temperature, const 
         return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
     sample_kernel<<<n_rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(
-        logits, temperature, top_k, top_p, uniform, out, weights, vocab, nullptr, nullptr, 0, nullptr, nullptr);
+        logits, temperature, top_k, top_p, uniform, out, weights, vocab, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -731,7 +819,7 @@ extern "C" size_t egpt_sample_workspace(int n_rows, int vocab) {
            + align256(r * kSamplePieces * (kTopBins + 1) * 8)            // masses
            + align256(r * kSamplePieces * (kTopBins + 1) * 4)            // counts
            + align256(r * (kSamplePieces + 1) * 4) + align256(r * 4) * 2   // offsets, cutoff, best
-           + align256(r * 8)                                               // mass of the row
+           + align256(r * 8) * 2 + align256(r * 4)                         // mass of the row; the direct draw's point, piece
            + align256(r * kArgmaxPieces * 8);                              // argmax pieces
 }
 
@@ -752,6 +840,8 @@ extern "C" int egpt_sample_wide(const float* logits, const float* temperature, c
     uint32_t* cutoff = reinterpret_cast<uint32_t*>(p);                         p += align256(r * 4);
     int32_t* best = reinterpret_cast<int32_t*>(p);                             p += align256(r * 4);
     unsigned long long* row_mass = reinterpret_cast<unsigned long long*>(p);   p += align256(r * 8);
+    unsigned long long* direct_target = reinterpret_cast<unsigned long long*>(p); p += align256(r * 8);
+    int32_t* direct_piece = reinterpret_cast<int32_t*>(p);                     p += align256(r * 4);
     float* pv = reinterpret_cast<float*>(p);
     int32_t* pi = reinterpret_cast<int32_t*>(pv + r * kArgmaxPieces);
     argmax_pieces_kernel<<<dim3(n_rows, kArgmaxPieces), 256, 0, s>>>(logits, pv, pi, vocab);
@@ -761,13 +851,14 @@ extern "C" int egpt_sample_wide(const float* logits, const float* temperature, c
     sample_hist_kernel<<<dim3(n_rows, kSamplePieces), 256, 0, s>>>(logits, temperature, best, piece_count, piece_mass, vocab);
     EGPT_CHECK_LAUNCH();
     sample_plan_kernel<<<n_rows, 64, 0, s>>>(temperature, top_k, top_p, piece_count, piece_mass, cutoff, offsets, row_mass,
-                                             vocab);
+                                             uniform, direct_piece, direct_target, vocab);
     EGPT_CHECK_LAUNCH();
     sample_compact_kernel<<<dim3(n_rows, kSamplePieces), 256, 0, s>>>(logits, temperature, best, cutoff, offsets, cand_w,
-                                                                      cand_idx, vocab);
+                                                                      cand_idx, direct_piece, vocab);
     EGPT_CHECK_LAUNCH();
     sample_kernel<<<n_rows, kSampleThreads, 0, s>>>(logits, temperature, top_k, top_p, uniform, out, cand_w, vocab, cand_idx,
-                                                    offsets + kSamplePieces, kSamplePieces + 1, best, row_mass);
+                                                    offsets + kSamplePieces, kSamplePieces + 1, best, row_mass,
+                                                    direct_piece, direct_target);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
