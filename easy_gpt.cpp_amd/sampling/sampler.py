@@ -70,11 +70,11 @@ class Sampler:
         if all(p.greedy for p in params):
             k.argmax(logits, out)
         else:
+            # one row per option, so that each is a contiguous view of one upload
             host = torch.tensor(
-                [[0.0 if p.greedy else p.temperature, p.top_p, uniform_for(p.seed, s, n)]
-                 for p, s, n in zip(params, serials, counts)], dtype=torch.float32)
+                [[0.0 if p.greedy else p.temperature for p in params], [p.top_p for p in params],
+                 [uniform_for(p.seed, s, n) for p, s, n in zip(params, serials, counts)]], dtype=torch.float32)
             topk = torch.tensor([p.top_k for p in params], dtype=torch.int32)
             host = host.to(logits.device)
-            k.sample(logits, host[:, 0].contiguous(), topk.to(logits.device), host[:, 1].contiguous(),
-                     host[:, 2].contiguous(), out)
+            k.sample(logits, host[0], topk.to(logits.device), host[1], host[2], out)
         return out.tolist()
