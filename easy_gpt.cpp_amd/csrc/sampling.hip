@@ -305,7 +305,10 @@ __device__ uint32_t select_by_mass(const float* __restrict__ w, int vocab, uint3
 // number of rows.  For a wide vocabulary three small kernels with kSamplePieces workgroups per row come first: they
 // count the weights by exponent (those within 2^-16 of the largest, which hold the top-k tokens and the top-p mass of
 // any distribution that is not nearly flat), decide below which exponent no token can be kept, and write the tokens at
-// or above it, in index order, into a list of candidates.  The selection then runs on that list, unchanged.
+// or above it, in index order, into a list of candidates.  The selection then runs on that list: one thread per
+// candidate when they are at most kSampleThreads (the usual case), the row-walking selection otherwise.  A row for
+// which neither cut is asked gets no list: the pieces' masses say in which piece the drawn point lies, and that
+// piece alone is walked.
 constexpr int kSamplePieces = 32;
 constexpr int kTopBins = 16;            // exponents 127 (weight 1.0) down to 112, one bin each; bin kTopBins: the rest
 
