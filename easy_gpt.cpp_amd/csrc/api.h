@@ -62,12 +62,13 @@ int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, 
                                const int32_t* block_table, int table_width, const int32_t* q_start,
                                const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
                                int hd, int page_size, float scale, int window, int shape, void* stream);
-// One decoded token per request: workgroups of n_waves wavefronts per (request, kv head, key split).
+// One decoded token per request: workgroups of n_waves wavefronts per (request, kv head, key split); lean != 0: the
+// variant with half the loads in flight per round and fewer registers.
 int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                                 const void* v_cache, const int32_t* block_table, int table_width,
                                 const int32_t* q_start, const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd,
                                 int page_size, float scale, int window, int n_splits, int n_waves, int combine,
-                                void* stream);
+                                int lean, void* stream);
 // The same with the QKV epilogue (partial sums, 1/rms, bias, rotation, store of the new key and value) folded in;
 // token t belongs to request t; rotation over the whole head.
 int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const float* row_ss, int ss_splits, int hidden,
@@ -75,7 +76,7 @@ int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const floa
                                 float* part_o, float* part_ml, void* k_cache,
                                 void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                                 const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
-                                int window, int n_splits, int n_waves, int combine, void* stream);
+                                int window, int n_splits, int n_waves, int combine, int lean, void* stream);
 int egpt_attention_combine(const float* part_o, const float* part_ml, void* out, int n_rows, int hd, int n_splits,
                            void* stream);
 // Products for m <= 16 rows whose x operand is computed while it is staged (see gemm_skinny.hip).

@@ -951,10 +951,9 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
 static int dispatch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                            const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                            const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
-                           int window, int n_splits, int n_waves, int combine, const FusedQkv* fused, hipStream_t s) {
-    // more workgroups than one and a half per CU: the variant with half the loads in flight and fewer registers
-    // (measured at head size 64: 1.65 against 1.68 ms a step with 480 workgroups, the same with 256)
-    const bool lean = static_cast<long>(n_seqs) * nkv * n_splits > 384;
+                           int window, int n_splits, int n_waves, int combine, bool lean, const FusedQkv* fused,
+                           hipStream_t s) {
+    // lean: the variant with half the loads in flight and fewer registers (the caller's choice, see the wrapper)
 #define EGPT_LAUNCH_DECODE(HD_, PF_)                                                                             \
     launch_decode<HD_, PF_>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len, \
                             n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, fused, s)
@@ -1030,7 +1029,7 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
                                            const void* k_cache, const void* v_cache, const int32_t* block_table,
                                            int table_width, const int32_t* q_start, const int32_t* kv_len, int n_seqs,
                                            int nq, int nkv, int hd, int page_size, float scale, int window,
-                                           int n_splits, int n_waves, int combine, void* stream) {
+                                           int n_splits, int n_waves, int combine, int lean, void* stream) {
     if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !kv_len) return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0 || n_splits < 1 ||
         (n_splits > 1 && (!part_o || !part_ml)))
@@ -1040,7 +1039,7 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
         return EGPT_UNSUPPORTED_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_decode(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, nullptr, s);
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, nullptr, s);
 }
 
 // The same with the QKV epilogue folded in: the queries, and the new token's key and value, are computed from
@@ -1054,7 +1053,7 @@ extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits,
                                            float* part_ml, void* k_cache, void* v_cache, const int32_t* block_table,
                                            int table_width, const int32_t* q_start, const int32_t* kv_len, int n_seqs,
                                            int nq, int nkv, int hd, int page_size, float scale, int window,
-                                           int n_splits, int n_waves, int combine, void* stream) {
+                                           int n_splits, int n_waves, int combine, int lean, void* stream) {
     if (!qkv_prod || in_splits < 1 || !cos_sin || !slots || !out || !k_cache || !v_cache ||
         !block_table || !q_start || !kv_len || (row_ss && (ss_splits < 1 || hidden < 1)))
         return EGPT_BAD_ARGUMENT;
@@ -1074,7 +1073,7 @@ extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits,
     f.k_cache_w = static_cast<bf16_t*>(k_cache); f.v_cache_w = static_cast<bf16_t*>(v_cache);
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_decode(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, &f, s);
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, &f, s);
 }
 
 // bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.

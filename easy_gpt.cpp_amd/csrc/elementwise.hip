@@ -572,4 +572,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 9; }
+extern "C" int egpt_abi_version(void) { return 10; }

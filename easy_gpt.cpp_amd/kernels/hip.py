@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 9:
+    if lib.egpt_abi_version() != 10:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -85,9 +85,9 @@ class HipKernels:
             "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
             "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
-            "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, vp],
+            "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, i, vp],
             "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
-                                            i, i, f, i, i, i, i, vp],
+                                            i, i, f, i, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_f32": [vp, vp, vp, vp, i, i, i, i, vp],
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
@@ -526,7 +526,7 @@ class HipKernels:
             # the GPU, which is the case when only decoded tokens are in the batch
             if max_q_len == 1 and t == b and nq // nkv <= 16:
                 # only decoded tokens: workgroups of several wavefronts per (request, kv head, key split)
-                n_splits, n_waves = self._decode_shape(b, nkv, hd, max_kv_len, combine)
+                n_splits, n_waves, lean = self._decode_shape(b, nkv, hd, max_kv_len, combine)
                 part_o = part_ml = None
                 if n_splits > 1:
                     part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=qkv.device)
@@ -534,7 +534,7 @@ class HipKernels:
                 self._run("egpt_paged_attention_decode", qkv.data_ptr(), out.data_ptr(), self._ptr(part_o),
                           self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
                           q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale), int(window),
-                          n_splits, n_waves, 1 if combine else 0, self._stream())
+                          n_splits, n_waves, 1 if combine else 0, lean, self._stream())
                 return (part_o, part_ml) if (n_splits > 1 and not combine) else None
             if max_q_len > 1 and page_size & (page_size - 1) == 0:
                 # prompt portions (and mixed batches): key/value tiles shared through LDS by the wavefronts of
@@ -569,7 +569,7 @@ class HipKernels:
 
     @staticmethod
     def _decode_shape(b, nkv, hd, max_kv_len, combine):
-        """(key splits, wavefronts per workgroup) of the decode attention kernel.  The kernel is a chain of round
+        """(key splits, wavefronts per workgroup, lean variant or not) of the decode attention kernel.  The kernel is a chain of round
         trips to memory, and a wavefront takes one per round of 4 (head size 64) or 2 key blocks of 32 keys, so
         there should be enough wavefronts for one round each, and with few requests for one key block each.
         The key range is split over workgroups when the requests alone do not fill the GPU; parts that the
@@ -589,14 +589,24 @@ class HipKernels:
             room = 2048 if hd == 64 else 512
             return max(1, min(wanted, most, max(1, room // pairs)))
 
+        n_splits = n_waves = 0
         if hd == 64 and pairs * key_blocks <= 8192:
-            n_splits = splits_for(8)
+            n_splits, n_waves = splits_for(8), 8
             # wide workgroups as long as each has a CU of its own: a few more than CUs, and those that share one set
             # the kernel's time (measured at 2,048-token contexts: 1.84 ms a step at batch 44 and 48 with 264 and 288
             # workgroups of eight wavefronts, 1.66 with 440 and 480 of four; 1.57 either way at batch 40)
-            if pairs * n_splits <= 256:
-                return n_splits, 8
-        return splits_for(4), 4
+            if pairs * n_splits > 256:
+                n_waves = 0
+        if not n_waves:
+            n_splits, n_waves = splits_for(4), 4
+        # The kernel's variant with half the loads in flight per round and fewer registers.  Head size 64: always,
+        # unless a wavefront walks so many key blocks that the rounds' depth counts (measured: 0.954 -> 0.933 ms a step
+        # at batch 8 and 2,048-token contexts, 0.872 -> 0.853 at batch 1, 1.135 -> 1.102 at batch 8 and 8,192 tokens,
+        # but 1.99 -> 2.03 at batch 8 and 32,000 tokens, 31 blocks per wavefront).  Head size 128: from one and a
+        # half workgroups per CU on (fewer: 1 to 2% slower than the full variant).
+        per_wave = -(-key_blocks // (n_splits * n_waves))
+        lean = per_wave <= 16 if hd == 64 else pairs * n_splits > 384
+        return n_splits, n_waves, 1 if lean else 0
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
                                k_cache, v_cache, block_table, q_start, kv_len, nq, nkv, hd, page_size, scale, window,
@@ -631,7 +641,7 @@ class HipKernels:
             self._need(row_ss, "row_ss", _F32, (ss_splits, t))
         if max_kv_len > table_width * page_size:
             raise ValueError(f"block table of width {table_width} cannot hold {max_kv_len} tokens at page size {page_size}")
-        n_splits, n_waves = self._decode_shape(b, nkv, hd, max_kv_len, combine)
+        n_splits, n_waves, lean = self._decode_shape(b, nkv, hd, max_kv_len, combine)
         part_o = part_ml = None
         if n_splits > 1:
             part_o = torch.empty((n_splits, t, nq, hd), dtype=_F32, device=prod.device)
@@ -640,7 +650,7 @@ class HipKernels:
                   float(eps), self._ptr(bias), cos_sin.data_ptr(), slots.data_ptr(), out.data_ptr(),
                   self._ptr(part_o), self._ptr(part_ml), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
                   table_width, q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale),
-                  int(window), n_splits, n_waves, 1 if combine else 0, self._stream())
+                  int(window), n_splits, n_waves, 1 if combine else 0, lean, self._stream())
         return (part_o, part_ml) if (n_splits > 1 and not combine) else None
 
     def swiglu(self, gate_up, out, row_ss=None, hidden=0, eps=0.0):
