@@ -577,8 +577,8 @@ class HipKernels:
         key_blocks = -(-max_kv_len // 32)
         pairs = b * nkv
 
-        def splits_for(n_waves):
-            per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (4 if hd == 64 else 2))
+        def splits_for(n_waves, blocks=None):
+            per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (blocks or (4 if hd == 64 else 2)))
             wanted = -(-key_blocks // per_round)
             # the output projection combines up to 8 parts in registers; more only for few requests with contexts
             # so long that 8 parts would leave every wavefront four rounds or more
@@ -591,7 +591,11 @@ class HipKernels:
 
         n_splits = n_waves = 0
         if hd == 64 and pairs * key_blocks <= 8192:
-            n_splits, n_waves = splits_for(8), 8
+            # a round of the variant that runs here is two key blocks; with few pairs, enough splits for one round
+            # per wavefront (measured at 2,048-token contexts: 1.17 -> 1.13 ms a step at batch 16, 1.36 -> 1.33 at 24)
+            n_splits, n_waves = splits_for(8, blocks=2), 8
+            if pairs * n_splits > 256:
+                n_splits = splits_for(8)
             # wide workgroups as long as each has a CU of its own: a few more than CUs, and those that share one set
             # the kernel's time (measured at 2,048-token contexts: 1.84 ms a step at batch 44 and 48 with 264 and 288
             # workgroups of eight wavefronts, 1.66 with 440 and 480 of four; 1.57 either way at batch 40)
