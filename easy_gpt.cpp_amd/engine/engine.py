@@ -82,7 +82,12 @@ class Engine:
         if tune_products and self.device.type == "cuda":
             from .. import kernels
 
-            kernels.tune_library_products(True)
+            try:
+                kernels.tune_library_products(True)
+            except Exception as e:       # the products then stay the library's first choice, which is always right
+                import warnings
+
+                warnings.warn(f"the library's products cannot be chosen by measurement here: {e}")
         self.page_size = int(page_size)
         if num_pages is None:
             if max_tokens is None:
