@@ -5,9 +5,12 @@ left-over keys afterwards (/root/reference/src/models/model_param_validation.cpp
 fixtures in /root/reference/test/model_param_validation_test.cpp:345-426).  Here one
 error lists every missing tensor, every unexpected tensor and every wrong shape.
 
-Stored dtypes: BF16 stays bfloat16, F16 becomes bfloat16, F32 stays float32 (F64
-becomes float32), integer tables become int32.  Parts cast 'compute' parameters to
-the engine's dtype when they take them.
+Stored dtypes: BF16 stays bfloat16, F32 stays float32, F16 and F64 become float32
+(every float16 value is a float32 value, so nothing is lost), integer tables become
+int32.  Parts cast 'compute' parameters to the engine's dtype when they take them:
+that is the only rounding between the file and the device, as in the reference,
+which decodes each element through float32 into the build's dtype
+(/root/reference/src/models/loader.cpp:173-198).
 """
 from __future__ import annotations
 
@@ -68,7 +71,7 @@ def check_names_and_shapes(
 
 _STORED_AS = {
     torch.bfloat16: torch.bfloat16,
-    torch.float16: torch.bfloat16,
+    torch.float16: torch.float32,
     torch.float32: torch.float32,
     torch.float64: torch.float32,
     torch.int32: torch.int32,

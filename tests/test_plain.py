@@ -65,6 +65,23 @@ def test_rope_offsets_of_the_reference():
                     assert abs(float(out[s, h, k + 2]) - (x1 * math.sin(ang) + x2 * math.cos(ang))) < 1e-6
 
 
+def test_rope_is_a_complex_multiplication():
+    # The pair (x_k, x_{k+hd/2}) read as the complex number x_k + i x_{k+hd/2} is multiplied by exp(i pos inv_freq_k):
+    # the library's complex product stands in for the two lines of /root/reference/src/ops.cpp:416-417.  A wrong
+    # sign, a swapped sine and cosine or interleaved pairs fail this.
+    g = torch.Generator().manual_seed(11)
+    for hd, theta in ((8, 10000.0), (6, 1e6)):
+        x = torch.randn(7, 3, hd, generator=g, dtype=F64)
+        pos = torch.tensor([0, 1, 2, 5, 40, 41, 1000])
+        half = hd // 2
+        inv = torch.tensor([theta ** (-2.0 * k / hd) for k in range(half)], dtype=F64)
+        z = torch.complex(x[..., :half], x[..., half:]) * torch.polar(torch.ones(7, half, dtype=F64), pos[:, None].double() * inv)[:, None, :]
+        ref = torch.cat([z.real, z.imag], dim=-1)
+        # the plain implementation makes its angles in float32 as the reference does: 1e-7 relative on an angle of 1000
+        assert torch.allclose(plain.rope(x, pos, theta), ref, atol=2e-4)
+        assert torch.allclose(plain.rope(x[:4], pos[:4], theta), ref[:4], atol=1e-6)
+
+
 def test_rope_invariants():
     g = torch.Generator().manual_seed(1)
     q = torch.randn(6, 2, 8, generator=g, dtype=F64)
@@ -168,11 +185,25 @@ def test_whole_model_invariants(tiny_models):
         shifted = plain.forward_logits(cfg, w, ids, first_position=3)
         assert torch.allclose(shifted, logits, atol=5e-5)
         # tied or not decides which matrix makes the logits
-        head = "model.embed_tokens.weight" if cfg["tie_word_embeddings"] else "lm_head.weight"
-        w2 = dict(w)
-        w2[head] = w[head] * 2
-        assert torch.allclose(plain.forward_logits(cfg, w2, ids)[-1] if head == "lm_head.weight" else logits[-1] * 0 + 1,
-                              logits[-1] * 2 if head == "lm_head.weight" else logits[-1] * 0 + 1, atol=1e-9)
+        if cfg["tie_word_embeddings"]:
+            # a stray output matrix in the file is not used, and the logits are those of an untied model whose
+            # output matrix is a copy of the embedding table
+            stray = dict(w, **{"lm_head.weight": torch.ones_like(w["model.embed_tokens.weight"])})
+            assert torch.equal(plain.forward_logits(cfg, stray, ids), logits)
+            untied = dict(w, **{"lm_head.weight": w["model.embed_tokens.weight"].clone()})
+            assert torch.equal(plain.forward_logits(dict(cfg, tie_word_embeddings=False), untied, ids), logits)
+            # doubling the table doubles the logits (the norms undo the doubling of the residual stream up to eps)
+            doubled = dict(w, **{"model.embed_tokens.weight": w["model.embed_tokens.weight"] * 2})
+            assert not torch.allclose(plain.forward_logits(cfg, doubled, ids), logits, atol=1e-3)
+        else:
+            doubled = dict(w, **{"lm_head.weight": w["lm_head.weight"] * 2})
+            assert torch.allclose(plain.forward_logits(cfg, doubled, ids), logits * 2, atol=1e-9)
+            # the embedding table is not the output matrix: changing only the rows of tokens that are not in the
+            # sequence changes nothing
+            absent = [t for t in range(cfg["vocab_size"]) if t not in set(ids)]
+            other = w["model.embed_tokens.weight"].clone()
+            other[absent] += 1.0
+            assert torch.equal(plain.forward_logits(cfg, dict(w, **{"model.embed_tokens.weight": other}), ids), logits)
 
 
 def test_window_matters_in_config_c(tiny_models):

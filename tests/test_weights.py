@@ -54,7 +54,7 @@ def test_roundtrip_and_dtypes(tmp_path):
 
 
 def test_stored_dtype_rules(tmp_path):
-    # bfloat16 stays, float16 becomes bfloat16, float32 stays, int64 becomes int32
+    # bfloat16 stays, float16 becomes float32 (exactly), float32 stays, int64 becomes int32
     from easy_gpt.cpp_amd.parts import ParamSpec
 
     t = {"w": torch.randn(3, 5).to(torch.bfloat16), "h": torch.randn(2).to(torch.float16), "f": torch.randn(2),
@@ -63,10 +63,52 @@ def test_stored_dtype_rules(tmp_path):
     specs = [ParamSpec("w", (3, 5)), ParamSpec("h", (2,)), ParamSpec("f", (2,)), ParamSpec("i", (5,), "int_table", "int32")]
     cw = CheckedWeights(str(tmp_path), specs)
     assert cw.get("w").dtype == torch.bfloat16 and torch.equal(cw.get("w"), t["w"])
-    assert cw.get("h").dtype == torch.bfloat16
+    assert cw.get("h").dtype == torch.float32 and torch.equal(cw.get("h"), t["h"].float())
     assert cw.get("f").dtype == torch.float32 and torch.equal(cw.get("f"), t["f"])
     assert cw.get("i").dtype == torch.int32 and cw.get("i").tolist() == [0, 1, 2, 3, 4]
     cw.close()
+
+
+def test_float16_checkpoint_is_rounded_once_on_the_way_to_the_engine(tmp_path):
+    # The reference decodes every stored element through float32 into the build's dtype
+    # (/root/reference/src/models/loader.cpp:173-198): a float32 engine holds the stored float16 values exactly,
+    # a bfloat16 engine rounds them once.
+    from easy_gpt.cpp_amd.parts import ParamSpec
+    from easy_gpt.cpp_amd.parts.base import Part
+
+    g = torch.Generator().manual_seed(3)
+    h = (torch.randn(64, 7, generator=g) * 0.02).to(torch.float16)
+    assert not torch.equal(h.to(torch.bfloat16).float(), h.float())      # these values do not fit bfloat16
+    write_safetensors(str(tmp_path / "model.safetensors"), {"h": h})
+    cw = CheckedWeights(str(tmp_path), [ParamSpec("h", (64, 7))])
+    got = cw.get("h")
+    cw.close()
+    assert torch.equal(Part._to(got, "compute", torch.float32, "cpu"), h.float())
+    assert torch.equal(Part._to(got, "compute", torch.bfloat16, "cpu"), h.float().to(torch.bfloat16))
+
+
+def test_file_format_agrees_with_the_safetensors_library(tmp_path):
+    # The format is pinned by something other than this repository's own writer: a file the library writes is
+    # read the same by SafetensorsFile, and a file write_safetensors writes is read the same by the library.
+    st = pytest.importorskip("safetensors.torch")
+    g = torch.Generator().manual_seed(4)
+    t = {
+        "model.a": torch.randn(3, 5, generator=g), "b": torch.randn(17, generator=g).to(torch.bfloat16),
+        "c.h": torch.randn(2, 2, 3, generator=g).to(torch.float16), "i": torch.arange(6, dtype=torch.int64).reshape(2, 3),
+        "j": torch.arange(4, dtype=torch.int32),
+    }
+    theirs, ours = str(tmp_path / "theirs.safetensors"), str(tmp_path / "ours.safetensors")
+    st.save_file(t, theirs, metadata={"format": "pt"})
+    with SafetensorsFile(theirs) as f:
+        assert set(f.names()) == set(t)
+        for k, v in t.items():
+            got = f.read(k)
+            assert got.dtype == v.dtype and got.shape == v.shape and torch.equal(got, v), k
+    write_safetensors(ours, t, metadata={"format": "pt", "seed": "4"})
+    back = st.load_file(ours)
+    assert set(back) == set(t)
+    for k, v in t.items():
+        assert back[k].dtype == v.dtype and torch.equal(back[k], v), k
 
 
 def test_complete_set_validates(tmp_path):
