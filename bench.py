@@ -22,7 +22,7 @@ sys.path.insert(0, ROOT)
 HBM_GBPS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# Qwen2.5-0.5B layer sizes (the third configuration of the baseline record)
+# Qwen2.5-0.5B layer sizes: the shape that the headline numbers are quoted on
 QWEN25_05B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 24, "hidden_size": 896,
     "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
@@ -35,7 +35,7 @@ NEW_TOKENS = 128
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 
-# The other layer sizes of the baseline record, for --shape (the default run and its record stay the 0.5B ones):
+# The larger Qwen2.5 layer sizes, for --shape (the default run and its record stay the 0.5B ones):
 # (config changes, layers of the model, prefix length of the decode runs)
 OTHER_SHAPES = {
     "1.5b": (dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
@@ -92,6 +92,46 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
     return 0
 
 
+def link_floor() -> int:
+    """What a chain of dependent kernels costs apart from its work: graphs of 125 links that each do next to nothing
+    (every thread one load of what the link before wrote, `trips - 1` further loads that depend on each other, one
+    store), replayed; microseconds per link by number of workgroups and of dependent round trips to memory."""
+    import torch
+
+    from easy_gpt.cpp_amd import kernels
+
+    k = kernels.backend()
+    links, table = 125, {}
+    for groups in (1, 64, 256, 1024, 4096):
+        n = groups * 256
+        a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+        for trips in (1, 2, 3, 5):
+            def chain():
+                src, dst = a, b
+                for _ in range(links):
+                    k.probe_link(src, dst, trips)
+                    src, dst = dst, src
+            chain()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                chain()
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            reps = 20
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                graph.replay()
+            torch.cuda.synchronize()
+            table[f"wg{groups}_trips{trips}"] = round((time.perf_counter() - t0) / reps / links * 1e6, 3)
+            print(f"[bench] {groups:5d} workgroups, {trips} dependent loads: {table[f'wg{groups}_trips{trips}']:.2f} us a link",
+                  file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "microseconds per link of a replayed graph of 125 dependent near-empty kernels",
+                      "unit": "us", "links": links, "table": table}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,10 +139,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--shape", default="0.5b", choices=["0.5b"] + sorted(OTHER_SHAPES),
-                    help="layer sizes: Qwen2.5-0.5B (the record's) or another size of the baseline record")
+                    help="layer sizes: Qwen2.5-0.5B (the default, which the headline numbers are quoted on), 1.5B or 7B")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prefix", type=int, default=None,
-                    help="tokens each request holds before decoding starts (default: the record's 2,048)")
+                    help="tokens each request holds before decoding starts (default: 2,048; 4,096 at the 7B sizes)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-tune", action="store_true",
@@ -112,8 +152,12 @@ def main() -> int:
     ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
     ap.add_argument("--serve", action="store_true",
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
-                         "each through the scheduler, prompts in portions of 512 (a workload of the baseline record)")
+                         "each through the scheduler, prompts in portions of 512 (the mixed serving workload)")
+    ap.add_argument("--link-floor", action="store_true",
+                    help="instead of the model: what a link of a chain of dependent, near-empty kernels costs in a graph")
     args = ap.parse_args()
+    if args.link_floor:
+        return link_floor()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
         return 2
@@ -155,7 +199,7 @@ def main() -> int:
     t_setup = time.time()
     tmp = tempfile.mkdtemp(prefix="egpt_bench_")
     write_random_model(tmp, cfg, seed=0, dtype=torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
-    new_tokens = max(NEW_TOKENS, args.warmup + args.steps)        # a longer run than the record's decodes further
+    new_tokens = max(NEW_TOKENS, args.warmup + args.steps)        # a longer run than the default decodes further
     tokens_per_request = -(-(PREFIX + new_tokens) // page_size) * page_size
     if args.serve:
         max_batch, tokens_per_request = SERVE_REQUESTS, -(-(2048 + SERVE_NEW_TOKENS) // page_size) * page_size

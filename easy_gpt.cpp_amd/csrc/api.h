@@ -102,6 +102,10 @@ size_t egpt_sample_workspace(int n_rows, int vocab);
 int egpt_sample_wide(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                      const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab, void* stream);
 
+// Measurement only: one link of a chain of dependent kernels that does next to nothing (see elementwise.hip);
+// in, out float32 [n] (in all zeros), `trips` dependent loads per thread.
+int egpt_probe_link(const float* in, float* out, int n, int trips, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -97,6 +97,7 @@ class HipKernels:
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
+            "egpt_probe_link": [vp, vp, i, i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -672,6 +673,13 @@ class HipKernels:
             self._need(row_ss, "row_ss", _F32, (ss_splits, t))
         self._run("egpt_swiglu", gate_up.data_ptr(), splits, self._ptr(row_ss), ss_splits, int(hidden), float(eps),
                   out.data_ptr(), t, inter, dt, self._stream())
+
+    def probe_link(self, src, dst, trips=1):
+        """Measurement only: dst = src through a kernel that does next to nothing but `trips` dependent loads."""
+        n = src.shape[0]
+        self._need(src, "src", _F32, (n,))
+        self._need(dst, "dst", _F32, (n,))
+        self._run("egpt_probe_link", src.data_ptr(), dst.data_ptr(), n, int(trips), self._stream())
 
     def argmax(self, logits, out):
         r, v = logits.shape

@@ -43,12 +43,17 @@ def read_safetensors(path: str) -> dict[str, torch.Tensor]:
     return out
 
 
-def read_model(model_dir: str, round_to_bf16: bool = False):
+def read_model(model_dir: str, round_to_bf16: bool = False, device: str = "cpu"):
+    """(config.json as a dict, {tensor name: float64 tensor}).  `device`: where the tensors are kept and the
+    model is computed; the functions below are the same torch code on any device (large shapes take minutes on
+    the CPU)."""
     with open(os.path.join(model_dir, "config.json")) as f:
         cfg = json.load(f)
     w = read_safetensors(os.path.join(model_dir, "model.safetensors"))
     if round_to_bf16:
         w = {k: v.to(torch.float32).to(torch.bfloat16).to(F64) for k, v in w.items()}
+    if device != "cpu":
+        w = {k: v.to(device) for k, v in w.items()}
     return cfg, w
 
 
@@ -79,8 +84,8 @@ def rope(x, positions, theta):
     x1' = x1 cos - x2 sin, x2' = x1 sin + x2 cos (/root/reference/src/ops.cpp:404-420)."""
     hd = x.shape[-1]
     half = hd // 2
-    inv = rope_inv_freq(hd, theta)
-    ang = (positions.to(torch.float32)[:, None] * inv[None, :]).to(F64)   # float32 product, as the reference
+    inv = rope_inv_freq(hd, theta).to(x.device)
+    ang = (positions.to(x.device, torch.float32)[:, None] * inv[None, :]).to(F64)   # float32 product, as the reference
     cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     x1, x2 = x[..., :half], x[..., half:]
     return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1)
@@ -104,7 +109,7 @@ def attention(q, k, v, n_heads, n_kv_heads, window=None):
     softmax over keys; out = sum p v (/root/reference/src/models/self_attn.cpp:247-255)."""
     s, _, hd = q.shape
     group = n_heads // n_kv_heads
-    ok = attention_scores_mask(s, window)
+    ok = attention_scores_mask(s, window).to(q.device)
     out = torch.empty_like(q)
     for h in range(n_heads):
         kh = h // group
@@ -145,15 +150,17 @@ def layer_window(cfg, layer):
     return None
 
 
-def forward_logits(cfg, w, token_ids, first_position=0):
+def forward_logits(cfg, w, token_ids, first_position=0, rows=None):
     """Logits [S, V] of one whole sequence: embedding gather, L pre-norm blocks
     (a = x + Attn(N1 x); y = a + MLP(N2 a), /root/reference/src/models/block.cpp:23-29), final norm,
     output projection with the embedding table when tied
     (/root/reference/src/models/gpt_model.cpp:310-333, /root/reference/src/models/embedding.cpp:54-81).
-    `first_position` shifts all positions (for the invariance test only)."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
+    `first_position` shifts all positions (for the invariance test only).  `rows`: only the logits at these
+    places, [len(rows), V] (the reference computes all of them and reads one)."""
+    table = w["model.embed_tokens.weight"]
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=table.device)
     eps = cfg.get("rms_norm_eps", 1e-6)
-    x = w["model.embed_tokens.weight"][ids]
+    x = table[ids]
     positions = torch.arange(len(ids)) + first_position
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
@@ -161,6 +168,8 @@ def forward_logits(cfg, w, token_ids, first_position=0):
         x = x + self_attention_block(xn, w, p + "self_attn.", cfg, positions, layer_window(cfg, i))
         xn = rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
         x = x + swiglu_mlp(xn, w, p + "mlp.")
+    if rows is not None:
+        x = x[torch.as_tensor(list(rows), dtype=torch.long, device=x.device)]
     xn = rms_norm(x, w["model.norm.weight"], eps)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return linear(xn, head)
