@@ -93,6 +93,19 @@ int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_split
 int egpt_gemm_gate_up_swiglu(const void* x, const void* w, void* out, int m, int inter, int k, int groups, void* stream);
 // scratch: n_rows * 32 floats followed by n_rows * 32 int32 (two-stage search for wide vocabularies), or null.
 int egpt_argmax(const float* logits, int32_t* out, void* scratch, int n_rows, int vocab, void* stream);
+// egpt_argmax for callers that cannot allocate device memory and have no workspace to pass (code under graph
+// capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The pieces
+// of the two-stage search live in a buffer inside the library's device image (256 KiB per GPU, held until the process
+// ends) instead of a workspace argument; the call allocates nothing and launches the same kernels as egpt_argmax.
+// At most EGPT_ARGMAX_STATIC_MAX_ROWS rows (more: EGPT_STATIC_SCRATCH_TOO_SMALL, nothing is launched).  The buffer needs
+// no clearing: every entry that the second stage reads is written by the first stage of the same call.  All calls on
+// one GPU share that GPU's buffer, so calls that overlap there (on different streams, or from different threads)
+// race; calls on one stream are ordered by the stream.  The stream must belong to the current device.
+// egpt_argmax_static_init resolves the buffer's address on the current device (once per device; the entry point
+// does it at its first call on a device otherwise): call it before a capture begins.
+#define EGPT_ARGMAX_STATIC_MAX_ROWS 1024
+int egpt_argmax_static_init(void);
+int egpt_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, void* stream);
 // weights: scratch for n_rows * vocab floats.
 int egpt_sample(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                 const float* uniform, int32_t* out, float* weights, int n_rows, int vocab, void* stream);

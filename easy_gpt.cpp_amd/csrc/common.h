@@ -84,6 +84,8 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 #define EGPT_BAD_ARGUMENT 1
 #define EGPT_UNSUPPORTED_SIZE 2
 #define EGPT_LAUNCH_FAILED 3
+#define EGPT_STATIC_SCRATCH_TOO_SMALL 4
+#define EGPT_STATIC_SCRATCH_UNRESOLVED 5
 
 #define EGPT_CHECK_LAUNCH()                                   \
     do {                                                      \

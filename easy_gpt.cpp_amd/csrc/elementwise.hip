@@ -594,8 +594,12 @@ extern "C" const char* egpt_error_string(int code) {
         case EGPT_BAD_ARGUMENT: return "bad argument (null pointer, negative size or unknown dtype)";
         case EGPT_UNSUPPORTED_SIZE: return "size not supported by this kernel";
         case EGPT_LAUNCH_FAILED: return "kernel launch failed";
+        case EGPT_STATIC_SCRATCH_TOO_SMALL:
+            return "more rows than the library's static scratch buffer holds (egpt_argmax_static takes at most 1024 rows)";
+        case EGPT_STATIC_SCRATCH_UNRESOLVED:
+            return "the device address of the library's static scratch buffer could not be resolved on the current device";
         default: return "unknown error";
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 10; }
+extern "C" int egpt_abi_version(void) { return 11; }

@@ -6,6 +6,8 @@
 // kept mass.  Here the kept set is found without sorting, by radix selection on the bit patterns of the
 // weights (four passes of eight bits over the row, which stays in cache; masses are added in fixed point so
 // that no decision depends on the order of additions), and the draw walks the kept weights in index order.
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -798,6 +800,43 @@ extern "C" int egpt_argmax(const float* logits, int32_t* out, void* scratch, int
     }
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
+}
+
+// ---- the same search without a workspace argument and without any allocation: the pieces live in the library's
+// device image.  In host code `argmax_static_scratch` is only a stand-in for the symbol: the memory's address on
+// a device comes from hipGetSymbolAddress with that device current, and every GPU has its own copy.
+static __device__ __align__(256) unsigned char argmax_static_scratch[EGPT_ARGMAX_STATIC_MAX_ROWS * kArgmaxPieces * 8];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+void* g_static_ptr[kMaxDevices] = {};
+
+// The buffer's address on the current device, resolved once per device; null on failure.
+void* static_scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(argmax_static_scratch)) != hipSuccess) return nullptr;
+        g_static_ptr[dev] = ptr;
+    }
+    return g_static_ptr[dev];
+}
+}  // namespace
+
+extern "C" int egpt_argmax_static_init(void) {
+    return static_scratch_of_current_device() ? EGPT_OK : EGPT_STATIC_SCRATCH_UNRESOLVED;
+}
+
+extern "C" int egpt_argmax_static(const float* logits, int32_t* out, int n_rows, int vocab, void* stream) {
+    if (!logits || !out || n_rows < 0 || vocab <= 0) return EGPT_BAD_ARGUMENT;
+    if (n_rows > EGPT_ARGMAX_STATIC_MAX_ROWS) return EGPT_STATIC_SCRATCH_TOO_SMALL;
+    if (n_rows == 0) return EGPT_OK;
+    void* scratch = static_scratch_of_current_device();
+    if (!scratch) return EGPT_STATIC_SCRATCH_UNRESOLVED;
+    return egpt_argmax(logits, out, scratch, n_rows, vocab, stream);
 }
 
 // weights: scratch for n_rows * vocab floats.

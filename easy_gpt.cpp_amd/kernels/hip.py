@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 10:
+    if lib.egpt_abi_version() != 11:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
