@@ -29,7 +29,10 @@ USAGE = """Usage: easy_llm [--model <dir>] [--prompt-file <path>] [--max-steps <
       --serve-idle-ms <n>    Accepted for compatibility; there is no stdin service to idle in (default: 2)
       --serve-stats-ms <n>   Stats log interval in milliseconds, 0 disables periodic logs (default: 1000)
       --model <dir>          Folder with config.json and model.safetensors (default: data/model)
+      --allow-unexpected-tensors  Only warn about tensors in the file that the model does not use, as the
+                             reference does; without it they are an error, listed with missing and misshapen ones
       --dtype <name>         bfloat16 or float32 (default: bfloat16)
+      --device <name>        torch device that holds the model (default: cuda:0; the kernels are for MI355X only)
       --random-weights <config.json>  Write a model folder with random weights from this config (to --model), then run
       --max-new-tokens <n>   Cap on new tokens per request instead of --max-steps
       --ignore-eos           Do not stop at the end token
@@ -65,6 +68,7 @@ class CliOptions:
     # beyond the reference
     model: str = "data/model"
     dtype: str = "bfloat16"
+    device: str = "cuda:0"
     random_weights: str = ""
     max_new_tokens: int = 0
     ignore_eos: bool = False
@@ -73,6 +77,7 @@ class CliOptions:
     cache_tokens: int = 65536
     page_size: int = 16
     tune_products: bool = False
+    allow_unexpected_tensors: bool = False
 
 
 class CliError(ValueError):
@@ -156,6 +161,8 @@ def parse_args(argv: list[str]) -> CliOptions:
             o.dtype = value(arg, "name")
             if o.dtype not in ("bfloat16", "float32", "bf16", "fp32"):
                 raise CliError(f"Unknown dtype: {o.dtype}")
+        elif arg == "--device":
+            o.device = value(arg, "name")
         elif arg == "--random-weights":
             o.random_weights = value(arg, "path")
         elif arg == "--max-new-tokens":
@@ -166,6 +173,8 @@ def parse_args(argv: list[str]) -> CliOptions:
             o.ignore_eos = True
         elif arg == "--tune-products":
             o.tune_products = True
+        elif arg == "--allow-unexpected-tensors":
+            o.allow_unexpected_tensors = True
         elif arg in ("--max-tokens-per-step", "--prefill-chunk", "--cache-tokens", "--page-size"):
             name = arg[2:].replace("-", "_")
             v = _number(int, value(arg), arg[2:].replace("-", " "))
@@ -240,9 +249,10 @@ def main(argv: list[str] | None = None) -> int:
 
     from .generate import LLM
 
-    llm = LLM(o.model, dtype=o.dtype, cache_tokens=o.cache_tokens, page_size=o.page_size,
+    llm = LLM(o.model, dtype=o.dtype, device=o.device, cache_tokens=o.cache_tokens, page_size=o.page_size,
               max_active=o.serve_max_active, max_admit_per_step=o.serve_prefill_batch,
-              max_tokens_per_step=o.max_tokens_per_step, prefill_chunk=o.prefill_chunk, tune_products=o.tune_products)
+              max_tokens_per_step=o.max_tokens_per_step, prefill_chunk=o.prefill_chunk, tune_products=o.tune_products,
+              allow_unexpected_tensors=o.allow_unexpected_tensors)
     last = [time.perf_counter()]
 
     def on_step(sched):
@@ -254,13 +264,17 @@ def main(argv: list[str] | None = None) -> int:
                   f"preemptions={s.preemptions}", file=sys.stderr, flush=True)
 
     t0 = time.perf_counter()
-    outputs = llm.generate(
+    requests = llm.generate_requests(
         prompts, max_new_tokens=o.max_new_tokens or 100, max_steps=None if o.max_new_tokens else o.max_steps,
         temperature=o.temperature, top_p=o.top_p, top_k=o.top_k, greedy=o.use_greedy, seed=o.seed,
         ignore_eos=o.ignore_eos, on_step=on_step,
     )
     dt = time.perf_counter() - t0
-    lines = [" ".join(str(t) for t in out) for out in outputs]
+    # a request that failed leaves an empty line (and its reason on stderr); the others keep their outputs
+    failed = [r for r in requests if r.status == "failed"]
+    for r in failed:
+        print(f"error: request {r.request_id} failed: {r.finish_reason}", file=sys.stderr)
+    lines = ["" if r.status == "failed" else " ".join(str(t) for t in r.output) for r in requests]
     if o.prompt_file:
         path = output_path_for(o.prompt_file)
         with open(path, "w", encoding="utf-8") as f:
@@ -270,7 +284,7 @@ def main(argv: list[str] | None = None) -> int:
         for ln in lines:
             print(ln)
     s = llm.last_stats
-    print(f"[summary] requests={len(outputs)} steps={s.steps} prompt_tokens={s.prompt_tokens} "
+    print(f"[summary] requests={len(requests)} failed={len(failed)} steps={s.steps} prompt_tokens={s.prompt_tokens} "
           f"generated={s.generated} preemptions={s.preemptions} seconds={dt:.3f} "
           f"tok_per_s={s.generated / dt if dt > 0 else 0:.1f}", file=sys.stderr)
-    return 0
+    return 1 if failed else 0

@@ -11,6 +11,7 @@ the true positions and nothing is padded.
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass, field
 from typing import Sequence
 
@@ -39,16 +40,18 @@ class StepEntry:
     want: Sequence[int] = field(default_factory=tuple)
 
 
-def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> Model:
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0", allow_unexpected_tensors: bool = False) -> Model:
     """Model folder -> model on the device: config.json picks the architecture, the weights
-    are checked by name and shape and then taken by the parts."""
+    are checked by name and shape and then taken by the parts.  A tensor that the model does not
+    declare is an error, listed with the missing and misshapen ones; allow_unexpected_tensors=True only
+    warns about it, as the reference does (/root/reference/src/models/model_param_validation.cpp:198-218)."""
     arch, cfg = load_model_config(model_dir)
     spec = arch.build_spec(cfg)
     model = build_model(spec)
-    weights = CheckedWeights(model_dir, model.param_specs(), spec.ignorable_tensors)
+    weights = CheckedWeights(model_dir, model.param_specs(), spec.ignorable_tensors, allow_unexpected_tensors)
     try:
         for name in weights.ignored:
-            print(f"[weights] tensor '{name}' is not used by this model and was ignored", flush=True)
+            print(f"[weights] tensor '{name}' is not used by this model and was ignored", file=sys.stderr, flush=True)
         torch_dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype
         model.load(weights.get, torch_dtype, torch.device(device))
     finally:
@@ -119,8 +122,9 @@ class Engine:
         self._has_windows = any(g.window is not None for g in groups)
 
     @classmethod
-    def from_dir(cls, model_dir: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
-        return cls(load_model(model_dir, dtype, device), **kw)
+    def from_dir(cls, model_dir: str, dtype="bfloat16", device="cuda:0", allow_unexpected_tensors: bool = False,
+                 **kw) -> "Engine":
+        return cls(load_model(model_dir, dtype, device, allow_unexpected_tensors), **kw)
 
     # ------------------------------------------------------------------ requests
     def add_request(self, request_id) -> RequestCache:

@@ -131,8 +131,14 @@ class Scheduler:
         total = min(len(r.prompt) + r.max_new_tokens, self.engine.max_position)
         # the last generated token is never stored, the one before it is
         need = self.cache.pages_for_tokens(max(len(r.prompt), total - 1))
-        return all(need <= pool.num_pages for pool, g in zip(self.cache.pools, self.cache.groups) if g.window is None) \
-            and all(pool.num_pages >= 1 for pool in self.cache.pools)
+        ps = self.cache.page_size
+        for pool, g in zip(self.cache.pools, self.cache.groups):
+            # a windowed group gives pages back as the window passes them: token by token it never holds more than
+            # the pages that a window can touch
+            most = need if g.window is None else min(need, -(-g.window // ps) + 1)
+            if most > pool.num_pages:
+                return False
+        return True
 
     def _fail(self, r: Request, reason: str) -> None:
         if r.status == "running":
@@ -244,9 +250,11 @@ class Scheduler:
                     self._fail(r, "the cache cannot hold this request even alone")
                     continue
                 count = min(r.pending(), cfg.prefill_chunk, budget)
-                first = self.cache.pages_for_tokens(count)
-                if any(first > pool.free_count - p for pool, p in zip(self.cache.pools, promised)):
-                    break
+                room = min((pool.free_count - p) * self.cache.page_size for pool, p in zip(self.cache.pools, promised))
+                if count > room:
+                    if self.running or room < 1:
+                        break           # it waits for pages that the running requests will give back
+                    count = room        # nobody runs, so nothing will be given back: its first portion is cut to the free pages
                 try:
                     self.engine.add_request(r.request_id)
                 except NoFreeSlot:

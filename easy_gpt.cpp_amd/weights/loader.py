@@ -39,15 +39,18 @@ def check_names_and_shapes(
     specs: Iterable[ParamSpec],
     ignorable: Iterable[str] = (),
     where: str = "weights",
+    allow_unexpected: bool = False,
 ) -> list[str]:
     """Compare the tensors on offer with the declared ones.  Raises one WeightsError that
-    lists all problems; returns the ignorable names that were present (to warn about)."""
+    lists all problems; returns the names that were present but are not used (to warn about): the
+    ignorable ones, and with allow_unexpected every other undeclared one, which the reference only
+    warns about too (/root/reference/src/models/model_param_validation.cpp:198-218)."""
     specs = list(specs)
     declared = {s.name: s for s in specs}
     missing = [s.name for s in specs if s.name not in available]
     ignorable = set(ignorable)
-    unexpected = [n for n in available if n not in declared and n not in ignorable]
-    ignored = [n for n in available if n not in declared and n in ignorable]
+    unexpected = [n for n in available if n not in declared and n not in ignorable and not allow_unexpected]
+    ignored = [n for n in available if n not in declared and (n in ignorable or allow_unexpected)]
     wrong = []
     for name, spec in declared.items():
         if name in available:
@@ -88,7 +91,8 @@ class CheckedWeights:
 
     INDEX = "model.safetensors.index.json"
 
-    def __init__(self, model_dir: str, specs: Iterable[ParamSpec], ignorable: Iterable[str] = ()):
+    def __init__(self, model_dir: str, specs: Iterable[ParamSpec], ignorable: Iterable[str] = (),
+                 allow_unexpected: bool = False):
         self.path = os.path.join(model_dir, "model.safetensors")
         self.files: list[SafetensorsFile] = []
         self._file_of: dict[str, SafetensorsFile] = {}
@@ -102,7 +106,8 @@ class CheckedWeights:
                 self.files.append(f)
                 self._file_of = {n: f for n in f.names()}
             available = {n: f.shape(n) for n, f in self._file_of.items()}
-            self.ignored = check_names_and_shapes(available, specs, ignorable, where=self.path)
+            self.ignored = check_names_and_shapes(available, specs, ignorable, where=self.path,
+                                                  allow_unexpected=allow_unexpected)
         except Exception:
             self.close()
             raise

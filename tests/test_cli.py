@@ -72,3 +72,86 @@ def test_main_errors_return_one(capsys):
     assert "No prompts provided" in capsys.readouterr().err
     assert main(["--help"]) == 0
     assert "Usage: easy_llm" in capsys.readouterr().out
+
+
+# ----------------------------------------------------------------------------- the body of main(), on the CPU
+@pytest.fixture()
+def emulated_backend():
+    from emulated_kernels import EmulatedKernels
+    from easy_gpt.cpp_amd import kernels
+
+    kernels.use_backend(EmulatedKernels())
+    yield
+    kernels.use_backend(None)
+
+
+def test_main_writes_random_weights_and_generates(tmp_path, capsys, emulated_backend):
+    # the whole command line with the tests' stand-in for the kernels: the model folder is written from a config and
+    # the seed, loaded, and the greedy tokens are the plain implementation's
+    import json
+
+    import plain_qwen2 as plain
+    from conftest import TINY_A
+
+    cfg_path, model = tmp_path / "cfg.json", tmp_path / "model"
+    cfg_path.write_text(json.dumps(TINY_A))
+    common = ["--model", str(model), "--dtype", "float32", "--device", "cpu", "--greedy", "--ignore-eos",
+              "--serve-stats-ms", "0", "--cache-tokens", "512"]
+    assert main(["--random-weights", str(cfg_path), "--seed", "3", "--max-new-tokens", "6", "5 17 3 99"] + common) == 0
+    out = capsys.readouterr()
+    cfg, w = plain.read_model(str(model))
+    assert [int(t) for t in out.out.split()] == plain.greedy_generate(cfg, w, [5, 17, 3, 99], 6)
+    assert "wrote random weights (seed 3)" in out.err and "[summary] requests=1 failed=0" in out.err
+    # a prompt file: one line of output per prompt in <stem>_output<ext> beside it (/root/reference/src/main.cpp:105-125),
+    # --max-steps as the cap on a request's whole length (/root/reference/src/continuous_batch_server.cpp:313)
+    prompts = tmp_path / "prompts.txt"
+    prompts.write_text("1 2 3\n\n  \n7,8,9,10,11\n400\n")
+    assert main(["-f", str(prompts), "-m", "8"] + common) == 0
+    capsys.readouterr()
+    lines = (tmp_path / "prompts_output.txt").read_text().splitlines()
+    expected = [plain.greedy_generate(cfg, w, p, max(1, 8 - len(p) + 1)) for p in ([1, 2, 3], [7, 8, 9, 10, 11], [400])]
+    assert [[int(t) for t in ln.split()] for ln in lines] == expected
+    assert [len(e) for e in expected] == [6, 4, 8]
+
+
+def test_main_reports_a_request_that_failed_and_keeps_the_others(tmp_path, capsys, emulated_backend):
+    import json
+
+    import plain_qwen2 as plain
+    from conftest import TINY_A
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    model = str(tmp_path / "model")
+    write_random_model(model, TINY_A, seed=0)
+    prompts = tmp_path / "p.txt"
+    prompts.write_text("1 2 3\n" + " ".join(str(i % 500) for i in range(100)) + "\n4 5\n")
+    # a cache of 64 tokens cannot hold the second request (100 tokens) even alone; the others are generated
+    rc = main(["-f", str(prompts), "--model", model, "--dtype", "float32", "--device", "cpu", "--greedy", "--ignore-eos",
+               "--max-new-tokens", "4", "--cache-tokens", "64", "--serve-stats-ms", "0"])
+    err = capsys.readouterr().err
+    assert rc == 1 and "request 1 failed" in err and "even alone" in err and "failed=1" in err
+    cfg, w = plain.read_model(model)
+    lines = (tmp_path / "p_output.txt").read_text().split("\n")
+    assert [int(t) for t in lines[0].split()] == plain.greedy_generate(cfg, w, [1, 2, 3], 4)
+    assert lines[1] == "" and [int(t) for t in lines[2].split()] == plain.greedy_generate(cfg, w, [4, 5], 4)
+
+
+def test_unexpected_tensors_are_an_error_unless_allowed(tmp_path, capsys, emulated_backend):
+    import torch
+
+    from conftest import TINY_A
+    from easy_gpt.cpp_amd.weights import SafetensorsFile, WeightsError, write_random_model, write_safetensors
+
+    model = str(tmp_path / "model")
+    write_random_model(model, TINY_A, seed=0)
+    path = str(tmp_path / "model" / "model.safetensors")
+    with SafetensorsFile(path) as f:
+        tensors = {n: f.read(n) for n in f.names()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.ones(8)
+    write_safetensors(path, tensors)
+    args = ["--model", model, "--dtype", "float32", "--device", "cpu", "--greedy", "--max-new-tokens", "2",
+            "--serve-stats-ms", "0", "--cache-tokens", "64", "1 2 3"]
+    with pytest.raises(WeightsError, match="unexpected tensors"):
+        main(args)
+    assert main(["--allow-unexpected-tensors"] + args) == 0
+    assert "rotary_emb.inv_freq' is not used by this model and was ignored" in capsys.readouterr().err

@@ -93,6 +93,48 @@ def test_mixed_batches_with_page_reuse(sharp_models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_the_general_step_kernel_by_kernel(sharp_models, name, dtype):
+    # no graphs at all: every step builds its own metadata (one packed upload, nothing padded) and runs kernel by
+    # kernel, which is what steps of more than `graph_tokens` tokens and models with per-request state do
+    cfg = TINY[name][0]
+    cap = cfg["max_position_embeddings"]
+    reqs = H.make_requests(cfg["vocab_size"], [min(n, cap) for n in (5, 100, 33, 77, 128, 60)], seed=23)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    for cut, trace in [("whole", H.trace_whole(reqs)), ("last32", H.trace_last_decoded(reqs, 32)),
+                       ("portions", H.trace_portions(reqs)), ("mixed", H.trace_mixed(reqs, seed=5, decode_tail=20))]:
+        eng = engine_for(sharp_models[name], dtype, page_size=16 if cut != "mixed" else 4, use_graphs=False,
+                         max_tokens=H.max_live_tokens(trace, 16))
+        rows = H.replay(eng, trace)
+        assert len(rows) == sum(len(v) for v in reqs.values())
+        H.assert_rows_match(rows, ref, tol_of(dtype), f"{name} {dtype} {cut}, no graphs")
+        assert not eng._decode_plans and not eng._row_plans and not eng._padded_plans
+        assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_beyond_the_graphs_sizes_take_the_general_step(sharp_models, dtype):
+    # graphs only up to 64 tokens a step here: the larger portions of the same trace take the general step, the
+    # smaller ones the graphs, and decoded tokens ride beside both
+    name = "D"
+    cfg = TINY[name][0]
+    reqs = H.make_requests(cfg["vocab_size"], [300, 200, 90], seed=24)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=(dtype == "bfloat16"))
+    a, b, c = reqs["r0"], reqs["r1"], reqs["r2"]
+    trace = [H.step_record(0, [("r0", a[:130], [0, 129])]),                                   # general
+             H.step_record(1, [("r0", a[130:131], [0]), ("r1", b[:100], [99])]),              # general, mixed
+             H.step_record(2, [("r1", b[100:140], [0, 39]), ("r0", a[131:132], [0])]),        # 41 tokens: rows graph
+             H.step_record(3, [("r0", a[132:133], [0]), ("r1", b[140:141], [0])]),            # decode graph
+             H.step_record(4, [("r2", c, list(range(90))), ("r0", a[133:134], [0]), ("r1", b[141:], [58])], ["r1", "r2"]),
+             H.step_record(5, [("r0", a[134:], list(range(166)))], ["r0"])]
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, 16))
+    eng.graph_tokens = 64
+    rows = H.replay(eng, trace)
+    H.assert_rows_match(rows, ref, tol_of(dtype), f"steps beyond the graphs {dtype}")
+    assert not eng._padded_plans and eng._row_plans and eng._decode_plans
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(sharp_models, dtype):
     # one request decoded token by token over many pages, another joining half way
     name = "C" if dtype == "float32" else "D"
