@@ -1,5 +1,4 @@
-from .manager import CacheManager, RequestCache
-from .pages import NoFreeSlot, OutOfPages
+from .manager import CacheManager, NoFreeSlot, OutOfPages, RequestCache
 from .storage import KVStorage, StateStorage
 
 __all__ = ["CacheManager", "KVStorage", "NoFreeSlot", "OutOfPages", "RequestCache", "StateStorage"]

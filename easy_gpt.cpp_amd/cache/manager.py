@@ -28,7 +28,15 @@ from __future__ import annotations
 import ctypes
 
 from ..parts.base import CacheNeed
-from .pages import NoFreeSlot, OutOfPages
+
+
+class OutOfPages(RuntimeError):
+    """Not enough free pages; nothing was taken."""
+
+
+class NoFreeSlot(RuntimeError):
+    """Every request slot is in use."""
+
 
 __all__ = ["CacheManager", "RequestCache", "OutOfPages", "NoFreeSlot"]
 

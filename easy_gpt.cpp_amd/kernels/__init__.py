@@ -29,10 +29,62 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
   swiglu(gate_up act[T,2I], out act[T,I])        out = silu(gate_up[:, :I]) * gate_up[:, I:]
   argmax(logits f32[R,V], out i32[R])            lowest index among equal maxima
   sample(logits f32[R,V], temperature f32[R], top_k i32[R], top_p f32[R], uniform f32[R], out i32[R])
+
+Beside these, a backend has fused variants that fold neighbouring operations into one kernel.  They are part of
+the contract too (`KernelBackend` below): each returns None (False for the decode attention) where it does not
+cover a case, and the caller then takes the unfused way.
 """
 from __future__ import annotations
 
+import contextlib
+
 _backend = None
+
+
+class KernelBackend:
+    """What parts may call on a backend beyond the operations listed above, with the answers of a backend that
+    fuses nothing.  `kernels.hip.HipKernels` overrides them where its kernels cover the shapes."""
+
+    name = "abstract"
+    fused_rows = 0          # products whose x operand is computed while it is staged take at most this many rows
+
+    def pinned_stream(self):
+        """Context manager within which every launch goes to the stream that is current on entry."""
+        return contextlib.nullcontext()
+
+    def product(self, x, w, unrounded=False):
+        """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up."""
+        raise NotImplementedError
+
+    def product_normed(self, h, delta, norm_weight, w):
+        """((h + delta) * norm_weight) w^T without the rows' 1/rms factor: (float32 partial sums [S, T, N], row sums
+        of squares [S2, T], h + delta as a new tensor), or None."""
+        return None
+
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w):
+        """swiglu(scale * sum of the partial sums gate_up) w^T as float32 partial sums, or None."""
+        return None
+
+    def product_attention(self, part_o, part_ml, w):
+        """(the combined parts of a split attention) w^T as float32 partial sums, or None."""
+        return None
+
+    def gate_up_swiglu(self, x, w):
+        """silu(x Wgate^T) * (x Wup^T) as act [T, I] in one kernel, or None."""
+        return None
+
+    def attention_decode_fused(self, *args, **kwargs):
+        """Bias, rotation, cache store and attention for single decoded tokens straight from the QKV product's partial
+        sums; False if not covered (nothing was done), else what paged_attention returns."""
+        return False
+
+    def combine_attention(self, part_o, part_ml, out):
+        """out act [T, nq*hd] from the parts of a split attention."""
+        raise NotImplementedError
+
+    def rope_table(self, positions, inv_freq):
+        """float32 [T, half, 2]: (cos, sin) of every token's angles, for the kernels that rotate; or None."""
+        return None
 
 
 class KernelsUnavailable(RuntimeError):

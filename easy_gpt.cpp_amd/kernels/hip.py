@@ -10,7 +10,7 @@ import ctypes
 
 import torch
 
-from . import KernelsUnavailable
+from . import KernelBackend, KernelsUnavailable
 
 _F32, _BF16, _I32 = torch.float32, torch.bfloat16, torch.int32
 _DT = {_F32: 0, _BF16: 1}
@@ -64,7 +64,7 @@ class _PinnedStream:
         return False
 
 
-class HipKernels:
+class HipKernels(KernelBackend):
     name = "hip-gfx950"
 
     def __init__(self):

@@ -103,7 +103,7 @@ class GQAttention(Mixer):
         if isinstance(x, PendingNorm):
             fused = None
             rms = x.rms()
-            if rms is not None and rot is not None and hasattr(k, "product_normed"):
+            if rms is not None and rot is not None:
                 fused = k.product_normed(x.h, x.delta, rms[0], self.w_qkv)
             if fused is not None:
                 prod, row_ss, h_new = fused
@@ -121,13 +121,13 @@ class GQAttention(Mixer):
             hd=self.head_dim, page_size=cache.page_size,
         )
         attn = torch.empty((t, self.q_size), dtype=dtype, device=device)
-        want_parts = self.b_o is None and hasattr(k, "product_attention") and t <= getattr(k, "fused_rows", 0)
+        want_parts = self.b_o is None and t <= k.fused_rows
         # ---- single decoded tokens: bias, rotation, the store of the new key and value and the attention over
         # the cache in one kernel, straight from the product's partial sums
         parts = False
-        cos_sin = self.position.table(ctx) if (rot is not None and hasattr(self.position, "table")) else None
+        cos_sin = self.position.table(ctx) if rot is not None else None
         if (prod.dim() == 3 and rot is not None and slots is not None and ctx.max_q_len == 1
-                and getattr(ctx, "rows_independent", True) and hasattr(k, "attention_decode_fused")):
+                and ctx.rows_independent):
             parts = k.attention_decode_fused(
                 prod, scale_args.get("row_ss"), scale_args.get("hidden", 0), scale_args.get("eps", 0.0), self.b_qkv,
                 ctx.positions, rot[0], rot[1], slots, attn, cache.k, cache.v, cache.block_table, ctx.q_start, ctx.kv_len,

@@ -104,6 +104,11 @@ class Norm(Part):
     returns norm(h) as act [T, H].  forward_rows does the same for selected rows without
     writing h back (used for the rows whose logits are wanted)."""
 
+    def rms_params(self) -> tuple[torch.Tensor, float] | None:
+        """(weight, eps) if this norm is y = x / sqrt(mean(x^2) + eps) * weight, so that a part may fold it into its
+        own first kernel; None for any other norm."""
+        return None
+
     def forward(self, h: torch.Tensor, delta: torch.Tensor | None) -> torch.Tensor:
         raise NotImplementedError
 
@@ -126,7 +131,7 @@ class PendingNorm:
 
     def rms(self):
         """(weight, eps) if the norm is y = x / rms(x) * weight, else None."""
-        return self.norm.rms_params() if hasattr(self.norm, "rms_params") else None
+        return self.norm.rms_params()
 
     def applied(self, h_new: torch.Tensor) -> None:
         self.h_after = h_new
@@ -146,6 +151,11 @@ class PositionEncoding(Part):
     """
 
     def rotary(self, device) -> tuple[torch.Tensor, int] | None:
+        return None
+
+    def table(self, ctx) -> torch.Tensor | None:
+        """For a rotary encoding: the step's cosines and sines float32 [T, rotary_dim / 2, 2], made once per step
+        and shared by the layers (`ctx.shared`); None if there is no such table."""
         return None
 
     def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:

@@ -48,7 +48,7 @@ class SwiGLU(FeedForward):
         if isinstance(x, PendingNorm):
             rms = x.rms()
             fused = None
-            if rms is not None and hasattr(k, "product_normed") and self.intermediate_size % 8 == 0:
+            if rms is not None and self.intermediate_size % 8 == 0:
                 fused = k.product_normed(x.h, x.delta, rms[0], self.w_gate_up)
             if fused is not None:
                 gate_up, row_ss, h_new = fused
@@ -62,12 +62,11 @@ class SwiGLU(FeedForward):
                 return k.product(act, self.w_down)
             x = x.materialize()
         t = x.shape[0]
-        if hasattr(k, "gate_up_swiglu"):
-            act = k.gate_up_swiglu(x, self.w_gate_up)    # a few dozen tokens: product and activation in one kernel
-            if act is not None:
-                return k.product(act, self.w_down)
+        act = k.gate_up_swiglu(x, self.w_gate_up)        # a few dozen tokens: product and activation in one kernel
+        if act is not None:
+            return k.product(act, self.w_down)
         gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]
-        if gate_up.dim() == 3 and hasattr(k, "product_swiglu"):
+        if gate_up.dim() == 3:
             out = k.product_swiglu(gate_up, None, self.hidden_size, 0.0, self.w_down)
             if out is not None:
                 return out

@@ -118,13 +118,9 @@ class Model:
     # ------------------------------------------------------------------ one step
     def forward(self, ctx) -> torch.Tensor | None:
         """Run the step described by `ctx`; returns float32 logits [rows, V] or None if no row is wanted."""
-        if hasattr(ctx, "shared"):
-            ctx.shared.clear()                       # per-step values that layers share are made anew every step
-        pin = getattr(kernels.backend(), "pinned_stream", None)
-        if pin is not None:
-            with pin():                              # one look-up of the current stream for the whole pass
-                return self._forward(ctx)
-        return self._forward(ctx)
+        ctx.shared.clear()                           # per-step values that layers share are made anew every step
+        with kernels.backend().pinned_stream():      # one look-up of the current stream for the whole pass
+            return self._forward(ctx)
 
     def _forward(self, ctx) -> torch.Tensor | None:
         h = self.embedding.forward(ctx.token_ids)

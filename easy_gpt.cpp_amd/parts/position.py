@@ -45,16 +45,11 @@ class RotaryHalfSplit(PositionEncoding):
     def table(self, ctx):
         """The step's cosines and sines [T, rotary_dim / 2, 2], computed by the first layer that asks and
         shared by the others (the angles depend on the positions only); None if the backend has no such kernel."""
-        k = kernels.backend()
-        shared = getattr(ctx, "shared", None)
-        if shared is None or not hasattr(k, "rope_table"):
-            return None
         key = ("rope_table", self.theta, self.rotary_dim)
-        tab = shared.get(key)
-        if tab is None:
+        if key not in ctx.shared:
             inv_freq, _ = self.rotary(ctx.positions.device)
-            tab = shared[key] = k.rope_table(ctx.positions, inv_freq)
-        return tab
+            ctx.shared[key] = kernels.backend().rope_table(ctx.positions, inv_freq)
+        return ctx.shared[key]
 
 
 class NoPosition(PositionEncoding):

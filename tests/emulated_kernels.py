@@ -10,6 +10,8 @@ from __future__ import annotations
 
 import torch
 
+from easy_gpt.cpp_amd.kernels import KernelBackend
+
 F64 = torch.float64
 
 
@@ -18,7 +20,7 @@ def _whole(t):
     return t.sum(0) if t is not None and t.dim() == 3 else t
 
 
-class EmulatedKernels:
+class EmulatedKernels(KernelBackend):
     name = "emulated"
 
     def product(self, x, w, unrounded=False):

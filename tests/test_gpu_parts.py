@@ -116,7 +116,7 @@ def test_attention_part_whole_and_cut(dtype, nq, nkv, hd, hidden, window, bias, 
         slots = (table[0, (positions // ps).long()] * ps + positions % ps).to(torch.int32)
         one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
         ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(n), kv_len=one(pos + n), max_q_len=n,
-                              max_kv_len=pos + n)
+                              max_kv_len=pos + n, shared={}, rows_independent=True)
         cache = CacheView(kc, vc, ps, table, slots, window, True)
         outs.append(whole(att.forward(x[pos : pos + n].to(DEV), ctx, cache, None)))
         pos += n
@@ -156,7 +156,8 @@ def test_pre_norm_block(dtype):
     positions = torch.arange(s, dtype=torch.int32, device=DEV)
     slots = (table[0, (positions // ps).long()] * ps + positions % ps).to(torch.int32)
     one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
-    ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(s), kv_len=one(s), max_q_len=s, max_kv_len=s)
+    ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(s), kv_len=one(s), max_q_len=s, max_kv_len=s, shared={},
+                          rows_independent=True)
     h, delta = block.forward(x.to(DEV).clone(), None, ctx, CacheView(kc, vc, ps, table, slots, None, True), None)
     got = h.double().cpu() + whole(delta).cpu()
     assert float((h.double().cpu() - a).abs().max()) <= tol(dtype) * float(a.abs().max())

@@ -91,6 +91,7 @@ def compare(rows, cfg, w, reqs, tol, what):
             scale = max(scale, float(ref[i].abs().max()))
             if d > worst:
                 worst, where = d, (rid, pos)
+    print(f"{what}: {len(rows)} rows, largest error {worst / scale:.2e} of the logit scale {scale:.2f}", flush=True)
     assert worst <= tol * scale, f"{what}: max |diff| {worst:.3e} at {where} exceeds {tol:g} x {scale:.3f}"
     return worst / scale
 

@@ -52,7 +52,7 @@ def test_trace_run_mixed_trace(tiny_models, tmp_path, dtype):
     trace = H.trace_mixed(reqs, seed=4, decode_tail=32, want_all=False)
     rows = run_trace(tiny_models[name], dtype, trace, str(tmp_path / "out"), H.max_live_tokens(trace, 64), cfg["vocab_size"])
     assert len(rows) > 150
-    H.assert_rows_match(rows, ref, H.FP32_TOL if dtype == "float32" else H.BF16_TOL, f"trace_run {dtype}")
+    H.assert_rows_match(rows, ref, H.FP32_TOL if dtype == "float32" else H.BF16_TOL_RANDOM, f"trace_run {dtype}")
 
 
 def test_trace_run_whole_and_last32(tiny_models, tmp_path):
