@@ -11,13 +11,15 @@ extern "C" {
 const char* egpt_error_string(int code);
 int egpt_abi_version(void);
 
-int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, int hidden, int vocab, int dtype,
-               void* stream);
+// The residual stream (`out` here, `h` below) is float32 [rows][hidden], or with fixed != 0 64-bit fixed point in
+// units of 2^-32 (see common.h), which the products of steps of few tokens add their partial results into.
+int egpt_embed(const int32_t* ids, const void* table, void* out, int fixed, int n_tokens, int hidden, int vocab,
+               int dtype, void* stream);
 // h += delta (delta may be null); out = rmsnorm(h) * weight.  rows == null: every row, h written back.
 // rows != null: only the listed rows, gathered into out[n_rows], h untouched.
 // A product may arrive as float32 partial sums of a split-k product, [n_splits][rows][cols]: then the
 // *_splits argument is > 0 and the consumer adds the splits up; 0 means one tensor of the activation type.
-int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
+int egpt_add_rmsnorm(void* h, int fixed, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
                      const void* weight, float eps, void* out, int n_rows, int hidden, int dtype, void* stream);
 // row_ss (may be null) float32 [ss_splits, n_tokens]: gate_up are float32 partial sums that still lack each row's factor
 // 1/sqrt(sum_s row_ss[s][t] / hidden + eps)
@@ -35,8 +37,10 @@ int egpt_qkv_rope_store(const void* qkv_in, int n_splits, const float* row_ss, i
 int egpt_rope_table(const int32_t* positions, const float* inv_freq, float* cos_sin, int n_tokens, int half, void* stream);
 // bfloat16 product for m <= 64 rows on the matrix cores, optionally split over k (see gemm_skinny.hip).
 // waves: wavefronts (of 16 columns of the result each) per workgroup, 4, 8 or 16; here and below.
-int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m, int n,
-                     int k, int n_splits, int waves, void* stream);
+// acc_fixed != null (here and in the products below): instead of writing partial sums, every workgroup adds its
+// part of the product into acc_fixed [m][n], a residual stream in fixed point, with integer atomics.
+int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, void* acc_fixed,
+                     int m, int n, int k, int n_splits, int waves, void* stream);
 // float32 product on the matrix cores (float32 operands and accumulation): out [n_splits][m][n] are partial sums over
 // n_splits ranges of k (bias only with one).  k % 4 == 0.  A row's values do not depend on m or on the other rows.
 int egpt_gemm_f32(const float* x, const float* w, const float* bias, float* out, int m, int n, int k, int n_splits,
@@ -80,14 +84,15 @@ int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const floa
 int egpt_attention_combine(const float* part_o, const float* part_ml, void* out, int n_rows, int hd, int n_splits,
                            void* stream);
 // Products for m <= 16 rows whose x operand is computed while it is staged (see gemm_skinny.hip).
-int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits, const void* norm_w,
-                          const void* w, float* out, float* ss_out, int m, int n, int k, int n_splits, int waves,
-                          void* stream);
+// h_fixed != 0: h_in is a fixed-point residual stream that is complete as it is (no delta, h_out unused).
+int egpt_gemm_skinny_norm(const void* h_in, int h_fixed, float* h_out, const float* delta, int delta_splits,
+                          const void* norm_w, const void* w, float* out, float* ss_out, int m, int n, int k,
+                          int n_splits, int waves, void* stream);
 int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits, int hidden,
-                            float eps, const void* w, float* out, int m, int n, int k, int n_splits, int waves,
-                            void* stream);
+                            float eps, const void* w, float* out, void* acc_fixed, int m, int n, int k, int n_splits,
+                            int waves, void* stream);
 int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd, const void* w,
-                          float* out, int m, int n, int n_splits, int waves, void* stream);
+                          float* out, void* acc_fixed, int m, int n, int n_splits, int waves, void* stream);
 // Gate/up product with SwiGLU for up to 64 rows (see gemm_gate_up.hip): out bfloat16 [m][inter] from x bfloat16 [m][k]
 // and w bfloat16 [2 * inter][k] (gate rows, then up rows); k % 8 == 0.
 int egpt_gemm_gate_up_swiglu(const void* x, const void* w, void* out, int m, int inter, int k, int groups, void* stream);

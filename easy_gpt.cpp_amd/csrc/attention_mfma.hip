@@ -520,6 +520,7 @@ struct FusedQkv {
     const int32_t* slots;     // [n_tokens] page * page_size + offset of the token's key and value
     bf16_t* k_cache_w;        // the caches again, writable
     bf16_t* v_cache_w;
+    unsigned trace_base;      // builds with EGPT_TRACE: the first record of this launch's workgroups
 };
 
 // Decoded tokens only (one query token per request, its heads of one kv group in one 16-row tile): a
@@ -549,6 +550,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     const int lj = lane % 16, lg = lane / 16;
     const int b = blockIdx.x, kh = blockIdx.y, split = blockIdx.z;
     const int group_size = nq / nkv;
+    EGPT_MARK(f.trace_base, 5, 0);
     const int kv = kv_len[b], tok = q_start[b];
     const int p = kv - 1;
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
@@ -738,7 +740,10 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     int kb0 = w_begin;
     do {
         load_round(kb0);
-        if (kb0 == w_begin) make_q();
+        if (kb0 == w_begin) {
+            make_q();
+            EGPT_MARK(f.trace_base, 5, 1);
+        }
         if constexpr (FUSED) {
             // the new token's key and value come from LDS, not from the cache line that was just written
             if (writer && kb0 <= kb_end - 1 && kb_end - 1 < min(w_end, kb0 + PF)) {
@@ -814,6 +819,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
         }
         kb0 += PF;
     } while (kb0 < w_end);
+    EGPT_MARK(f.trace_base, 5, 2);
     float l = l_run;
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
@@ -852,6 +858,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
             }
         }
     }
+    EGPT_MARK(f.trace_base, 5, 3);
 }
 
 // out[row, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits; one wavefront per row.
@@ -929,16 +936,18 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
     size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
     if (fused) lds += 18 * HD * sizeof(bf16_t);          // 16 query heads, the new key and value
     if (lds > 64 * 1024) return EGPT_UNSUPPORTED_SIZE;
+    FusedQkv fq = fused ? *fused : FusedQkv{};
+    fq.trace_base = EGPT_TRACE_TAKE(grid);
     if (fused)
         attention_decode_kernel<HD, PF, true><<<grid, n_waves * kWave, lds, s>>>(
             nullptr, static_cast<bf16_t*>(out), part_o, part_ml, static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, kv_len, n_tokens, nq, nkv,
-            page_size, scale, window, n_splits, *fused);
+            page_size, scale, window, n_splits, fq);
     else
         attention_decode_kernel<HD, PF, false><<<grid, n_waves * kWave, lds, s>>>(
             static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
             static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
-            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, FusedQkv{});
+            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq);
     EGPT_CHECK_LAUNCH();
     if (n_splits > 1 && combine) {
         attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
@@ -965,6 +974,7 @@ static int dispatch_decode(const void* qkv, void* out, float* part_o, float* par
 }  // namespace egpt
 
 using namespace egpt;
+EGPT_TRACE_ATTACH(attention_mfma)
 
 // Prompt portions (and mixed batches) with keys and values shared through LDS by the wavefronts of a
 // workgroup.  Same operands and meaning as egpt_paged_attention_mfma with n_splits == 1; page sizes that are

@@ -42,6 +42,24 @@ __device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, 
     rb = __fmaf_rn(a, s, __fmul_rn(b, c));
 }
 
+// The residual stream of steps of few tokens in 64-bit fixed point (units of 2^-32).  Several workgroups that split
+// a product's k range add their partial results straight into it with integer atomics: integer addition does not
+// care for the order, so the sum is the same bits whatever the scheduling, and the kernels that read the stream
+// read one small tensor instead of every workgroup's partial sums.  A float32 value times 2^32 is an integer for
+// every magnitude of 2^-8 and above and is rounded to one below; the stream holds magnitudes below 2^31.
+typedef long long fixed_t;
+constexpr float kFixedOne = 4294967296.0f;
+__device__ __forceinline__ fixed_t to_fixed(float v) { return __float2ll_rn(v * kFixedOne); }
+__device__ __forceinline__ float fixed_to_float(fixed_t v) { return __ll2float_rn(v) * (1.0f / kFixedOne); }
+__device__ __forceinline__ void fixed_add(fixed_t* p, float v) {
+    atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(to_fixed(v)));
+}
+// what a residual stream of either kind is read and written as
+__device__ __forceinline__ float residual_load(const float* p) { return *p; }
+__device__ __forceinline__ float residual_load(const fixed_t* p) { return fixed_to_float(*p); }
+__device__ __forceinline__ void residual_store(float* p, float v) { *p = v; }
+__device__ __forceinline__ void residual_store(fixed_t* p, float v) { *p = to_fixed(v); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
@@ -78,6 +96,45 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 }
 
 }  // namespace egpt
+
+// Timestamps from inside kernels, for builds with -DEGPT_TRACE only (an ordinary build has none of this).
+// EGPT_MARK(base, kernel, phase): the first thread of a workgroup stores the wall clock (units of 10 ns) of `phase`
+// (0 to 3) into record `base + workgroup` of a buffer that the host attached with
+// egpt_trace_attach_<file>(buffer, capacity); a launcher takes `base` for its grid from egpt_trace_take, so a
+// captured graph's nodes keep their records over replays.  A decode step is a chain of short dependent kernels;
+// what a link's time is made of (launch, the first load's way from memory, arithmetic, the tail) shows only
+// from inside.  A record is five words: (kernel << 48 | workgroup), then the four phases' clocks.
+#ifdef EGPT_TRACE
+extern "C" unsigned egpt_trace_take(unsigned n_workgroups);
+namespace egpt {
+static __device__ unsigned long long* trace_buf = nullptr;
+static __device__ unsigned int trace_cap = 0;
+__device__ __forceinline__ void trace_mark(unsigned base, unsigned kernel, unsigned phase) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (threadIdx.x == 0 && trace_buf) {
+        const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        if (base + wg < trace_cap) {
+            unsigned long long* rec = trace_buf + static_cast<size_t>(base + wg) * 5;
+            if (phase == 0) rec[0] = (static_cast<unsigned long long>(kernel) << 48) | wg;
+            rec[1 + phase] = wall_clock64();
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+}  // namespace egpt
+#define EGPT_MARK(base, kernel, phase) egpt::trace_mark(base, kernel, phase)
+#define EGPT_TRACE_TAKE(grid) egpt_trace_take((grid).x * (grid).y * (grid).z)
+#define EGPT_TRACE_ATTACH(file)                                                                          \
+    extern "C" int egpt_trace_attach_##file(void* buf, unsigned cap) {                                   \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(egpt::trace_buf), &buf, sizeof(buf)) != hipSuccess) return 1;   \
+        if (hipMemcpyToSymbol(HIP_SYMBOL(egpt::trace_cap), &cap, sizeof(cap)) != hipSuccess) return 1;   \
+        return 0;                                                                                        \
+    }
+#else
+#define EGPT_MARK(base, kernel, phase) do {} while (0)
+#define EGPT_TRACE_TAKE(grid) 0u
+#define EGPT_TRACE_ATTACH(file)
+#endif
 
 // Error codes returned by every entry point (0 = launched).
 #define EGPT_OK 0

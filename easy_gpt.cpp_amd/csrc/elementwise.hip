@@ -31,30 +31,31 @@ struct ProductView {
 };
 
 // ----------------------------------------------------------------------------- embedding
-// x[t, :] = E[id_t, :]   (/root/reference/src/models/embedding.cpp:54-76); output float32.
-template <typename T>
-__global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+// x[t, :] = E[id_t, :]   (/root/reference/src/models/embedding.cpp:54-76); output: the residual stream, float32 or
+// fixed point.
+template <typename T, typename R>
+__global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table, R* __restrict__ out,
                              int hidden, int vocab) {
     const int t = blockIdx.x;
     int id = ids[t];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // ids are range-checked on the host; never read outside
     const T* row = table + static_cast<size_t>(id) * hidden;
-    float* o = out + static_cast<size_t>(t) * hidden;
-    for (int j = threadIdx.x; j < hidden; j += blockDim.x) o[j] = to_float(row[j]);
+    R* o = out + static_cast<size_t>(t) * hidden;
+    for (int j = threadIdx.x; j < hidden; j += blockDim.x) residual_store(o + j, to_float(row[j]));
 }
 
 // ----------------------------------------------------------------------------- add + RMSNorm
 // ss = sum x^2 (float32), inv = 1/sqrt(ss/H + eps), y = x * inv * w
 // (/root/reference/src/models/norm.cpp:47-59, /root/reference/src/cuda/ops/self_attn_detail.cuh:385-418).
 // The residual addition h += delta happens here too, in float32.
-template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
+template <typename T, typename R>
+__global__ void add_rmsnorm_kernel(R* __restrict__ h, ProductView<T> delta,
                                    const int32_t* __restrict__ rows, const T* __restrict__ weight, float eps,
                                    T* __restrict__ out, int hidden) {
     __shared__ float scratch[16];
     const int r = blockIdx.x;
     const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
-    float* hrow = h + src * hidden;
+    R* hrow = h + src * hidden;
     const bool has_delta = delta.present();
     const size_t dbase = src * hidden;
     const bool write_back = (rows == nullptr) && has_delta;
@@ -64,10 +65,10 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
     float kept = 0.f, kept_w = 0.f;
     float ss = 0.f;
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-        float v = hrow[j];
+        float v = residual_load(hrow + j);
         if (one_pass) kept_w = to_float(weight[j]);
         if (has_delta) v += delta.at(dbase + j);
-        if (write_back) hrow[j] = v;
+        if (write_back) residual_store(hrow + j, v);
         ss += v * v;
         kept = v;
     }
@@ -79,7 +80,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, ProductView<T> delta,
         return;
     }
     for (int j = threadIdx.x; j < hidden; j += blockDim.x) {
-        float v = hrow[j];                       // already updated when written back
+        float v = residual_load(hrow + j);       // already updated when written back
         if (has_delta && !write_back) v += delta.at(dbase + j);
         orow[j] = from_float<T>(v * inv * to_float(weight[j]));
     }
@@ -385,17 +386,20 @@ __global__ __launch_bounds__(256) void qkv_rope_store_rows_kernel(const IN* __re
 
 using namespace egpt;
 
-extern "C" int egpt_embed(const int32_t* ids, const void* table, float* out, int n_tokens, int hidden, int vocab,
-                          int dtype, void* stream) {
-    if (!ids || !table || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0) return EGPT_BAD_ARGUMENT;
+extern "C" int egpt_embed(const int32_t* ids, const void* table, void* out, int fixed, int n_tokens, int hidden,
+                          int vocab, int dtype, void* stream) {
+    if (!ids || !table || !out || n_tokens < 0 || hidden <= 0 || vocab <= 0 || (dtype != 0 && dtype != 1))
+        return EGPT_BAD_ARGUMENT;
     if (n_tokens == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == 0)
-        embed_kernel<float><<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), out, hidden, vocab);
-    else if (dtype == 1)
-        embed_kernel<bf16_t><<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), out, hidden, vocab);
+    if (dtype == 0 && !fixed)
+        embed_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), static_cast<float*>(out), hidden, vocab);
+    else if (dtype == 0)
+        embed_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const float*>(table), static_cast<fixed_t*>(out), hidden, vocab);
+    else if (!fixed)
+        embed_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), static_cast<float*>(out), hidden, vocab);
     else
-        return EGPT_BAD_ARGUMENT;
+        embed_kernel<<<n_tokens, 256, 0, s>>>(ids, static_cast<const bf16_t*>(table), static_cast<fixed_t*>(out), hidden, vocab);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -410,9 +414,9 @@ static ProductView<T> make_view(const void* p, int n_splits, size_t split_stride
     return v;
 }
 
-extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, int delta_rows, const int32_t* rows,
-                                const void* weight, float eps, void* out, int n_rows, int hidden, int dtype,
-                                void* stream) {
+extern "C" int egpt_add_rmsnorm(void* h, int fixed, const void* delta, int delta_splits, int delta_rows,
+                                const int32_t* rows, const void* weight, float eps, void* out, int n_rows, int hidden,
+                                int dtype, void* stream) {
     if (!h || !weight || !out || n_rows < 0 || hidden <= 0 || delta_splits < 0) return EGPT_BAD_ARGUMENT;
     if (delta && delta_rows <= 0) return EGPT_BAD_ARGUMENT;
     if (n_rows == 0) return EGPT_OK;
@@ -420,29 +424,30 @@ extern "C" int egpt_add_rmsnorm(float* h, const void* delta, int delta_splits, i
     // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for
     const int threads = (delta_splits > 1 || hidden >= 4096) ? 1024 : (hidden >= 2048 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
-    if (dtype == 1 && delta_splits <= 1 && hidden % 8 == 0 && n_rows >= 32) {
+    if (dtype == 1 && delta_splits <= 1 && hidden % 8 == 0 && n_rows >= 32 && !fixed) {
         const int threads = hidden >= 2048 ? 256 : 128;
+        float* hf = static_cast<float*>(h);
         if (delta_splits == 0)
             add_rmsnorm_vec8_kernel<bf16_t><<<n_rows, threads, 0, s>>>(
-                h, static_cast<const bf16_t*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
+                hf, static_cast<const bf16_t*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
                 static_cast<bf16_t*>(out), hidden);
         else   // one float32 "partial sum": a product written out in float32
             add_rmsnorm_vec8_kernel<float><<<n_rows, threads, 0, s>>>(
-                h, static_cast<const float*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
+                hf, static_cast<const float*>(delta), rows, static_cast<const bf16_t*>(weight), eps,
                 static_cast<bf16_t*>(out), hidden);
         EGPT_CHECK_LAUNCH();
         return EGPT_OK;
     }
-    if (dtype == 0)
-        add_rmsnorm_kernel<float><<<n_rows, threads, 0, s>>>(h, make_view<float>(delta, delta_splits, stride), rows,
-                                                             static_cast<const float*>(weight), eps,
-                                                             static_cast<float*>(out), hidden);
-    else if (dtype == 1)
-        add_rmsnorm_kernel<bf16_t><<<n_rows, threads, 0, s>>>(h, make_view<bf16_t>(delta, delta_splits, stride), rows,
-                                                              static_cast<const bf16_t*>(weight), eps,
-                                                              static_cast<bf16_t*>(out), hidden);
-    else
-        return EGPT_BAD_ARGUMENT;
+    if (dtype != 0 && dtype != 1) return EGPT_BAD_ARGUMENT;
+#define EGPT_NORM(T_, R_)                                                                                              \
+    add_rmsnorm_kernel<T_, R_><<<n_rows, threads, 0, s>>>(static_cast<R_*>(h), make_view<T_>(delta, delta_splits, stride), \
+                                                          rows, static_cast<const T_*>(weight), eps,                  \
+                                                          static_cast<T_*>(out), hidden)
+    if (dtype == 0 && !fixed) EGPT_NORM(float, float);
+    else if (dtype == 0) EGPT_NORM(float, fixed_t);
+    else if (!fixed) EGPT_NORM(bf16_t, float);
+    else EGPT_NORM(bf16_t, fixed_t);
+#undef EGPT_NORM
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
@@ -588,6 +593,16 @@ extern "C" int egpt_probe_link(const float* in, float* out, int n, int trips, vo
     return EGPT_OK;
 }
 
+#ifdef EGPT_TRACE
+static unsigned g_trace_next = 0;
+extern "C" unsigned egpt_trace_take(unsigned n_workgroups) {
+    const unsigned base = g_trace_next;
+    g_trace_next += n_workgroups;
+    return base;
+}
+extern "C" void egpt_trace_reset(void) { g_trace_next = 0; }
+#endif
+
 extern "C" const char* egpt_error_string(int code) {
     switch (code) {
         case EGPT_OK: return "ok";
@@ -602,4 +617,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 11; }
+extern "C" int egpt_abi_version(void) { return 12; }

@@ -42,11 +42,13 @@ struct SkinnyArgs {
     const bf16_t* bias;
     float* out_f32;
     bf16_t* out_bf16;
+    fixed_t* acc_fixed;        // [m][n] residual stream in fixed point that the product is added into, or null
     int m, n, k, steps_per_split;
     // kPlain
     const bf16_t* x;
     // kNorm
     const float* h_in;
+    const fixed_t* h_in_fixed; // the residual stream in fixed point instead of h_in (then no delta, no h_out)
     float* h_out;
     const float* delta;        // [delta_splits][m][k] or null
     int delta_splits;
@@ -62,6 +64,7 @@ struct SkinnyArgs {
     const float* part_o;
     const float* part_ml;
     int a_splits, nq, hd;
+    unsigned trace_base;       // builds with EGPT_TRACE: the first record of this launch's workgroups
 };
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p, bool ok) {
@@ -129,6 +132,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
     const int li = lane % 16, lg = lane / 16;
     const int split = blockIdx.y;
     const int m = a.m, n = a.n, k = a.k;
+    EGPT_MARK(a.trace_base, PRO, 0);
     const int n0 = (blockIdx.x * NW + wave) * kRowsPerWave;
     const int total_steps = (k + kStep - 1) / kStep;
     const int step_begin = split * a.steps_per_split;
@@ -216,12 +220,26 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
             float f[8];
             if constexpr (PRO == kNorm) {
                 const size_t idx = static_cast<size_t>(r) * k + kc;
-                load8f(a.h_in + idx, f);
                 const uint4 wv = *reinterpret_cast<const uint4*>(a.norm_w + kc);
-                if (a.delta) add_splits8<INF>(a.delta + idx, a.delta_splits, static_cast<size_t>(m) * k, f);
-                if (blockIdx.x == 0) {
-                    *reinterpret_cast<f32x4*>(a.h_out + idx) = f32x4{f[0], f[1], f[2], f[3]};
-                    *reinterpret_cast<f32x4*>(a.h_out + idx + 4) = f32x4{f[4], f[5], f[6], f[7]};
+                if (a.h_in_fixed) {
+                    // the stream as the products before left it: nothing to add, nothing to write back
+                    fixed_t hv[8];
+                    const uint4* hp = reinterpret_cast<const uint4*>(a.h_in_fixed + idx);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint4 d = hp[q];
+                        hv[2 * q] = static_cast<fixed_t>((static_cast<unsigned long long>(d.y) << 32) | d.x);
+                        hv[2 * q + 1] = static_cast<fixed_t>((static_cast<unsigned long long>(d.w) << 32) | d.z);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = fixed_to_float(hv[j]);
+                } else {
+                    load8f(a.h_in + idx, f);
+                    if (a.delta) add_splits8<INF>(a.delta + idx, a.delta_splits, static_cast<size_t>(m) * k, f);
+                    if (blockIdx.x == 0) {
+                        *reinterpret_cast<f32x4*>(a.h_out + idx) = f32x4{f[0], f[1], f[2], f[3]};
+                        *reinterpret_cast<f32x4*>(a.h_out + idx + 4) = f32x4{f[4], f[5], f[6], f[7]};
+                    }
                 }
                 const uint32_t wb[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
@@ -360,8 +378,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
             }
         }
         __syncthreads();
+        EGPT_MARK(a.trace_base, PRO, 1);
         if (n_steps > 0) products(0, a_cur);
         if (n_steps > 1) products(1, a_next);
+        EGPT_MARK(a.trace_base, PRO, 2);
         if constexpr (PRO == kNorm) {
             if (blockIdx.x == 0 && tid < m)
                 a.ss_out[split * m + tid] = (n_steps > 0 ? ss_part[0][tid] : 0.f) + (n_steps > 1 ? ss_part[1][tid] : 0.f);
@@ -434,6 +454,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
         }
     }
     // D layout: lane (li, lg) holds rows lg*4 + v of the 16 x 16 tile (an n index) at column li (an m index)
+    if (a.acc_fixed) {
+        // Into the residual stream with atomics.  As the tiles lie in the registers, neighbouring lanes hold
+        // neighbouring rows of x, far apart in memory, and an atomic instruction would touch a cache line per
+        // lane; through LDS the workgroup's tile is turned so that neighbouring threads add to neighbouring
+        // columns of one row (a quarter of the time for the down projection of the 0.5B sizes).
+        if constexpr (MT == 1) {
+            __shared__ float turned[16][NW * 16 + 1];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) turned[li][wave * 16 + lg * 4 + v] = acc[0][v];
+            __syncthreads();
+            const int col0 = blockIdx.x * NW * 16;
+            for (int idx = tid; idx < m * NW * 16; idx += kThreads) {
+                const int r = idx / (NW * 16), c = idx % (NW * 16);
+                if (col0 + c < n) fixed_add(a.acc_fixed + static_cast<size_t>(r) * n + col0 + c, turned[r][c]);
+            }
+        }
+        EGPT_MARK(a.trace_base, PRO, 3);
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int mm = t * 16 + li;
@@ -450,6 +489,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
                 a.out_f32[(static_cast<size_t>(split) * m + mm) * n + nn] = val;
         }
     }
+    EGPT_MARK(a.trace_base, PRO, 3);
 }
 
 // The product for 17 to 64 rows and many columns: x stays in LDS for the workgroup's whole k range (up to
@@ -555,6 +595,7 @@ static dim3 skinny_grid(int n, int n_splits, int waves) {
     do {                                                                                                     \
         const dim3 grid = skinny_grid(a.n, n_splits, waves);                                                 \
         hipStream_t s_ = static_cast<hipStream_t>(stream);                                                   \
+        a.trace_base = EGPT_TRACE_TAKE(grid);                                                                \
         if (waves == 4) gemm_skinny_kernel<MT_, PRO_, INF_, 4><<<grid, 256, 0, s_>>>(a);                     \
         else if (waves == 8) gemm_skinny_kernel<MT_, PRO_, INF_, 8><<<grid, 512, 0, s_>>>(a);                \
         else gemm_skinny_kernel<MT_, PRO_, INF_, 16><<<grid, 1024, 0, s_>>>(a);                              \
@@ -563,16 +604,18 @@ static dim3 skinny_grid(int n, int n_splits, int waves) {
 }  // namespace egpt
 
 using namespace egpt;
+EGPT_TRACE_ATTACH(gemm_skinny)
 
 // out_f32 != null: float32 [n_splits][m][n] partial sums (bias only allowed with n_splits == 1).
 // out_bf16 != null: bfloat16 [m][n], n_splits must be 1.
-extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16, int m,
-                                int n, int k, int n_splits, int waves, void* stream) {
-    if (!x || !w || (!out_f32 && !out_bf16) || (out_f32 && out_bf16) || m <= 0 || n <= 0 || k <= 0 || n_splits <= 0 ||
+extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, float* out_f32, void* out_bf16,
+                                void* acc_fixed, int m, int n, int k, int n_splits, int waves, void* stream) {
+    const int n_outs = (out_f32 ? 1 : 0) + (out_bf16 ? 1 : 0) + (acc_fixed ? 1 : 0);
+    if (!x || !w || n_outs != 1 || m <= 0 || n <= 0 || k <= 0 || n_splits <= 0 ||
         (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
-    if (m > 64 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
-    if (n_splits > 1 && (bias || out_bf16)) return EGPT_BAD_ARGUMENT;
+    if (m > 64 || (k % 8) != 0 || (acc_fixed && m > 16)) return EGPT_UNSUPPORTED_SIZE;
+    if ((n_splits > 1 && (bias || out_bf16)) || (acc_fixed && bias)) return EGPT_BAD_ARGUMENT;
     SkinnyArgs a = {};
     if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
     a.x = static_cast<const bf16_t*>(x);
@@ -580,8 +623,9 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
     a.bias = static_cast<const bf16_t*>(bias);
     a.out_f32 = out_f32;
     a.out_bf16 = static_cast<bf16_t*>(out_bf16);
+    a.acc_fixed = static_cast<fixed_t*>(acc_fixed);
     a.m = m; a.n = n; a.k = k;
-    if (waves != 16 && m > 16 && a.steps_per_split <= kResidentSteps && n >= 4096) {
+    if (waves != 16 && m > 16 && a.steps_per_split <= kResidentSteps && n >= 4096 && !acc_fixed) {
         // many columns, more than one tile of rows, a k range that fits in LDS: x resident, one round of loads
         const dim3 grid = skinny_grid(n, n_splits, waves);
         hipStream_t s_ = static_cast<hipStream_t>(stream);
@@ -610,19 +654,22 @@ extern "C" int egpt_gemm_skinny(const void* x, const void* w, const void* bias, 
 
 // out[split][m][n] = partial sums of ((h_in + sum delta) * norm_w) w^T; h_out = h_in + sum delta;
 // ss_out[split][m] = sums of squares of h_out over the split's k range.  m <= 16, k % 8 == 0.
-extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const float* delta, int delta_splits,
+extern "C" int egpt_gemm_skinny_norm(const void* h_in, int h_fixed, float* h_out, const float* delta, int delta_splits,
                                      const void* norm_w, const void* w, float* out, float* ss_out, int m, int n, int k,
                                      int n_splits, int waves, void* stream) {
-    if (!h_in || !h_out || h_in == h_out || !norm_w || !w || !out || !ss_out || m <= 0 || n <= 0 || k <= 0 ||
+    if (!h_in || !norm_w || !w || !out || !ss_out || m <= 0 || n <= 0 || k <= 0 ||
         delta_splits < 0 || (delta && delta_splits == 0) || (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
+    if (h_fixed ? (delta != nullptr) : (!h_out || h_in == h_out)) return EGPT_BAD_ARGUMENT;
     if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
     SkinnyArgs a = {};
     if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
     a.w = static_cast<const bf16_t*>(w);
     a.out_f32 = out;
     a.m = m; a.n = n; a.k = k;
-    a.h_in = h_in; a.h_out = h_out; a.delta = delta; a.delta_splits = delta ? delta_splits : 0;
+    if (h_fixed) a.h_in_fixed = static_cast<const fixed_t*>(h_in);
+    else a.h_in = static_cast<const float*>(h_in);
+    a.h_out = h_out; a.delta = delta; a.delta_splits = delta ? delta_splits : 0;
     a.norm_w = static_cast<const bf16_t*>(norm_w);
     a.ss_out = ss_out;
     // Many partial sums to add and few workgroups (which then need not share a CU): more loads in flight.
@@ -642,9 +689,9 @@ extern "C" int egpt_gemm_skinny_norm(const float* h_in, float* h_out, const floa
 // out[split][m][n] = partial sums of swiglu(inv_rms * sum gate_up) w^T, gate_up [gu_splits][m][2k];
 // inv_rms[m] = 1 / sqrt(sum_s ss_in[s][m] / hidden + eps), or 1 if ss_in is null.
 extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, const float* ss_in, int ss_splits,
-                                       int hidden, float eps, const void* w, float* out, int m, int n, int k,
-                                       int n_splits, int waves, void* stream) {
-    if (!gate_up || gu_splits < 1 || !w || !out || m <= 0 || n <= 0 || k <= 0 || (ss_in && (ss_splits < 1 || hidden < 1)) ||
+                                       int hidden, float eps, const void* w, float* out, void* acc_fixed, int m, int n,
+                                       int k, int n_splits, int waves, void* stream) {
+    if (!gate_up || gu_splits < 1 || !w || (!out == !acc_fixed) || m <= 0 || n <= 0 || k <= 0 || (ss_in && (ss_splits < 1 || hidden < 1)) ||
         (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     if (m > 16 || (k % 8) != 0) return EGPT_UNSUPPORTED_SIZE;
@@ -652,6 +699,7 @@ extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, cons
     if (int e = check_splits(k, n_splits, &a.steps_per_split)) return e;
     a.w = static_cast<const bf16_t*>(w);
     a.out_f32 = out;
+    a.acc_fixed = static_cast<fixed_t*>(acc_fixed);
     a.m = m; a.n = n; a.k = k;
     a.gu = gate_up; a.gu_splits = gu_splits; a.ss_in = ss_in; a.ss_splits = ss_splits;
     a.inv_hidden = ss_in ? 1.0f / static_cast<float>(hidden) : 0.f;
@@ -664,8 +712,9 @@ extern "C" int egpt_gemm_skinny_swiglu(const float* gate_up, int gu_splits, cons
 // out[split][m][n] = partial sums of (combined attention output) w^T; part_o [a_splits][m*nq][hd] unnormalised
 // partial outputs, part_ml [a_splits][m*nq][2] their (maximum, sum); k = nq * hd.
 extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, int a_splits, int nq, int hd,
-                                     const void* w, float* out, int m, int n, int n_splits, int waves, void* stream) {
-    if (!part_o || !part_ml || a_splits < 1 || nq < 1 || hd < 1 || !w || !out || m <= 0 || n <= 0 ||
+                                     const void* w, float* out, void* acc_fixed, int m, int n, int n_splits, int waves,
+                                     void* stream) {
+    if (!part_o || !part_ml || a_splits < 1 || nq < 1 || hd < 1 || !w || (!out == !acc_fixed) || m <= 0 || n <= 0 ||
         (waves != 4 && waves != 8 && waves != 16))
         return EGPT_BAD_ARGUMENT;
     const int k = nq * hd;
@@ -675,6 +724,7 @@ extern "C" int egpt_gemm_skinny_attn(const float* part_o, const float* part_ml, 
     if ((a.steps_per_split * kStep + hd - 1) / hd + 1 > kMaxLocalHeads) return EGPT_UNSUPPORTED_SIZE;
     a.w = static_cast<const bf16_t*>(w);
     a.out_f32 = out;
+    a.acc_fixed = static_cast<fixed_t*>(acc_fixed);
     a.m = m; a.n = n; a.k = k;
     a.part_o = part_o; a.part_ml = part_ml; a.a_splits = a_splits; a.nq = nq; a.hd = hd;
     EGPT_SKINNY(1, kAttn, 8);

@@ -52,8 +52,16 @@ class KernelBackend:
         """Context manager within which every launch goes to the stream that is current on entry."""
         return contextlib.nullcontext()
 
-    def product(self, x, w, unrounded=False):
-        """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up."""
+    def residual_dtype(self, n_tokens, act_dtype):
+        """The type of a step's residual stream: float32, or int64 (64-bit fixed point in units of 2^-32) where the
+        backend's products can add themselves into the stream (`residual=`)."""
+        import torch
+
+        return torch.float32
+
+    def product(self, x, w, unrounded=False, residual=None):
+        """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up; or, given
+        a residual stream in fixed point that the backend can add the product into, that stream."""
         raise NotImplementedError
 
     def product_normed(self, h, delta, norm_weight, w):
@@ -61,12 +69,14 @@ class KernelBackend:
         of squares [S2, T], h + delta as a new tensor), or None."""
         return None
 
-    def product_swiglu(self, gate_up, row_ss, hidden, eps, w):
-        """swiglu(scale * sum of the partial sums gate_up) w^T as float32 partial sums, or None."""
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, residual=None):
+        """swiglu(scale * sum of the partial sums gate_up) w^T as float32 partial sums (or added into `residual`,
+        which is then returned), or None."""
         return None
 
-    def product_attention(self, part_o, part_ml, w):
-        """(the combined parts of a split attention) w^T as float32 partial sums, or None."""
+    def product_attention(self, part_o, part_ml, w, residual=None):
+        """(the combined parts of a split attention) w^T as float32 partial sums (or added into `residual`, which is
+        then returned), or None."""
         return None
 
     def gate_up_swiglu(self, x, w):

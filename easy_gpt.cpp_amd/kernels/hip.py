@@ -12,7 +12,7 @@ import torch
 
 from . import KernelBackend, KernelsUnavailable
 
-_F32, _BF16, _I32 = torch.float32, torch.bfloat16, torch.int32
+_F32, _BF16, _I32, _I64 = torch.float32, torch.bfloat16, torch.int32, torch.int64
 _DT = {_F32: 0, _BF16: 1}
 
 
@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 11:
+    if lib.egpt_abi_version() != 12:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -75,14 +75,14 @@ class HipKernels(KernelBackend):
         lib.egpt_error_string.restype = ctypes.c_char_p
         lib.egpt_error_string.argtypes = [i]
         sigs = {
-            "egpt_embed": [vp, vp, vp, i, i, i, i, vp],
-            "egpt_add_rmsnorm": [vp, vp, i, i, vp, vp, f, vp, i, i, i, vp],
+            "egpt_embed": [vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_add_rmsnorm": [vp, i, vp, i, i, vp, vp, f, vp, i, i, i, vp],
             "egpt_swiglu": [vp, i, vp, i, i, f, vp, i, i, i, vp],
             "egpt_qkv_rope_store": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, vp],
             "egpt_rope_table": [vp, vp, vp, i, i, vp],
-            "egpt_gemm_skinny_norm": [vp, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, vp],
-            "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, i, i, i, i, i, vp],
-            "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, i, i, i, i, vp],
+            "egpt_gemm_skinny_norm": [vp, i, vp, vp, i, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
             "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, i, vp],
@@ -90,7 +90,7 @@ class HipKernels(KernelBackend):
                                             i, i, f, i, i, i, i, i, vp],
             "egpt_linear": [vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_f32": [vp, vp, vp, vp, i, i, i, i, vp],
-            "egpt_gemm_skinny": [vp, vp, vp, vp, vp, i, i, i, i, i, vp],
+            "egpt_gemm_skinny": [vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
@@ -169,30 +169,56 @@ class HipKernels(KernelBackend):
         t = token_ids.shape[0]
         self._need(token_ids, "token_ids", _I32, (t,))
         self._need(table, "table")
-        self._need(out, "out", _F32, (t, h))
-        self._run("egpt_embed", token_ids.data_ptr(), table.data_ptr(), out.data_ptr(), t, h, v, dt, self._stream())
+        self._need(out, "out", None, (t, h))
+        self._run("egpt_embed", token_ids.data_ptr(), table.data_ptr(), out.data_ptr(), self._fixed(out, "out"), t, h, v,
+                  dt, self._stream())
+
+    # ------------------------------------------------------------------ the residual stream in fixed point
+    fixed_residual_elements = 1 << 20    # splits x rows x columns of a product that is added with atomics, at most
+
+    def residual_dtype(self, n_tokens: int, act_dtype) -> torch.dtype:
+        """The type of the residual stream of a step: float32, or for few tokens in bfloat16 64-bit fixed point (int64
+        in units of 2^-32).  Products whose k range is split over workgroups then add their parts straight into the
+        stream with integer atomics (`residual=` below), which gives the same bits in any order, and the kernels
+        that read the stream read one small tensor instead of every workgroup's partial sums."""
+        return _I64 if (act_dtype == _BF16 and 0 < n_tokens <= self.fused_rows) else _F32
+
+    @staticmethod
+    def _fixed(t: torch.Tensor, name: str) -> int:
+        if t.dtype not in (_F32, _I64):
+            raise TypeError(f"{name} (a residual stream) must be float32 or int64 fixed point, got {t.dtype}")
+        return 1 if t.dtype == _I64 else 0
+
+    def _residual_target(self, residual, t: int, n: int, splits: int):
+        """The stream to add a [t, n] product into, or None if it is to be returned as partial sums."""
+        if residual is None or residual.dtype != _I64 or tuple(residual.shape) != (t, n):
+            return None
+        if splits * t * n > self.fixed_residual_elements:
+            return None                  # so many atomics that partial sums and their reader are faster
+        self._need(residual, "residual", _I64, (t, n))
+        return residual
 
     def add_rmsnorm(self, h, delta, weight, eps, out):
         t, hid = h.shape
         dt = self._act(out, "out")
-        self._need(h, "h", _F32)
+        self._need(h, "h")
         self._need(weight, "weight", out.dtype, (hid,))
         self._need(out, "out", None, (t, hid))
         splits = self._product(delta, "delta", out.dtype, t, hid) if delta is not None else 0
-        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), splits, t, None, weight.data_ptr(), float(eps),
-                  out.data_ptr(), t, hid, dt, self._stream())
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._fixed(h, "h"), self._ptr(delta), splits, t, None,
+                  weight.data_ptr(), float(eps), out.data_ptr(), t, hid, dt, self._stream())
 
     def rows_add_rmsnorm(self, h, delta, rows, weight, eps, out):
         t, hid = h.shape
         r = rows.shape[0]
         dt = self._act(out, "out")
-        self._need(h, "h", _F32)
+        self._need(h, "h")
         self._need(rows, "rows", _I32, (r,))
         self._need(weight, "weight", out.dtype, (hid,))
         self._need(out, "out", None, (r, hid))
         splits = self._product(delta, "delta", out.dtype, t, hid) if delta is not None else 0
-        self._run("egpt_add_rmsnorm", h.data_ptr(), self._ptr(delta), splits, t, rows.data_ptr(), weight.data_ptr(),
-                  float(eps), out.data_ptr(), r, hid, dt, self._stream())
+        self._run("egpt_add_rmsnorm", h.data_ptr(), self._fixed(h, "h"), self._ptr(delta), splits, t, rows.data_ptr(),
+                  weight.data_ptr(), float(eps), out.data_ptr(), r, hid, dt, self._stream())
 
     @staticmethod
     def _library_rows(m: int, n: int, k: int) -> bool:
@@ -227,7 +253,7 @@ class HipKernels(KernelBackend):
                 # weight-streaming MFMA kernel (a very wide output with more than one tile of rows: workgroups
                 # of 8 wavefronts stage x half as often)
                 self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), self._ptr(bias),
-                          out.data_ptr() if to_f32 else None, None if to_f32 else out.data_ptr(), m, n, k, 1,
+                          out.data_ptr() if to_f32 else None, None if to_f32 else out.data_ptr(), None, m, n, k, 1,
                           8 if (m > 16 and n >= 65536) else 4, self._stream())
                 return out
             # many rows: the library's matrix product; float32 output (logits) unrounded
@@ -312,7 +338,10 @@ class HipKernels(KernelBackend):
             return None
         if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
             return None
-        self._need(h, "h", _F32)
+        fixed = self._fixed(h, "h")
+        if fixed and delta is not None:
+            return None                  # a stream in fixed point with something still to add: the norm's own kernel adds it
+        self._need(h, "h")
         self._need(w, "w", _BF16, (n, k))
         self._need(norm_weight, "norm_weight", _BF16, (k,))
         d_splits = 0
@@ -323,14 +352,16 @@ class HipKernels(KernelBackend):
         s, waves = splits or auto_s, waves or auto_w
         out = torch.empty((s, t, n), dtype=_F32, device=h.device)
         ss = torch.empty((s, t), dtype=_F32, device=h.device)
-        h_new = torch.empty_like(h)
-        self._run("egpt_gemm_skinny_norm", h.data_ptr(), h_new.data_ptr(), self._ptr(delta), d_splits,
-                  norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, waves, self._stream())
+        h_new = h if fixed else torch.empty_like(h)      # a stream in fixed point is complete: nothing is added here
+        self._run("egpt_gemm_skinny_norm", h.data_ptr(), fixed, None if fixed else h_new.data_ptr(), self._ptr(delta),
+                  d_splits, norm_weight.data_ptr(), w.data_ptr(), out.data_ptr(), ss.data_ptr(), t, n, k, s, waves,
+                  self._stream())
         return out, ss, h_new
 
-    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=20, waves=None):
+    def product_swiglu(self, gate_up, row_ss, hidden, eps, w, max_splits=20, waves=None, residual=None):
         """swiglu(scale * sum gate_up) w^T for float32 partial sums gate_up [S, T, 2I]; scale is the rows' 1/rms
-        from row_ss [S2, T] (or 1).  Returns float32 partial sums [S3, T, N] or None if not covered."""
+        from row_ss [S2, T] (or 1).  Returns float32 partial sums [S3, T, N] or None if not covered; with a residual
+        stream in fixed point [T, N] the product is added into it instead and the stream is returned."""
         if gate_up.dim() != 3 or gate_up.dtype != _F32 or w.dtype != _BF16:
             return None
         g_splits, t, two_i = gate_up.shape
@@ -355,14 +386,16 @@ class HipKernels(KernelBackend):
             # every workgroup computes its share of x from all of gate_up's partial sums: with few columns,
             # wider workgroups (which share the staged x) do that work fewer times
             waves = 8 if -(-n // 64) * s <= 512 else 4
-        out = torch.empty((s, t, n), dtype=_F32, device=w.device)
+        target = self._residual_target(residual, t, n, s)
+        out = None if target is not None else torch.empty((s, t, n), dtype=_F32, device=w.device)
         self._run("egpt_gemm_skinny_swiglu", gate_up.data_ptr(), int(g_splits), self._ptr(row_ss), ss_splits, int(hidden),
-                  float(eps), w.data_ptr(), out.data_ptr(), t, n, k, s, waves, self._stream())
-        return out
+                  float(eps), w.data_ptr(), self._ptr(out), self._ptr(target), t, n, k, s, waves, self._stream())
+        return out if target is None else target
 
-    def product_attention(self, part_o, part_ml, w, max_splits=None, waves=None):
+    def product_attention(self, part_o, part_ml, w, max_splits=None, waves=None, residual=None):
         """(combined attention output) w^T from the parts of a split attention: part_o [S, T, nq, hd],
-        part_ml [S, T, nq, 2].  Returns float32 partial sums [S2, T, N] or None if not covered."""
+        part_ml [S, T, nq, 2].  Returns float32 partial sums [S2, T, N] or None if not covered; with a residual
+        stream in fixed point [T, N] the product is added into it instead and the stream is returned."""
         a_splits, t, nq, hd = part_o.shape
         n, k = w.shape
         if w.dtype != _BF16 or k != nq * hd or not 0 < t <= self.fused_rows or hd % 8 or a_splits > 64:
@@ -382,10 +415,11 @@ class HipKernels(KernelBackend):
         s = -(-steps // per)
         if -(-per * 128 // hd) + 1 > 8:
             return None
-        out = torch.empty((s, t, n), dtype=_F32, device=w.device)
+        target = self._residual_target(residual, t, n, s)
+        out = None if target is not None else torch.empty((s, t, n), dtype=_F32, device=w.device)
         self._run("egpt_gemm_skinny_attn", part_o.data_ptr(), part_ml.data_ptr(), int(a_splits), int(nq), int(hd),
-                  w.data_ptr(), out.data_ptr(), t, n, s, waves, self._stream())
-        return out
+                  w.data_ptr(), self._ptr(out), self._ptr(target), t, n, s, waves, self._stream())
+        return out if target is None else target
 
     def gate_up_swiglu(self, x, w, groups=None):
         """silu(x Wgate^T) * (x Wup^T) as act [T, I] for w = [Wgate; Wup] ([2I, k]), in one kernel: for 17 to 64
@@ -418,27 +452,29 @@ class HipKernels(KernelBackend):
         self._run("egpt_attention_combine", part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), t * nq, hd,
                   int(a_splits), self._stream())
 
-    def product(self, x, w, unrounded=False):
+    def product(self, x, w, unrounded=False, residual=None):
         """x w^T for a consumer that takes partial sums: returns act [m, n], or float32 [splits, m, n] whose sum
         over splits is the product (few rows in bfloat16: the k range is split over workgroups).  unrounded=True
         asks for float32 also from the many-row library product (as [1, m, n]): for consumers that go on computing
         with the values before they round, such as the bias and rotation of queries and keys, where a rounding
-        in between is the largest single contribution to the bfloat16 error of the logits."""
+        in between is the largest single contribution to the bfloat16 error of the logits.  With a residual stream
+        in fixed point [m, n], a product of few rows is added into it instead and the stream is returned."""
         m, k = x.shape
         n = w.shape[0]
         if x.dtype == _BF16 and m > 0 and k % 8 == 0 and not self._library_rows(m, n, k):
             self._need(x, "x")
             self._need(w, "w", x.dtype, (n, k))
             s = self._n_splits(m, n, k)
+            target = self._residual_target(residual, m, n, s) if m <= self.fused_rows else None
             if m > 16 and n >= 4096:
                 # more than one tile of rows and many columns: the kernel that keeps x in LDS for a k range of up
                 # to 8 steps; as few splits as that allows (none at all for k <= 1024: no partial sums)
                 steps = -(-k // 128)
                 s = -(-steps // 8)
-            out = torch.empty((s, m, n), dtype=_F32, device=x.device)
-            self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, k, s, 4,
-                      self._stream())
-            return out
+            out = None if target is not None else torch.empty((s, m, n), dtype=_F32, device=x.device)
+            self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, self._ptr(out), None, self._ptr(target),
+                      m, n, k, s, 4, self._stream())
+            return out if target is None else target
         if unrounded and x.dtype == _BF16 and m > 0 and k % 8 == 0:
             # many rows: the library's product (the reference uses cuBLAS for every linear layer), written out in
             # float32; it goes on as a single "partial sum" [1, m, n]

@@ -100,6 +100,7 @@ class GQAttention(Mixer):
         # product's staging of x; the rows' 1/rms factor is applied by the epilogue kernel below.
         scale_args = {}
         prod = None
+        pending = x if isinstance(x, PendingNorm) else None
         if isinstance(x, PendingNorm):
             fused = None
             rms = x.rms()
@@ -138,13 +139,16 @@ class GQAttention(Mixer):
                 scale_args = dict(scale_args, cos_sin=cos_sin)
             parts = self._epilogue_and_attention(k, prod, t, width, dtype, device, rot, slots, common, scale_args, ctx,
                                                  cache, attn, want_parts)
+        # the output projection: into the residual stream itself where that takes additions (then nothing is returned)
+        residual = pending.residual() if pending is not None else None
         if parts is not None:
-            out = k.product_attention(parts[0], parts[1], self.w_o)
+            out = k.product_attention(parts[0], parts[1], self.w_o, residual=residual)
             if out is not None:
-                return out
+                return None if out is residual else out
             k.combine_attention(parts[0], parts[1], attn)
         if self.b_o is None:
-            return k.product(attn, self.w_o)            # the residual add that follows sums partial sums up
+            out = k.product(attn, self.w_o, residual=residual)   # else the residual add that follows sums partial sums up
+            return None if out is residual else out
         out = torch.empty((t, self.hidden_size), dtype=dtype, device=device)
         k.linear(attn, self.w_o, self.b_o, out)
         return out

@@ -136,6 +136,13 @@ class PendingNorm:
     def applied(self, h_new: torch.Tensor) -> None:
         self.h_after = h_new
 
+    def residual(self) -> torch.Tensor | None:
+        """The residual stream after the addition (known once `applied` or `materialize` was called), if it is of
+        the kind that a part may add its own output into (64-bit fixed point, `kernels.residual_dtype`): the part
+        passes it to the backend's product as `residual=` and returns None if the product went there."""
+        h = self.h_after
+        return h if h is not None and h.dtype == torch.int64 else None
+
     def materialize(self) -> torch.Tensor:
         x = self.norm.forward(self.h, self.delta)      # adds delta into h in place
         self.h_after = self.h
@@ -167,7 +174,8 @@ class Mixer(Part):
 
     forward(x, ctx, cache, state) -> act [T, H]; x is the normed input act [T, H];
     ctx is the engine's StepContext; cache a CacheView if `cache_need()` is not None;
-    state a StateView if `state_need()` is not None.
+    state a StateView if `state_need()` is not None.  A part that was given a PendingNorm may add its output
+    into that norm's residual stream itself (`PendingNorm.residual()`) and then returns None.
     """
 
     takes_pending_norm = False     # True: forward may be given a PendingNorm instead of x
@@ -183,7 +191,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """forward(x) -> act [T, H] for x act [T, H]; tokens are independent."""
+    """forward(x) -> act [T, H] for x act [T, H]; tokens are independent.  As a mixer, it may add its output into a
+    PendingNorm's residual stream itself and return None."""
 
     takes_pending_norm = False
 
@@ -194,8 +203,9 @@ class FeedForward(Part):
 class Block:
     """Arrangement of one layer's parts around the residual stream.
 
-    forward(h, delta, ctx, cache, state) -> (h', delta'): `h` float32 [T, H] is the residual
-    stream and `delta` the not-yet-added output of the previous layer (None for the first);
+    forward(h, delta, ctx, cache, state) -> (h', delta'): `h` [T, H] is the residual stream (float32, or
+    64-bit fixed point in steps of few tokens: parts never look into it, they hand it to the backend) and
+    `delta` the not-yet-added output of the previous layer (None for the first, or when that layer added it itself);
     h' is the residual stream after this layer's additions but one (it may be `h` updated in
     place, or a new tensor) and delta' this layer's not-yet-added output, so that the
     addition fuses with whatever norm comes next.

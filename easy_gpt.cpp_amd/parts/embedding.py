@@ -31,8 +31,10 @@ class TokenEmbedding(Part):
         self.table = self._to(get(self.prefix + "weight"), "compute", dtype, device)
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        out = torch.empty((token_ids.shape[0], self.hidden_size), dtype=torch.float32, device=token_ids.device)
-        kernels.backend().embed(token_ids, self.table, out)
+        k = kernels.backend()
+        out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device,
+                          dtype=k.residual_dtype(token_ids.shape[0], self.table.dtype))     # the residual stream
+        k.embed(token_ids, self.table, out)
         return out
 
 

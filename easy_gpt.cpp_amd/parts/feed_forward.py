@@ -45,7 +45,14 @@ class SwiGLU(FeedForward):
         k = kernels.backend()
         # With few tokens: the norm folds into the first product's staging of x, and SwiGLU (with the rows'
         # 1/rms factor) into the second's.
+        residual = None
+
+        def down(act):
+            out = k.product(act, self.w_down, residual=residual)     # else added to the residual stream by the next norm
+            return None if out is residual else out
+
         if isinstance(x, PendingNorm):
+            pending = x
             rms = x.rms()
             fused = None
             if rms is not None and self.intermediate_size % 8 == 0:
@@ -53,26 +60,28 @@ class SwiGLU(FeedForward):
             if fused is not None:
                 gate_up, row_ss, h_new = fused
                 x.applied(h_new)
-                out = k.product_swiglu(gate_up, row_ss, self.hidden_size, rms[1], self.w_down)
+                residual = pending.residual()
+                out = k.product_swiglu(gate_up, row_ss, self.hidden_size, rms[1], self.w_down, residual=residual)
                 if out is not None:
-                    return out
+                    return None if out is residual else out
                 # SwiGLU by itself; it applies the rows' pending 1/rms factor
                 act = torch.empty((h_new.shape[0], self.intermediate_size), dtype=self.w_down.dtype, device=h_new.device)
                 k.swiglu(gate_up, act, row_ss=row_ss, hidden=self.hidden_size, eps=rms[1])
-                return k.product(act, self.w_down)
+                return down(act)
             x = x.materialize()
+            residual = pending.residual()
         t = x.shape[0]
         act = k.gate_up_swiglu(x, self.w_gate_up)        # a few dozen tokens: product and activation in one kernel
         if act is not None:
-            return k.product(act, self.w_down)
+            return down(act)
         gate_up = k.product(x, self.w_gate_up)           # act [T, 2I] or float32 partial sums [S, T, 2I]
         if gate_up.dim() == 3:
-            out = k.product_swiglu(gate_up, None, self.hidden_size, 0.0, self.w_down)
+            out = k.product_swiglu(gate_up, None, self.hidden_size, 0.0, self.w_down, residual=residual)
             if out is not None:
-                return out
+                return None if out is residual else out
         act = torch.empty((t, self.intermediate_size), dtype=x.dtype, device=x.device)
         k.swiglu(gate_up, act)
-        return k.product(act, self.w_down)               # added to the residual stream by the next norm
+        return down(act)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

@@ -23,7 +23,7 @@ def _whole(t):
 class EmulatedKernels(KernelBackend):
     name = "emulated"
 
-    def product(self, x, w, unrounded=False):
+    def product(self, x, w, unrounded=False, residual=None):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype)
         self.linear(x, w, None, out)
         return out

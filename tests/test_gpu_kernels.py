@@ -108,7 +108,7 @@ def test_skinny_product_and_partial_sums(k, m, n, kk):
             continue
         for waves in (4, 8, 16):                 # wavefronts per workgroup
             out = torch.full((s, m, n), 7.0, dtype=torch.float32, device=DEV)
-            k._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, m, n, kk, s, waves,
+            k._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), None, out.data_ptr(), None, None, m, n, kk, s, waves,
                    k._stream())
             assert float((out.double().sum(0).cpu() - ref).abs().max()) <= 3e-6 * scale, (s, waves)
     out32 = torch.empty(m, n, dtype=torch.float32, device=DEV)
@@ -209,6 +209,82 @@ def test_consumers_add_partial_sums_up(k):
     assert float((got.double().cpu().view(t, -1, hd) - refq).abs().max()) <= 1.6e-2 * float(refq.abs().max())
     assert torch.equal(kc[0, :, 3, :], got.view(t, -1, hd)[0, nq : nq + nkv])
     assert torch.equal(vc[3, :, :, 2], got.view(t, -1, hd)[3, nq + nkv :])
+
+
+def to_fixed(t):
+    """float32 -> the residual stream's 64-bit fixed point (units of 2^-32), as the kernels convert"""
+    return torch.round(t.double() * 2.0 ** 32).to(torch.int64)
+
+
+def from_fixed(t):
+    return t.double() / 2.0 ** 32
+
+
+@pytest.mark.parametrize("t,hid,inter,nq,hd", [(8, 896, 4864, 14, 64), (1, 200, 328, 5, 40), (16, 1536, 1000, 12, 128),
+                                                (5, 120, 200, 3, 40)])
+def test_residual_stream_in_fixed_point(k, t, hid, inter, nq, hd):
+    # The stream of a step of few tokens is int64 in units of 2^-32.  Embedding and norms read and write it, the
+    # products whose k range is split over workgroups add their parts into it with integer atomics: the sum is
+    # the exact sum of the float32 parts (a float32 times 2^32 is an integer here), the same bits in any order.
+    dtype = torch.bfloat16
+    assert k.residual_dtype(t, dtype) == torch.int64 and k.residual_dtype(t, torch.float32) == torch.float32
+    assert k.residual_dtype(17, dtype) == torch.float32
+    # embedding
+    table = rnd(50, hid, dtype=dtype, seed=1)
+    ids = torch.arange(t, dtype=torch.int32, device=DEV) * 3
+    h = torch.empty(t, hid, dtype=torch.int64, device=DEV)
+    k.embed(ids, table, h)
+    assert torch.equal(h, to_fixed(table[ids.long()].float()))
+    # norm of the stream, with and without something to add (an ordinary tensor, or partial sums), all rows or some
+    nw = (1 + rnd(hid, seed=2, scale=0.1)).to(dtype)
+    parts = rnd(3, t, hid, seed=3)
+    for delta in (None, parts[0].to(dtype), parts):
+        hh = h.clone()
+        out = torch.empty(t, hid, dtype=dtype, device=DEV)
+        k.add_rmsnorm(hh, delta, nw, 1e-6, out)
+        added = 0 if delta is None else (delta.double() if delta.dim() == 2 else delta.double().sum(0))
+        want = from_fixed(h) + added
+        assert float((from_fixed(hh) - want).abs().max()) <= 1e-6 * float(want.abs().max())
+        ref = plain.rms_norm(want.cpu(), nw.double().cpu(), 1e-6)
+        assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+        rows = torch.tensor([t - 1, 0], dtype=torch.int32, device=DEV)
+        out2 = torch.empty(2, hid, dtype=dtype, device=DEV)
+        h_before = h.clone()
+        k.rows_add_rmsnorm(h_before, delta, rows, nw, 1e-6, out2)
+        assert torch.equal(h_before, h)                                       # rows only: the stream is not written
+        assert float((out2.double().cpu() - ref[[t - 1, 0]]).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    # the product with the norm folded in reads the stream as it is: the same as from the float32 stream
+    w = rnd(200, hid, dtype=dtype, seed=4, scale=0.05)
+    hf = from_fixed(h).float()
+    a, b = k.product_normed(h, None, nw, w), k.product_normed(hf, None, nw, w)
+    assert a[2] is h and torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert k.product_normed(h, parts, nw, w) is None                          # something to add: the norm's own kernel
+    # products added into the stream: plain, with SwiGLU folded in, with the attention parts' combination folded in
+    x = rnd(t, inter, dtype=dtype, seed=5)
+    w_down = rnd(hid, inter, dtype=dtype, seed=6, scale=0.05)
+    for run in range(2):                                                       # the same bits every time
+        hh = h.clone()
+        assert k.product(x, w_down, residual=hh) is hh
+        want = from_fixed(h) + k.product(x, w_down).double().sum(0)
+        assert torch.equal(hh, to_fixed(from_fixed(h)) + sum(to_fixed(p) for p in k.product(x, w_down)))
+        assert float((from_fixed(hh) - want).abs().max()) <= 1e-9 * float(want.abs().max())
+    gu = rnd(2, t, 2 * inter, seed=7)
+    if inter % 8 == 0:
+        parts_out = k.product_swiglu(gu, None, hid, 0.0, w_down)
+        hh = h.clone()
+        if parts_out is not None:
+            assert k.product_swiglu(gu, None, hid, 0.0, w_down, residual=hh) is hh
+            assert torch.equal(hh, h + sum(to_fixed(p) for p in parts_out))
+    po = rnd(4, t, nq, hd, seed=8)
+    pml = torch.stack([rnd(4, t, nq, seed=9), 1 + rnd(4, t, nq, seed=10).abs()], dim=-1).contiguous()
+    w_o = rnd(hid, nq * hd, dtype=dtype, seed=11, scale=0.05)
+    parts_out = k.product_attention(po, pml, w_o)
+    if parts_out is not None:
+        hh = h.clone()
+        assert k.product_attention(po, pml, w_o, residual=hh) is hh
+        assert torch.equal(hh, h + sum(to_fixed(p) for p in parts_out))
+    # a stream of another shape, or a float32 one, is not added into: partial sums come back as before
+    assert k.product(x, w_down, residual=hf).dim() == 3
 
 
 @pytest.mark.parametrize("t,hid,n,d_splits", [(1, 896, 1152, 0), (8, 896, 9728, 4), (16, 200, 130, 3), (5, 1536, 2048, 13),
