@@ -95,38 +95,46 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
 def link_floor() -> int:
     """What a chain of dependent kernels costs apart from its work: graphs of 125 links that each do next to nothing
     (every thread one load of what the link before wrote, `trips - 1` further loads that depend on each other, one
-    store), replayed; microseconds per link by number of workgroups and of dependent round trips to memory."""
+    store), replayed; microseconds per link by number of workgroups and of dependent round trips to memory, with
+    the further loads near (within the few kilobytes that the link before wrote: L2) or far (anywhere in 1 GiB: HBM)."""
     import torch
 
     from easy_gpt.cpp_amd import kernels
 
     k = kernels.backend()
     links, table = 125, {}
-    for groups in (1, 64, 256, 1024, 4096):
-        n = groups * 256
-        a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
-        for trips in (1, 2, 3, 5):
-            def chain():
-                src, dst = a, b
-                for _ in range(links):
-                    k.probe_link(src, dst, trips)
-                    src, dst = dst, src
-            chain()
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+    far = 1 << 28                                       # floats: dependent loads that range over 1 GiB miss every cache
+    far_a, far_b = torch.zeros(far, device="cuda"), torch.zeros(far, device="cuda")
+    for where in ("near", "far"):
+        for groups in (1, 64, 256, 1024, 4096):
+            n = groups * 256
+            if where == "near":
+                a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+            else:
+                a, b = far_a, far_b
+            for trips in (1, 2, 3, 5):
+                def chain():
+                    src, dst = a, b
+                    for _ in range(links):
+                        k.probe_link(src, dst, trips, n)
+                        src, dst = dst, src
                 chain()
-            for _ in range(3):
-                graph.replay()
-            torch.cuda.synchronize()
-            reps = 20
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                graph.replay()
-            torch.cuda.synchronize()
-            table[f"wg{groups}_trips{trips}"] = round((time.perf_counter() - t0) / reps / links * 1e6, 3)
-            print(f"[bench] {groups:5d} workgroups, {trips} dependent loads: {table[f'wg{groups}_trips{trips}']:.2f} us a link",
-                  file=sys.stderr, flush=True)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    chain()
+                for _ in range(3):
+                    graph.replay()
+                torch.cuda.synchronize()
+                reps = 20
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    graph.replay()
+                torch.cuda.synchronize()
+                key = f"{where}_wg{groups}_trips{trips}"
+                table[key] = round((time.perf_counter() - t0) / reps / links * 1e6, 3)
+                print(f"[bench] {groups:5d} workgroups, {trips} dependent loads ({where}): {table[key]:.2f} us a link",
+                      file=sys.stderr, flush=True)
     print(json.dumps({"metric": "microseconds per link of a replayed graph of 125 dependent near-empty kernels",
                       "unit": "us", "links": links, "table": table}), flush=True)
     return 0

@@ -121,8 +121,9 @@ int egpt_sample_wide(const float* logits, const float* temperature, const int32_
                      const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab, void* stream);
 
 // Measurement only: one link of a chain of dependent kernels that does next to nothing (see elementwise.hip);
-// in, out float32 [n] (in all zeros), `trips` dependent loads per thread.
-int egpt_probe_link(const float* in, float* out, int n, int trips, void* stream);
+// in, out float32 [span] (in all zeros), one workgroup per 256 of the first n elements, `trips` dependent loads per
+// thread, all but the first anywhere in the span.
+int egpt_probe_link(const float* in, float* out, int n, int trips, int span, void* stream);
 
 #ifdef __cplusplus
 }

@@ -116,7 +116,8 @@ __device__ __forceinline__ void trace_mark(unsigned base, unsigned kernel, unsig
         if (base + wg < trace_cap) {
             unsigned long long* rec = trace_buf + static_cast<size_t>(base + wg) * 5;
             if (phase == 0) rec[0] = (static_cast<unsigned long long>(kernel) << 48) | wg;
-            rec[1 + phase] = wall_clock64();
+            // low words of the wall clock (10 ns) and of the shader clock (cycles): the two together give the clock rate
+            rec[1 + phase] = (wall_clock64() & 0xffffffffull) | (static_cast<unsigned long long>(clock64()) << 32);
         }
     }
     __builtin_amdgcn_sched_barrier(0);

@@ -570,25 +570,26 @@ extern "C" int egpt_rope_table(const int32_t* positions, const float* inv_freq, 
 // ---- a link of a chain of dependent kernels that does next to nothing: what the runtime and the memory system
 // charge a decode step per kernel and per dependent round trip, apart from any useful work.  Thread i reads in[i]
 // (written by the link before), then makes `trips - 1` further loads, each at an address that depends on the value
-// loaded before, and writes out[i].
+// loaded before, and writes out[i].  The further loads range over `span` elements of `in`: a span as small as the
+// grid keeps them in L2, a span of hundreds of megabytes sends every one to another page of HBM.
 namespace egpt {
 __global__ __launch_bounds__(256) void probe_link_kernel(const float* __restrict__ in, float* __restrict__ out, int n,
-                                                         int trips) {
+                                                         int trips, int span) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float v = in[i];
-    int at = i;
+    long at = i;
     for (int r = 1; r < trips; ++r) {
-        at = (at + 4099 + static_cast<int>(v)) % n;       // v is zero throughout, but only the load can tell
+        at = (at * 16 + 1048583 + static_cast<long>(v)) % span;       // v is zero throughout, but only the load can tell
         v += __builtin_nontemporal_load(in + at);
     }
     out[i] = v;
 }
 }  // namespace egpt
 
-extern "C" int egpt_probe_link(const float* in, float* out, int n, int trips, void* stream) {
-    if (!in || !out || n <= 0 || trips < 1) return EGPT_BAD_ARGUMENT;
-    probe_link_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(in, out, n, trips);
+extern "C" int egpt_probe_link(const float* in, float* out, int n, int trips, int span, void* stream) {
+    if (!in || !out || n <= 0 || trips < 1 || span < n) return EGPT_BAD_ARGUMENT;
+    probe_link_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(in, out, n, trips, span);
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

@@ -278,10 +278,10 @@ def test_residual_stream_in_fixed_point(k, t, hid, inter, nq, hd):
     po = rnd(4, t, nq, hd, seed=8)
     pml = torch.stack([rnd(4, t, nq, seed=9), 1 + rnd(4, t, nq, seed=10).abs()], dim=-1).contiguous()
     w_o = rnd(hid, nq * hd, dtype=dtype, seed=11, scale=0.05)
-    parts_out = k.product_attention(po, pml, w_o)
+    parts_out = k.product_attention(po, pml, w_o, max_splits=4)
     if parts_out is not None:
         hh = h.clone()
-        assert k.product_attention(po, pml, w_o, residual=hh) is hh
+        assert k.product_attention(po, pml, w_o, max_splits=4, residual=hh) is hh
         assert torch.equal(hh, h + sum(to_fixed(p) for p in parts_out))
     # a stream of another shape, or a float32 one, is not added into: partial sums come back as before
     assert k.product(x, w_down, residual=hf).dim() == 3
