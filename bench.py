@@ -66,6 +66,8 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
         sched = Scheduler(engine, SchedulerConfig(max_active=SERVE_REQUESTS, max_admit_per_step=8,
                                                   max_tokens_per_step=args.serve_budget,
                                                   prefill_chunk=min(SERVE_CHUNK, args.serve_budget)), eos_token_id=-1)
+        if args.no_lookahead:
+            sched.lookahead = False
         for i, n in enumerate(lens):
             sched.add(Request(f"s{rep}_{i}", torch.randint(0, vocab, (n,), generator=g).tolist(), SamplingParams(greedy=True),
                               max_new_tokens=SERVE_NEW_TOKENS, ignore_eos=True))
@@ -87,7 +89,7 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
         "config": {"model": f"{name} layer sizes", "requests": SERVE_REQUESTS, "prompt_tokens": sum(lens),
                    "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": min(SERVE_CHUNK, args.serve_budget),
                    "max_tokens_per_step": args.serve_budget,
-                   "preemptions": st.preemptions, "sampling": "greedy"},
+                   "preemptions": st.preemptions, "steps_launched_ahead": st.steps_ahead, "sampling": "greedy"},
     }), flush=True)
     return 0
 
@@ -161,6 +163,8 @@ def main() -> int:
     ap.add_argument("--serve", action="store_true",
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
                          "each through the scheduler, prompts in portions of 512 (the mixed serving workload)")
+    ap.add_argument("--no-lookahead", action="store_true",
+                    help="with --serve: the scheduler waits for a step's tokens before it launches the next step")
     ap.add_argument("--link-floor", action="store_true",
                     help="instead of the model: what a link of a chain of dependent, near-empty kernels costs in a graph")
     args = ap.parse_args()

@@ -243,8 +243,24 @@ class Engine:
             cache_location=self.model.cache_location, group_windows=[n.window for n in self.cache.groups],
         )
 
+    # ------------------------------------------------------------------ the next decode step, tokens still on the device
+    @property
+    def supports_lookahead(self) -> bool:
+        return self.use_graphs
+
+    def step_decode_ahead(self, request_ids: Sequence, tokens: torch.Tensor) -> torch.Tensor:
+        """A decode step of one token per request whose token ids the host has not seen yet: `tokens` int32 [B] on
+        the device, row i the next token of request_ids[i] (what the sampler left behind the step before).  The
+        step is queued behind whatever writes `tokens`, so a scheduler can launch it before it waits for that
+        step's tokens, and the GPU goes from one step into the next.  Logits [B, vocab] as from `step`."""
+        if not self.use_graphs:
+            raise RuntimeError("steps are launched ahead only from captured graphs")
+        if tokens.dtype != torch.int32 or tuple(tokens.shape) != (len(request_ids),) or tokens.device != self.device:
+            raise ValueError("tokens must be int32 [number of requests] on the engine's device")
+        return self._step_decode([StepEntry(rid, (0,), (0,)) for rid in request_ids], device_tokens=tokens)
+
     # ------------------------------------------------------------------ one token per request, from a graph
-    def _step_decode(self, entries) -> torch.Tensor:
+    def _step_decode(self, entries, device_tokens: torch.Tensor | None = None) -> torch.Tensor:
         """The step for batches of single tokens that all want their logits: the same model code, captured
         once per (batch size, block-table width) into a device graph and replayed with new metadata.  The
         launch of some two hundred kernels costs more host time than they run on the device; the graph
@@ -289,6 +305,8 @@ class Engine:
         key = (rows, tuple(widths), kv_bound)
         plan = self._plan(self._decode_plans, key, lambda: _DecodePlan(self, rows, widths, kv_bound))
         plan.fill(rcs, tokens)
+        if device_tokens is not None:
+            plan.ctx.token_ids[:b].copy_(device_tokens, non_blocking=True)      # (behind the upload of the metadata)
         logits = self._run(plan)
         self.cache.commit_step(rcs, [1] * b)
         return logits[:b]

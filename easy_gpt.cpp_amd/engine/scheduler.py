@@ -8,6 +8,12 @@ on a FIFO queue and a stack of free slots (/root/reference/src/continuous_batch_
 that is decoding contributes its last token, and what is left of the step's token budget goes to
 prompt portions in arrival order.
 
+Decoding runs one step ahead of the host where it can: while a decode step is on the GPU, the next one (the same
+requests, one token each) is launched behind it with its token ids taken on the device from what the sampler leaves
+there, and only then does the host wait for the first step's tokens.  So the GPU goes from step to step without waiting
+for the host's bookkeeping, and a request that ends on an end token has computed one token too many, which is thrown
+away.  Ends that can be foreseen (the token limit, max_position_embeddings) are not run past.
+
 When pages run out:
   * a request waiting for admission keeps waiting (first in, first out: nobody overtakes it);
   * a prompt portion is cut down to what fits, or skipped for this step;
@@ -84,8 +90,20 @@ class PlannedEntry:
 
 
 @dataclass
+class _Launched:
+    """A step that is on the GPU: what was planned, and the tokens it will give."""
+
+    entries: list
+    tokens: object               # sampling.PendingTokens, or None if no entry of the step samples
+    samplers: list
+    t0: float
+
+
+@dataclass
 class Stats:
     steps: int = 0
+    steps_ahead: int = 0        # decode steps launched before the tokens of the step before them were seen
+    discarded: int = 0          # tokens computed for a request after its end token, and thrown away
     prompt_tokens: int = 0
     decode_tokens: int = 0
     generated: int = 0
@@ -109,6 +127,8 @@ class Scheduler:
         self.done: list[Request] = []
         self.stats = Stats()
         self._serial = 0
+        self.lookahead = bool(getattr(engine, "supports_lookahead", False))
+        self._ahead: _Launched | None = None      # the step after the one being waited for, already launched
 
     # ------------------------------------------------------------------ submitting
     def add(self, request: Request) -> Request:
@@ -124,7 +144,7 @@ class Scheduler:
         return request
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._ahead is not None)
 
     # ------------------------------------------------------------------ deciding
     def _fits_alone(self, r: Request) -> bool:
@@ -278,32 +298,82 @@ class Scheduler:
                 self._preempt(self.running[-1])
 
     # ------------------------------------------------------------------ running
-    def step(self) -> list[Request]:
-        """Plan one step, run it, sample, finish what is done.  Returns the requests that finished."""
-        entries = self.plan()
-        if not entries:
-            return []
+    def _launch(self, entries: list[PlannedEntry]) -> _Launched:
+        """Run a planned step on the engine and start sampling; nothing here waits for the GPU."""
         t0 = time.perf_counter()
         batch = []
         for e in entries:
             toks = e.request.tokens(e.start, e.count)
             batch.append(StepEntry(e.request.request_id, toks, [e.count - 1] if e.samples else []))
         logits = self.engine.step(batch)
-        finished: list[Request] = []
+        return self._launched(entries, logits, t0, 0)
+
+    def _launched(self, entries, logits, t0, ahead: int) -> _Launched:
         samplers = [e for e in entries if e.samples]
         for e in entries:
             e.request.computed += e.count
-            if e.count == 1 and e.request.output and e.samples and e.start >= len(e.request.prompt):
+            if e.count == 1 and (e.request.output or ahead) and e.samples and e.start >= len(e.request.prompt):
                 self.stats.decode_tokens += 1
             else:
                 self.stats.prompt_tokens += e.count
+        tokens = None
         if samplers:
-            tokens = self.sampler.sample(
+            tokens = self.sampler.sample_async(
                 logits, [e.request.params for e in samplers], [e.request.serial for e in samplers],
-                [len(e.request.output) for e in samplers],
+                [len(e.request.output) + ahead for e in samplers],
             )
-            for e, tok in zip(samplers, tokens):
+        return _Launched(entries, tokens, samplers, t0)
+
+    def _launch_ahead(self, now: _Launched) -> _Launched | None:
+        """The step after `now`, if it is certain to be `now`'s requests decoding one token each: nobody waits,
+        every running request is sampled in `now`, none of them ends with that token for a reason known before the
+        token is (its limit of new tokens, max_position_embeddings), and the pages their next tokens need are free.
+        Its token ids are `now`'s sampled tokens, taken on the device."""
+        if not self.lookahead or self.waiting or now.tokens is None:
+            return None
+        entries = now.entries
+        if len(now.samplers) != len(entries) or len(entries) != len(self.running):
+            return None
+        cache = self.cache
+        requests, ps = cache.requests, cache.page_size
+        need = [0] * len(cache.pools)
+        limit = self.engine.max_position
+        for e in entries:
+            r = e.request
+            n_out = len(r.output) + 1                     # with the token that `now` is sampling
+            if n_out >= r.max_new_tokens or len(r.prompt) + n_out >= limit or r.computed != len(r.prompt) + n_out - 1:
+                return None
+            rc = requests[r.request_id]
+            want = (rc.num_tokens + ps) // ps
+            for g, have in enumerate(rc.table_lens):
+                if want > have:
+                    need[g] += want - have
+        if any(n > pool.free_count for n, pool in zip(need, cache.pools)):
+            return None
+        t0 = time.perf_counter()
+        logits = self.engine.step_decode_ahead([e.request.request_id for e in entries], now.tokens.device)
+        nxt = [PlannedEntry(e.request, e.request.computed, 1, True) for e in entries]
+        self.stats.steps_ahead += 1
+        return self._launched(nxt, logits, t0, 1)
+
+    def step(self) -> list[Request]:
+        """One step: plan it and run it (or take the one that was launched ahead), launch the step after it if that
+        can be known, then wait for this step's tokens and finish what is done.  Returns the requests that finished."""
+        now, self._ahead = self._ahead, None
+        if now is None:
+            entries = self.plan()
+            if not entries:
+                return []
+            now = self._launch(entries)
+        self._ahead = self._launch_ahead(now)
+        finished: list[Request] = []
+        if now.samplers:
+            tokens = now.tokens.result()
+            for e, tok in zip(now.samplers, tokens):
                 r = e.request
+                if r.status != "running":
+                    self.stats.discarded += 1           # launched ahead of the end token that finished the request
+                    continue
                 r.output.append(int(tok))
                 self.stats.generated += 1
                 reason = ""
@@ -321,7 +391,7 @@ class Scheduler:
                     self.done.append(r)
                     finished.append(r)
         self.stats.steps += 1
-        self.stats.step_seconds += time.perf_counter() - t0
+        self.stats.step_seconds += time.perf_counter() - now.t0
         self.stats.pages_high_water = max(self.stats.pages_high_water, max(p.high_water for p in self.cache.pools))
         return finished
 

@@ -1,3 +1,3 @@
-from .sampler import Sampler, SamplingParams, uniform_for
+from .sampler import PendingTokens, Sampler, SamplingParams, uniform_for
 
-__all__ = ["Sampler", "SamplingParams", "uniform_for"]
+__all__ = ["PendingTokens", "Sampler", "SamplingParams", "uniform_for"]

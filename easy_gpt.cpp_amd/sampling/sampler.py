@@ -55,6 +55,28 @@ def uniform_for(seed: int, serial: int, n: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class PendingTokens:
+    """Sampled tokens that are still on their way: `device` int32 [R] holds them as soon as the stream gets there
+    (the next step can take its token ids from it without the host ever seeing them), `result()` waits for the copy
+    to the host that was queued right behind the sampling kernel, and for nothing queued after it."""
+
+    def __init__(self, device: torch.Tensor):
+        self.device = device
+        self._host = None
+        self._event = None
+        if device.is_cuda:
+            self._host = torch.empty(device.shape, dtype=device.dtype, pin_memory=True)
+            self._host.copy_(device, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record()
+
+    def result(self) -> list[int]:
+        if self._event is None:
+            return self.device.tolist()
+        self._event.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
@@ -62,6 +84,11 @@ class Sampler:
     def sample(self, logits: torch.Tensor, params: list[SamplingParams], serials: list[int], counts: list[int]) -> list[int]:
         """One token per row of `logits` [R, V]; row r belongs to request serials[r], which has
         produced counts[r] tokens so far."""
+        return self.sample_async(logits, params, serials, counts).result()
+
+    def sample_async(self, logits: torch.Tensor, params: list[SamplingParams], serials: list[int],
+                     counts: list[int]) -> PendingTokens:
+        """The same without waiting for the tokens (`PendingTokens`)."""
         r = logits.shape[0]
         if not (len(params) == len(serials) == len(counts) == r):
             raise ValueError("one SamplingParams, serial and count per row of logits is needed")
@@ -77,4 +104,4 @@ class Sampler:
             topk = torch.tensor([p.top_k for p in params], dtype=torch.int32)
             host = host.to(logits.device)
             k.sample(logits, host[0], topk.to(logits.device), host[1], host[2], out)
-        return out.tolist()
+        return PendingTokens(out)

@@ -564,3 +564,34 @@ def test_temperature_generation_and_preemption(tiny_models):
     assert a == b
     assert again == a              # the seed decides: the same engine gives the same tokens again
     assert other_seed != a         # and another seed other ones (96 draws at temperature 0.8)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_one_step_ahead_of_the_host_gives_the_same_tokens(tiny_models, dtype):
+    # the scheduler launches a decode step before it has seen the tokens of the step before it (the token ids go from
+    # the sampler to the next step on the device); with greedy and with temperature sampling, with requests that end
+    # on an end token (one token too many is computed for them and thrown away) and on their limits, the tokens are
+    # those of a scheduler that waits for every step
+    from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    cfg = TINY["B"][0]
+    eng = engine_for(tiny_models["B"], dtype, max_tokens=2048, max_requests=8)
+    prompts = list(H.make_requests(cfg["vocab_size"], [3, 40, 17, 9, 1], seed=91).values())
+
+    def run(lookahead, eos, params):
+        sched = Scheduler(eng, SchedulerConfig(max_active=8, prefill_chunk=16, max_tokens_per_step=64), eos_token_id=eos)
+        sched.lookahead = lookahead
+        reqs = [sched.add(Request(i, p, params, max_new_tokens=20 + 3 * i)) for i, p in enumerate(prompts)]
+        sched.run()
+        assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+        return [r.output for r in reqs], [r.finish_reason for r in reqs], sched.stats
+
+    for params in (SamplingParams(greedy=True), SamplingParams(temperature=0.9, top_k=50, top_p=0.9, seed=3)):
+        free_run, _, _ = run(False, -1, params)
+        eos = free_run[2][7]                                  # the third request ends on its eighth token (or before)
+        waiting, why_w, st_w = run(False, eos, params)
+        ahead, why_a, st_a = run(True, eos, params)
+        assert ahead == waiting and why_a == why_w and "eos" in why_a and "length" in why_a
+        assert st_w.steps_ahead == 0 and st_a.steps_ahead > 10 and st_a.discarded >= 1
+        assert st_a.generated == st_w.generated == sum(len(o) for o in ahead)

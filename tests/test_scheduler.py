@@ -7,6 +7,7 @@ import torch
 from emulated_kernels import EmulatedKernels
 from easy_gpt.cpp_amd import kernels
 from easy_gpt.cpp_amd.cache import CacheManager
+from easy_gpt.cpp_amd.engine import StepEntry
 from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
 from easy_gpt.cpp_amd.parts import CacheNeed
 from easy_gpt.cpp_amd.sampling import SamplingParams
@@ -58,6 +59,21 @@ class FakeEngine:
             self.cache.commit(rc, len(e.tokens))
         self.cache.check()
         return torch.stack(rows) if rows else None
+
+
+class FakeAheadEngine(FakeEngine):
+    """The same with the entry that takes a decode step's token ids from what the sampler left "on the device"."""
+
+    supports_lookahead = True
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.ahead_steps = 0
+
+    def step_decode_ahead(self, request_ids, tokens):
+        assert tokens.dtype == torch.int32 and tokens.shape == (len(request_ids),)
+        self.ahead_steps += 1
+        return self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(request_ids, tokens.tolist())])
 
 
 def expected_output(prompt, n_new, eos=-1):
@@ -125,6 +141,54 @@ def test_a_first_portion_is_cut_to_the_free_pages_when_every_layer_has_a_window(
     r = s.add(Request("r", list(range(1, 41)), GREEDY, max_new_tokens=5))
     s.run()
     assert r.status == "failed" and "even alone" in r.finish_reason
+
+
+def test_decoding_runs_one_step_ahead_of_the_host():
+    # three requests decode side by side: from the step in which the last prompt ends, every step is launched before
+    # the tokens of the step before it are seen; ends that can be foreseen are not run past, an end token costs one
+    # token that is thrown away, and the outputs are what they are without looking ahead
+    prompts = {"a": [3, 4], "b": [5, 6, 7, 8, 9], "c": [1]}
+    out_b = expected_output(prompts["b"], 12)
+    eos = out_b[6]                                     # b ends on its seventh token
+    plain_outputs = {}
+    for engine_class in (FakeEngine, FakeAheadEngine):
+        eng = engine_class(num_pages=100)
+        s = Scheduler(eng, SchedulerConfig(max_active=4), eos_token_id=eos)
+        reqs = {k: s.add(Request(k, p, GREEDY, max_new_tokens=n, ignore_eos=(k != "b")))
+                for (k, p), n in zip(prompts.items(), (9, 12, 15))}
+        s.run()
+        outs = {k: r.output for k, r in reqs.items()}
+        if engine_class is FakeEngine:
+            plain_outputs = outs
+            assert s.stats.steps_ahead == 0
+            continue
+        assert outs == plain_outputs
+        assert outs["b"] == expected_output(prompts["b"], 12, eos=eos) and reqs["b"].finish_reason == "eos"
+        assert reqs["a"].finish_reason == reqs["c"].finish_reason == "length"
+        assert s.stats.steps_ahead == eng.ahead_steps > 8 and s.stats.discarded == 1
+        # tokens fed per request: the prompt and every output but the last; b one more (the step that was in flight
+        # when its end token was seen); a and c end on their limits, which is never run past
+        fed = {k: sum(n for step in eng.log for rid, n, _ in step if rid == k) for k in prompts}
+        assert fed == {"a": 2 + 8, "b": 5 + len(outs["b"]), "c": 1 + 14}
+        assert s.stats.generated == sum(len(o) for o in outs.values())
+        assert eng.cache.free_pages() == [100] and not eng.cache.requests and not s.has_work()
+
+
+def test_looking_ahead_stops_where_pages_or_the_batch_change():
+    # so few pages that requests are preempted, and requests that join later: steps are launched ahead only while the
+    # batch stays what it is and its next pages are free; the tokens are the same as without looking ahead
+    rng = random.Random(5)
+    prompts = [[rng.randrange(VOCAB) for _ in range(rng.randint(1, 30))] for _ in range(7)]
+    outs = []
+    for engine_class in (FakeEngine, FakeAheadEngine):
+        eng = engine_class(num_pages=24)
+        s = Scheduler(eng, SchedulerConfig(max_active=3, max_admit_per_step=2, max_tokens_per_step=16, prefill_chunk=8))
+        reqs = [s.add(Request(i, p, GREEDY, max_new_tokens=10 + i)) for i, p in enumerate(prompts)]
+        s.run()
+        outs.append([r.output for r in reqs])
+        assert all(r.output == expected_output(r.prompt, 10 + i) for i, r in enumerate(reqs))
+        assert eng.cache.free_pages() == [24]
+    assert outs[0] == outs[1]
 
 
 def test_eos_is_kept_and_stops():
@@ -201,11 +265,12 @@ def test_prompt_portion_is_cut_to_the_free_pages():
 
 
 @pytest.mark.parametrize("seed", range(6))
-def test_random_workloads_finish_with_the_right_tokens(seed):
+@pytest.mark.parametrize("ahead", [False, True])
+def test_random_workloads_finish_with_the_right_tokens(seed, ahead):
     rng = random.Random(seed)
     ps = rng.choice([2, 4, 8])
     # room for the longest request alone (30 + 12 tokens) and a little more, so that pages run short often
-    eng = FakeEngine(num_pages=-(-44 // ps) + rng.randint(0, 10), page_size=ps, max_requests=5)
+    eng = (FakeAheadEngine if ahead else FakeEngine)(num_pages=-(-44 // ps) + rng.randint(0, 10), page_size=ps, max_requests=5)
     cfg = SchedulerConfig(max_active=rng.randint(1, 5), max_admit_per_step=rng.randint(1, 3),
                           max_tokens_per_step=rng.randint(4, 40), prefill_chunk=rng.randint(2, 16))
     s = Scheduler(eng, cfg)
