@@ -6,7 +6,9 @@ and a 2,048-token prefill, for the Qwen2.5-0.5B layer sizes with random weights.
 
 A step is one decode step of the whole batch: the engine's step function on one token per request, greedy
 sampling on the device, and the sampled tokens brought to the host (a server needs them there to detect the
-end of a request).  Prints one JSON line.
+end of a request).  Steps are launched as the scheduler launches them: one step ahead of the host, the token ids
+going from the sampler to the next step on the device (--no-lookahead waits for every step's tokens first).
+Prints one JSON line.
 """
 import argparse
 import json
@@ -164,7 +166,8 @@ def main() -> int:
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
                          "each through the scheduler, prompts in portions of 512 (the mixed serving workload)")
     ap.add_argument("--no-lookahead", action="store_true",
-                    help="with --serve: the scheduler waits for a step's tokens before it launches the next step")
+                    help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
+                         "the decode loop otherwise)")
     ap.add_argument("--link-floor", action="store_true",
                     help="instead of the model: what a link of a chain of dependent, near-empty kernels costs in a graph")
     args = ap.parse_args()
@@ -274,16 +277,31 @@ def main() -> int:
             last.append(sampler.sample(out, [greedy], [0], [0])[0])
         params, serials = [greedy] * batch, list(range(batch))
 
-        def one_step(tokens, n):
-            logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(rids, tokens)])
-            return sampler.sample(logits, params, serials, [n] * batch)      # ends with the tokens on the host
+        # As the scheduler decodes: a step is launched before the host has seen the tokens of the step before it
+        # (its token ids go from the sampler to the step on the device), then the host waits for that earlier step's
+        # tokens.  Every step's tokens reach the host inside the timed region.
+        def launch(pending, n):
+            if pending is None or args.no_lookahead:
+                tokens = last if pending is None else pending.result()
+                logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(rids, tokens)])
+            else:
+                logits = engine.step_decode_ahead(rids, pending.device)
+            return sampler.sample_async(logits, params, serials, [n] * batch)
 
+        pending = None
         for i in range(warmup):
-            last = one_step(last, i)
+            nxt = launch(pending, i)
+            if pending is not None:
+                pending.result()
+            pending = nxt
+        pending.result()
         sync()
         t0 = time.perf_counter()
         for i in range(steps):
-            last = one_step(last, warmup + i)
+            nxt = launch(pending, warmup + i)
+            pending.result()                       # the tokens of the step before, on the host
+            pending = nxt
+        pending.result()
         sync()
         sec = time.perf_counter() - t0
         for rid in rids:
