@@ -144,6 +144,76 @@ def link_floor() -> int:
     return 0
 
 
+def anatomy(args, base: dict, name: str) -> int:
+    """What the kernels of one decode step spend their time on, seen from inside: the step is replayed from its graph
+    with the library's trace build, whose product and decode-attention kernels write the wall clock of four phases per
+    workgroup (start; operands staged or queries made; matrix products done; results stored).  Per kind of kernel,
+    medians over the layers, in microseconds: the gap from the end of the kernel before to the first workgroup's
+    start, the ramp until the last workgroup has started, the phases of the median workgroup, and the span from the
+    first start to the last end.  Timestamps cost a little: the step takes a few per cent longer than in bench runs."""
+    import statistics
+    import tempfile
+
+    import torch
+
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.engine import Engine, StepEntry
+    from easy_gpt.cpp_amd.kernels.hip import HipKernels
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    k = HipKernels(trace=True)
+    kernels.use_backend(k)
+    batch, prefix = args.batch, PREFIX
+    tmp = tempfile.mkdtemp(prefix="egpt_bench_")
+    write_random_model(tmp, base, seed=0, dtype=torch.bfloat16)
+    engine = Engine.from_dir(tmp, dtype="bfloat16", device="cuda:0", page_size=args.page_size,
+                             max_tokens=batch * (prefix + 256) + 2048, max_requests=batch + 1)
+    g = torch.Generator().manual_seed(0)
+    rids = [f"d{i}" for i in range(batch)]
+    for rid in rids:
+        engine.add_request(rid)
+        engine.step([StepEntry(rid, torch.randint(0, base["vocab_size"], (prefix,), generator=g).tolist(), [prefix - 1])])
+    for i in range(6):
+        engine.step([StepEntry(rid, [5 + i], [0]) for rid in rids])
+    buf = k.trace_attach()
+    for rep in range(3):
+        buf.zero_()
+        torch.cuda.synchronize()
+        engine.step([StepEntry(rid, [77 + rep], [0]) for rid in rids])
+        torch.cuda.synchronize()
+    launches = k.trace_records(buf)
+    kinds: dict = {}
+    prev_end, rates = None, []
+    for launch in launches:
+        wgs = [w["us"] for w in launch["workgroups"]]
+        first, last_start = min(w[0] for w in wgs), max(w[0] for w in wgs)
+        end = max(w[3] for w in wgs)
+        med = lambda j: statistics.median(w[j] - w[0] for w in wgs if w[j]) if any(w[j] for w in wgs) else None
+        key = (k.TRACED_KERNELS.get(launch["kernel"], str(launch["kernel"])), len(wgs))
+        kinds.setdefault(key, []).append((first - prev_end if prev_end is not None else 0.0, last_start - first,
+                                          med(1), med(2), med(3), end - first))
+        prev_end = end
+        for w in launch["workgroups"]:
+            if w["us"][3] > w["us"][0] + 0.5:
+                rates.append(((w["cycles"][3] - w["cycles"][0]) & 0xffffffff) / (w["us"][3] - w["us"][0]))
+    rows = []
+    print(f"{'kernel':46s} {'wgs':>5s} {'calls':>5s} | {'gap':>5s} {'ramp':>5s} {'staged':>6s} {'mfma':>5s} {'stored':>6s} {'span':>5s}",
+          file=sys.stderr)
+    for (kind, n_wgs), v in kinds.items():
+        m = [None if any(x[i] is None for x in v) else round(statistics.median(x[i] for x in v), 2) for i in range(6)]
+        rows.append({"kernel": kind, "workgroups": n_wgs, "calls": len(v), "gap": m[0], "ramp": m[1], "staged": m[2],
+                     "mfma": m[3], "stored": m[4], "span": m[5]})
+        f = lambda x: "    -" if x is None else f"{x:5.2f}"
+        print(f"{kind:46s} {n_wgs:5d} {len(v):5d} | {f(m[0])} {f(m[1])} {f(m[2]):>6s} {f(m[3])} {f(m[4]):>6s} {f(m[5])}", file=sys.stderr)
+    marks = [w["us"] for launch in launches for w in launch["workgroups"]]
+    total = max(w[3] for w in marks) - min(w[0] for w in marks)
+    rates.sort()
+    print(json.dumps({"metric": f"anatomy of a decode step at batch {batch} ({name}, prefix {prefix}), microseconds",
+                      "first_start_to_last_end_us": round(total, 1), "shader_clock_mhz": round(rates[len(rates) // 2]),
+                      "kernels": rows}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -168,6 +238,9 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
+    ap.add_argument("--anatomy", action="store_true",
+                    help="instead of timing: one decode step at --batch seen from inside its kernels (the library's trace "
+                         "build, compiled at the first call)")
     ap.add_argument("--link-floor", action="store_true",
                     help="instead of the model: what a link of a chain of dependent, near-empty kernels costs in a graph")
     args = ap.parse_args()
@@ -190,6 +263,8 @@ def main() -> int:
         PREFIX, CONTEXT = args.prefix, args.prefix + 2048
     if args.layers is None:
         args.layers = FULL_LAYERS
+    if args.anatomy:
+        return anatomy(args, dict(base, num_hidden_layers=args.layers), name)
     if args.warmup + args.steps > CONTEXT - PREFIX:
         print(f"--warmup + --steps must stay within the context of {CONTEXT} after a prefix of {PREFIX}")
         return 2

@@ -16,7 +16,7 @@ _F32, _BF16, _I32, _I64 = torch.float32, torch.bfloat16, torch.int32, torch.int6
 _DT = {_F32: 0, _BF16: 1}
 
 
-def _load_library() -> ctypes.CDLL:
+def _load_library(trace: bool = False) -> ctypes.CDLL:
     if not torch.cuda.is_available():
         raise KernelsUnavailable(
             "no GPU is visible to torch; this engine has no CPU path (its kernels are HIP code for gfx950)"
@@ -24,7 +24,7 @@ def _load_library() -> ctypes.CDLL:
     from ..csrc import build
 
     try:
-        path = build.ensure_built()
+        path = build.ensure_trace_built() if trace else build.ensure_built()
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
@@ -67,9 +67,12 @@ class _PinnedStream:
 class HipKernels(KernelBackend):
     name = "hip-gfx950"
 
-    def __init__(self):
-        lib = _load_library()
+    def __init__(self, trace: bool = False):
+        """trace=True loads the library's variant with timestamps from inside the kernels (measurements only:
+        `trace_attach`, `trace_records`)."""
+        lib = _load_library(trace)
         self.lib = lib
+        self.trace = bool(trace)
         self._pinned = None
         vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
         lib.egpt_error_string.restype = ctypes.c_char_p
@@ -105,6 +108,44 @@ class HipKernels(KernelBackend):
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = i
+
+    # ------------------------------------------------------------------ timestamps from inside kernels (trace build)
+    TRACED_FILES = ("gemm_skinny", "attention_mfma")
+    TRACED_KERNELS = {0: "product", 1: "product, norm in front", 2: "product, SwiGLU in front",
+                      3: "product, attention parts combined in front", 5: "decode attention"}
+
+    def trace_attach(self, capacity: int = 1 << 20) -> torch.Tensor:
+        """Attach a buffer of `capacity` records (five int64 each) that the traced kernels write their workgroups'
+        timestamps into; returns it.  Records are numbered in the order of launches since the library was loaded,
+        so a captured graph's kernels keep their records over replays."""
+        if not self.trace:
+            raise RuntimeError("this is not the library's trace build (HipKernels(trace=True))")
+        buf = torch.zeros((capacity, 5), dtype=torch.int64, device="cuda")
+        for name in self.TRACED_FILES:
+            fn = getattr(self.lib, f"egpt_trace_attach_{name}")
+            fn.argtypes, fn.restype = [ctypes.c_void_p, ctypes.c_uint], ctypes.c_int
+            if fn(buf.data_ptr(), capacity) != 0:
+                raise RuntimeError("the trace buffer could not be attached")
+        return buf
+
+    @staticmethod
+    def trace_records(buf: torch.Tensor) -> list[dict]:
+        """The kernel launches that wrote into `buf` since it was last cleared, in order of time: for each its kernel
+        id, and per workgroup the wall clock (microseconds) and shader clock (cycles) of its four phases."""
+        rec = buf.cpu()
+        live = (rec[:, 1] != 0).nonzero().flatten().tolist()
+        rows = rec.tolist()
+        launches, cur = [], None
+        for i in live:
+            tag, *marks = rows[i]
+            kid, wg = (tag >> 48) & 0xffff, tag & 0xffffffff
+            if cur is None or wg == 0 or kid != cur["kernel"]:
+                cur = {"kernel": kid, "workgroups": []}
+                launches.append(cur)
+            cur["workgroups"].append({"us": [(m & 0xffffffff) / 100.0 for m in marks],
+                                      "cycles": [(m >> 32) & 0xffffffff for m in marks]})
+        launches.sort(key=lambda l: min(w["us"][0] for w in l["workgroups"]))
+        return launches
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
