@@ -8,7 +8,8 @@ A step is one decode step of the whole batch: the engine's step function on one 
 sampling on the device, and the sampled tokens brought to the host (a server needs them there to detect the
 end of a request).  Steps are launched as the scheduler launches them: one step ahead of the host, the token ids
 going from the sampler to the next step on the device (--no-lookahead waits for every step's tokens first).
-Prints one JSON line.
+Prints one JSON line.  The default run adds the same quantities at further context lengths and at the 1.5B and 7B
+layer sizes to `points` (see FURTHER_CONTEXTS below; --no-further-points skips them).
 """
 import argparse
 import json
@@ -214,6 +215,161 @@ def anatomy(args, base: dict, name: str) -> int:
     return 0
 
 
+# The further points of the default run, beside decode_b1 and decode_b64.  Each name starts with what differs from the
+# headline shape, then the quantity as there (decode_b<batch>: decoded tokens a second; prefill: tokens a second):
+#   ctx8k_, ctx32k_  the 0.5B sizes with prefixes of 8,192 and 32,640 tokens (prefill: one prompt of that length in one step)
+#   q1p5b_           Qwen2.5-1.5B layer sizes (28 layers, hidden 1536, 12 / 2 heads of 128, intermediate 8960, vocabulary
+#                    151936, tied), prefixes of 2,048 tokens, a 2,048-token prefill
+#   q7b_             Qwen2.5-7B layer sizes (28 layers, hidden 3584, 28 / 4 heads of 128, intermediate 18944, vocabulary
+#                    152064, untied), prefixes of 4,096 tokens, a 2,048-token prefill
+FURTHER_CONTEXTS = (("ctx8k", 8192), ("ctx32k", 32640))
+FURTHER_SHAPES = (("q1p5b", "1.5b"), ("q7b", "7b"))
+FURTHER_WARMUP, FURTHER_STEPS = 4, 32
+
+
+def remove_folder(path: str) -> None:
+    for f in os.listdir(path):
+        os.remove(os.path.join(path, f))
+    os.rmdir(path)
+
+
+def further_points(args, model_dir: str, cfg: dict, g) -> dict:
+    """Decode at batch 1 / 8 / 64 and a prefill at further context lengths (the model in `model_dir`) and at the larger
+    layer sizes (random weights drawn on the GPU), all layers of each model: a flat dict of tokens a second."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.sampling import Sampler
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    points, page = {}, args.page_size
+    warm, steps = FURTHER_WARMUP, FURTHER_STEPS
+    room = 3 * (warm + steps) + page                    # the first request decodes in all three runs
+
+    def rate(label, what, tokens, sec):
+        points[f"{label}_{what}"] = round(tokens / sec, 1)
+        print(f"[bench] {label} {what}: {tokens / sec:.1f} tok/s, {sec / (steps if what != 'prefill' else 1) * 1e3:.3f} ms",
+              file=sys.stderr, flush=True)
+
+    longest = max(p for _, p in FURTHER_CONTEXTS)
+    engine = Engine.from_dir(model_dir, dtype=args.dtype, device="cuda:0", page_size=page,
+                             max_tokens=65 * (-(-(longest + room) // page) * page), max_requests=66,
+                             tune_products=not args.no_tune)
+    sampler = Sampler(engine.device)
+    for label, prefix in FURTHER_CONTEXTS:              # the prefixes are filled once and decoded as 64, 8 and 1
+        rate(label, "prefill", prefix, prefill_seconds(engine, cfg["vocab_size"], prefix, g, reps=3))
+        rids, last = fill_requests(engine, sampler, cfg["vocab_size"], prefix, 64, g)
+        for b in (64, 8, 1):
+            sub = last[:b]
+            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids[:b], sub, warm, steps, args.no_lookahead))
+            last[:b] = sub
+        for rid in rids:
+            engine.finish(rid)
+    del engine, sampler
+    torch.cuda.empty_cache()
+
+    for label, shape in FURTHER_SHAPES:
+        changes, n_layers, prefix = OTHER_SHAPES[shape]
+        other = dict(QWEN25_05B, **changes, num_hidden_layers=n_layers)
+        t0 = time.time()
+        tmp = tempfile.mkdtemp(prefix="egpt_bench_")
+        write_random_model(tmp, other, seed=0, dtype=torch.bfloat16, device="cuda:0")
+        engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page,
+                                 max_tokens=64 * (-(-(prefix + warm + steps) // page) * page) + PREFILL_TOKENS,
+                                 max_requests=65, tune_products=not args.no_tune)
+        remove_folder(tmp)
+        sampler = Sampler(engine.device)
+        print(f"[bench] {label} model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+        rate(label, "prefill", PREFILL_TOKENS, prefill_seconds(engine, other["vocab_size"], PREFILL_TOKENS, g, reps=5))
+        for b in (1, 8, 64):
+            rids, last = fill_requests(engine, sampler, other["vocab_size"], prefix, b, g)
+            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids, last, warm, steps, args.no_lookahead))
+            for rid in rids:
+                engine.finish(rid)
+        del engine, sampler
+        torch.cuda.empty_cache()
+    return points
+
+
+def prefill_seconds(engine, vocab: int, tokens: int, g, reps: int = 10) -> float:
+    """One prompt of `tokens` tokens in one step, logits at its last place: the median of `reps` after one warm-up."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    ids = torch.randint(0, vocab, (tokens,), generator=g).tolist()
+    times = []
+    for rep in range(reps + 1):
+        engine.add_request("prefill")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry("prefill", ids, [tokens - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.finish("prefill")
+    return sorted(times[1:])[len(times[1:]) // 2]
+
+
+def fill_requests(engine, sampler, vocab: int, prefix: int, batch: int, g):
+    """`batch` requests with prefixes of `prefix` random tokens in the cache (untimed); their ids and next tokens."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine import StepEntry
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    greedy = SamplingParams(greedy=True)
+    rids, last = [f"d{i}" for i in range(batch)], []
+    for rid in rids:
+        engine.add_request(rid)
+        p = torch.randint(0, vocab, (prefix,), generator=g).tolist()
+        out = engine.step([StepEntry(rid, p, [prefix - 1])])
+        last.append(sampler.sample(out, [greedy], [0], [0])[0])
+    return rids, last
+
+
+def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_lookahead: bool = False) -> float:
+    """Seconds of `steps` decode steps of the requests `rids` after `warmup` untimed ones.
+
+    As the scheduler decodes: a step is launched before the host has seen the tokens of the step before it (its
+    token ids go from the sampler to the step on the device), then the host waits for that earlier step's tokens.
+    Every step's tokens reach the host inside the timed region."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine import StepEntry
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    batch = len(rids)
+    params, serials = [SamplingParams(greedy=True)] * batch, list(range(batch))
+
+    def launch(pending, n):
+        if pending is None or no_lookahead:
+            tokens = last if pending is None else pending.result()
+            logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(rids, tokens)])
+        else:
+            logits = engine.step_decode_ahead(rids, pending.device)
+        return sampler.sample_async(logits, params, serials, [n] * batch)
+
+    pending = None
+    for i in range(warmup):
+        nxt = launch(pending, i)
+        if pending is not None:
+            pending.result()
+        pending = nxt
+    if pending is not None:
+        last[:] = pending.result()
+    pending = None
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        nxt = launch(pending, warmup + i)
+        if pending is not None:
+            pending.result()                       # the tokens of the step before, on the host
+        pending = nxt
+    last[:] = pending.result()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -230,6 +386,8 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true",
                     help="take the library's first choice for its matrix products instead of the measured one")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--no-further-points", action="store_true",
+                    help="skip the points at 8k and 32k prefixes and at the 1.5B and 7B layer sizes")
     ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
     ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
     ap.add_argument("--serve", action="store_true",
@@ -296,16 +454,16 @@ def main() -> int:
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
                              max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1,
                              tune_products=not args.no_tune)
-    for f in os.listdir(tmp):
-        os.remove(os.path.join(tmp, f))
-    os.rmdir(tmp)
     sampler = Sampler(engine.device)
-    greedy = SamplingParams(greedy=True)
     g = torch.Generator().manual_seed(0)
     print(f"[bench] model ready in {time.time() - t_setup:.1f} s", file=sys.stderr, flush=True)
 
     if args.serve:
+        remove_folder(tmp)
         return serve_workload(engine, name, args, vocab)
+    # the further points stand beside the default run's record only
+    further = not (args.no_points or args.no_further_points or args.shape != "0.5b" or args.prefix is not None
+                   or args.layers != FULL_LAYERS or args.dtype != "bfloat16" or args.batch != 8)
 
     # per-step work of the model, for the rooflines
     layer_weights = (h * (nq + 2 * nkv) * hd + (nq + 2 * nkv) * hd + nq * hd * h + 3 * h * inter + 2 * h) * elem
@@ -317,68 +475,22 @@ def main() -> int:
         attention = 2.0 * t * (t + 1) * hd * nq                                  # QK^T and PV over the causal half
         return layers * (linear + attention) + 2.0 * vocab * h                   # logits at the last place only
 
-    def sync():
-        torch.cuda.synchronize()
-
     # ---------------------------------------------------------------- prefill of 2,048 tokens, one request, one step
     prefill = None
     if not args.no_points or args.prefill_only:
-        ids = torch.randint(0, vocab, (PREFILL_TOKENS,), generator=g).tolist()
-        times = []
-        for rep in range(11):                                  # the first one warms up; the median of ten counts
-            engine.add_request("prefill")
-            sync()
-            t0 = time.perf_counter()
-            engine.step([StepEntry("prefill", ids, [PREFILL_TOKENS - 1])])
-            sync()
-            times.append(time.perf_counter() - t0)
-            engine.finish("prefill")
-        sec = sorted(times[1:])[len(times[1:]) // 2]
+        sec = prefill_seconds(engine, vocab, PREFILL_TOKENS, g)
         prefill = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
                    "frac": round(prefill_flops(PREFILL_TOKENS) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     if args.prefill_only:
         print(json.dumps({"metric": f"prefill tok/s at 2,048 tokens ({name})", "prefill": prefill}), flush=True)
+        remove_folder(tmp)
         return 0
 
     # ---------------------------------------------------------------- decoding at each batch size
     def decode_run(batch: int, warmup: int, steps: int):
-        rids = [f"d{i}" for i in range(batch)]
-        prompts = [torch.randint(0, vocab, (PREFIX,), generator=g).tolist() for _ in rids]
-        last = []
-        for rid, p in zip(rids, prompts):                      # untimed: fill the cache with the prefixes
-            engine.add_request(rid)
-            out = engine.step([StepEntry(rid, p, [PREFIX - 1])])
-            last.append(sampler.sample(out, [greedy], [0], [0])[0])
-        params, serials = [greedy] * batch, list(range(batch))
-
-        # As the scheduler decodes: a step is launched before the host has seen the tokens of the step before it
-        # (its token ids go from the sampler to the step on the device), then the host waits for that earlier step's
-        # tokens.  Every step's tokens reach the host inside the timed region.
-        def launch(pending, n):
-            if pending is None or args.no_lookahead:
-                tokens = last if pending is None else pending.result()
-                logits = engine.step([StepEntry(rid, [tok], [0]) for rid, tok in zip(rids, tokens)])
-            else:
-                logits = engine.step_decode_ahead(rids, pending.device)
-            return sampler.sample_async(logits, params, serials, [n] * batch)
-
-        pending = None
-        for i in range(warmup):
-            nxt = launch(pending, i)
-            if pending is not None:
-                pending.result()
-            pending = nxt
-        pending.result()
-        sync()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            nxt = launch(pending, warmup + i)
-            pending.result()                       # the tokens of the step before, on the host
-            pending = nxt
-        pending.result()
-        sync()
-        sec = time.perf_counter() - t0
+        rids, last = fill_requests(engine, sampler, vocab, PREFIX, batch, g)
+        sec = decode_seconds(engine, sampler, rids, last, warmup, steps, args.no_lookahead)
         for rid in rids:
             engine.finish(rid)
         mean_ctx = PREFIX + warmup + (steps + 1) / 2.0
@@ -420,6 +532,10 @@ def main() -> int:
     if prefill is not None:
         line["prefill"] = prefill
     points = {f"decode_b{b}": round(b * args.steps / results[b][0], 1) for b in batches if b != args.batch}
+    del engine
+    if further:
+        points.update(further_points(args, tmp, cfg, g))
+    remove_folder(tmp)
     if points:
         line["points"] = points
     print(json.dumps(line), flush=True)

@@ -2,7 +2,9 @@
 
 Distributions: matrices, embeddings and biases ~ N(0, 0.02); norm scales ~ 1 + N(0, 0.02).
 Each tensor is drawn from its own generator keyed by (seed, tensor name), so the
-values do not depend on the order in which tensors are made.  (The reference only
+values do not depend on the order in which tensors are made; they do depend on the
+device that draws them (the CPU unless asked otherwise: a GPU draws a large model's
+tensors in seconds, with other values for the same seed).  (The reference only
 has unseeded uniform constructors that nothing uses, /root/reference/src/models/linear.cpp:15-24.)
 """
 from __future__ import annotations
@@ -22,41 +24,42 @@ from .safetensors_io import write_safetensors
 _STD = 0.02
 
 
-def _generator(seed: int, name: str) -> torch.Generator:
+def _generator(seed: int, name: str, device: str = "cpu") -> torch.Generator:
     digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    g = torch.Generator(device="cpu")
+    g = torch.Generator(device=device)
     g.manual_seed(int.from_bytes(digest[:8], "little") & (2**63 - 1))
     return g
 
 
-def random_tensor(spec: ParamSpec, seed: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    g = _generator(seed, spec.name)
+def random_tensor(spec: ParamSpec, seed: int, dtype: torch.dtype = torch.float32, device: str = "cpu") -> torch.Tensor:
+    """The tensor that `spec` declares, drawn on `device` and returned in host memory."""
+    g = _generator(seed, spec.name, device)
     if spec.role == "int_table":
-        return torch.randint(0, 2**15, spec.shape, generator=g, dtype=torch.int32)
-    t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * _STD
+        return torch.randint(0, 2**15, spec.shape, generator=g, dtype=torch.int32, device=device).cpu()
+    t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * _STD
     if spec.role == "norm_scale":
         t = t + 1.0
     if spec.dtype == "float32":
-        return t
-    return t.to(dtype)
+        return t.cpu()
+    return t.to(dtype).cpu()
 
 
-def random_tensors(specs, seed: int, dtype: torch.dtype = torch.float32) -> dict[str, torch.Tensor]:
-    return {s.name: random_tensor(s, seed, dtype) for s in specs}
+def random_tensors(specs, seed: int, dtype: torch.dtype = torch.float32, device: str = "cpu") -> dict[str, torch.Tensor]:
+    return {s.name: random_tensor(s, seed, dtype, device) for s in specs}
 
 
 def write_random_model(
-    model_dir: str, config: Mapping[str, Any], seed: int, dtype: torch.dtype = torch.float32
+    model_dir: str, config: Mapping[str, Any], seed: int, dtype: torch.dtype = torch.float32, device: str = "cpu"
 ) -> str:
     """Write `model_dir/config.json` and `model_dir/model.safetensors` for the architecture that
-    `config` (a config.json mapping) names.  Returns model_dir."""
+    `config` (a config.json mapping) names, its tensors drawn on `device`.  Returns model_dir."""
     arch = resolve_architecture(config)
     typed = arch.config_class.from_dict(config, where="config")
     model = build_model(arch.build_spec(typed))
     os.makedirs(model_dir, exist_ok=True)
     with open(os.path.join(model_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(dict(config), f, indent=1)
-    tensors = random_tensors(model.param_specs(), seed, dtype)
+    tensors = random_tensors(model.param_specs(), seed, dtype, device)
     write_safetensors(
         os.path.join(model_dir, "model.safetensors"), tensors, metadata={"format": "pt", "seed": str(seed)}
     )
