@@ -38,10 +38,10 @@ def qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
                     dict(intermediate_size=cfg.intermediate_size, activation=cfg.hidden_act),
                     prefix=p + "mlp.",
                 ),
-                mixer_norm=PartSpec("rmsnorm", dict(eps=cfg.rms_norm_eps), prefix=p + "input_layernorm."),
-                feed_forward_norm=PartSpec(
-                    "rmsnorm", dict(eps=cfg.rms_norm_eps), prefix=p + "post_attention_layernorm."
-                ),
+                norms={
+                    "mixer": PartSpec("rmsnorm", dict(eps=cfg.rms_norm_eps), prefix=p + "input_layernorm."),
+                    "feed_forward": PartSpec("rmsnorm", dict(eps=cfg.rms_norm_eps), prefix=p + "post_attention_layernorm."),
+                },
             )
         )
     return ModelSpec(

@@ -1,4 +1,4 @@
 from .manager import CacheManager, NoFreeSlot, OutOfPages, RequestCache
-from .storage import KVStorage, StateStorage
+from .storage import PagedStorage, StateStorage
 
-__all__ = ["CacheManager", "KVStorage", "NoFreeSlot", "OutOfPages", "RequestCache", "StateStorage"]
+__all__ = ["CacheManager", "PagedStorage", "NoFreeSlot", "OutOfPages", "RequestCache", "StateStorage"]

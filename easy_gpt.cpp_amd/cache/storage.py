@@ -1,4 +1,4 @@
-"""Device memory behind the cache manager: key/value slabs per group and per-request state records."""
+"""Device memory behind the cache manager: the paged tensors of every group and per-request state records."""
 from __future__ import annotations
 
 import torch
@@ -6,11 +6,12 @@ import torch
 from ..parts.base import StateNeed
 
 
-class KVStorage:
-    """For each group, keys as [slabs, num_pages, n_kv_heads, page_size, head_dim] and values
-    transposed within a page, [slabs, num_pages, n_kv_heads, head_dim, page_size].
+class PagedStorage:
+    """The paged tensors of every cache group: for each group and each tensor its mixers declared
+    (`CacheNeed.tensors`), one allocation [slabs, num_pages, *page_shape], a slab per cache id of the group.
 
-    One head's part of a page is contiguous in both.  A key's features are contiguous (the
+    Attention declares keys [n_kv_heads, page_size, head_dim] and values [n_kv_heads, head_dim, page_size] per
+    page.  One head's part of a page is contiguous in both.  A key's features are contiguous (the
     score product sums over features); a feature's values over the page's tokens are
     contiguous (the output product sums over tokens): each is the order in which the matrix
     cores take their operands, so the attention kernels load them as they lie.  Pages are
@@ -18,27 +19,32 @@ class KVStorage:
 
     def __init__(self, groups, slabs_per_group, num_pages, page_size: int, dtype: torch.dtype, device):
         self.page_size = page_size
-        self.k: list[torch.Tensor] = []
-        self.v: list[torch.Tensor] = []
+        self.tensors: list[dict[str, torch.Tensor]] = []
         for need, n_slabs, pages in zip(groups, slabs_per_group, num_pages):
-            k_shape = (n_slabs, pages, need.n_kv_heads, page_size, need.head_dim)
-            v_shape = (n_slabs, pages, need.n_kv_heads, need.head_dim, page_size)
-            self.k.append(torch.zeros(k_shape, dtype=dtype, device=device))
-            self.v.append(torch.zeros(v_shape, dtype=dtype, device=device))
+            names = [t.name for t in need.tensors]
+            if len(set(names)) != len(names):
+                raise ValueError(f"a cache need names a tensor twice: {names}")
+            self.tensors.append({
+                t.name: torch.zeros((n_slabs, pages, *t.page_shape(page_size)),
+                                    dtype=torch.float32 if t.dtype == "float32" else dtype, device=device)
+                for t in need.tensors
+            })
 
-    def slab(self, group: int, index: int):
-        return self.k[group][index], self.v[group][index]
+    def slab(self, group: int, index: int) -> dict[str, torch.Tensor]:
+        return {name: t[index] for name, t in self.tensors[group].items()}
 
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.k + self.v)
+        return sum(t.numel() * t.element_size() for g in self.tensors for t in g.values())
 
 
 class StateStorage:
-    """One record per request slot for every state id a model declares."""
+    """One record per request slot for every state id a model declares, and one more that belongs to no
+    request (`pad_slot`): rows that pad a step to its graph's size read and write that one."""
 
     def __init__(self, needs: dict[int, StateNeed], max_requests: int, device):
+        self.pad_slot = max_requests
         self.data = {
-            sid: torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+            sid: torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
             for sid, need in needs.items()
         }
 

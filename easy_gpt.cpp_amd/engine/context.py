@@ -54,10 +54,12 @@ class StepContext:
 
     def cache_view(self, cache_id: int, writes: bool) -> CacheView:
         g, j = self.cache_location[cache_id]
-        k, v = self.kv_storage.slab(g, j)
         t = self.groups[g]
-        return CacheView(k, v, self.page_size, t.block_table, t.slots, self.group_windows[g], writes)
+        return CacheView(self.kv_storage.slab(g, j), self.page_size, t.block_table, t.slots, self.group_windows[g], writes)
 
     def state_view(self, state_id: int) -> StateView:
         fresh = [kv == q for kv, q in zip(self.kv_len_host, self.q_len_host)]
-        return StateView(self.state_storage.data[state_id], self.state_slots, self.state_slots_host, fresh)
+        if "fresh_device" not in self.shared:            # a request is new when this step's tokens are all it holds
+            self.shared["fresh_device"] = self.kv_len == self.q_len
+        return StateView(self.state_storage.data[state_id], self.state_slots, self.state_slots_host, fresh,
+                         self.shared["fresh_device"])

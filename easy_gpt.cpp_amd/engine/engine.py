@@ -19,7 +19,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import _ints
-from ..cache import CacheManager, KVStorage, RequestCache, StateStorage
+from ..cache import CacheManager, PagedStorage, RequestCache, StateStorage
 from ..config.registry import load_model_config
 from ..parts.model import Model, build_model
 from ..weights.loader import CheckedWeights
@@ -102,7 +102,7 @@ class Engine:
         # a step that runs from a padded graph (`_step_padded`) put their keys and values.
         self._pad_first_page = int(num_pages)
         self._pad_pages = -(-(self.PAD_TO - 1) // self.page_size)
-        self.kv = KVStorage(
+        self.kv = PagedStorage(
             groups, [len(g.cache_ids) for g in model.cache_groups], [num_pages + self._pad_pages] * len(groups),
             self.page_size, model.dtype, self.device,
         )
@@ -440,6 +440,7 @@ class _PaddedPlan:
         # the device must not be freed)
         self.cache, self.page_size = engine.cache, engine.page_size
         self.pad_first_page, self.pad_pages = engine._pad_first_page, engine._pad_pages
+        self.pad_state_slot = engine.states.pad_slot
         dev = engine.device
         n_groups = len(widths)
         ps = engine.page_size
@@ -501,7 +502,7 @@ class _PaddedPlan:
         q_start[b:] = t_pad
         q_len[b:] = 0
         kv_len[b:] = 0
-        state_slots[b:] = 0
+        state_slots[b:] = self.pad_state_slot
         q_start[b], q_len[b], kv_len[b] = t, pad, pad
         want_rows[: len(want)] = want
         want_rows[len(want) :] = 0
@@ -562,6 +563,7 @@ class _DecodePlan:
         self.c_widths = _ints(self.widths)
         self.cache = engine.cache
         self.pad_page, self.page_size = engine._pad_first_page, ps
+        self.pad_state_slot = engine.states.pad_slot
         self.copied = None           # event after the last host-to-device copy
         self.graph = None
         self.logits = None
@@ -576,7 +578,7 @@ class _DecodePlan:
         tables_changed = self.cache.fill_decode(handles, self.c_widths, self.host_small.data_ptr(),
                                                 self.host_tab.data_ptr(), self.row_state.ctypes.data, rows=rows)
         self.ctx.kv_len_host = [rc.num_tokens + 1 for rc in rcs] + [1] * (rows - b)
-        self.ctx.state_slots_host = [rc.slot for rc in rcs] + [0] * (rows - b)
+        self.ctx.state_slots_host = [rc.slot for rc in rcs] + [self.pad_state_slot] * (rows - b)
         if b < rows:
             # the padding: token 0 at position 0, alone in its context, all on the first slot of the padding's page
             # (the same key and value from every such row)
@@ -587,7 +589,7 @@ class _DecodePlan:
             small[2, b:] = np.arange(b, rows, dtype=np.int32)
             small[3, b:] = 1
             small[4, b:] = 1
-            small[5, b:] = 0
+            small[5, b:] = self.pad_state_slot           # the state record that belongs to no request
             small[6, b:] = np.arange(b, rows, dtype=np.int32)
             small[7:, b:] = self.pad_page * self.page_size
             tab = self.host_tab.numpy()

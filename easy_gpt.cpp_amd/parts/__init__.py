@@ -11,7 +11,9 @@ from .base import (
     FeedForward,
     Mixer,
     Norm,
+    PagedTensor,
     Part,
+    PendingNorm,
     PositionEncoding,
     StateNeed,
     StateView,
@@ -23,7 +25,7 @@ from .spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunSpec
 
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block", "CacheGroup", "CacheNeed",
-    "CacheView", "FeedForward", "LayerSpec", "Mixer", "Model", "ModelSpec", "Norm", "ParamSpec", "Part",
-    "PartSpec", "PositionEncoding", "RunSpec", "StateNeed", "StateView", "build_model", "make_part",
+    "CacheView", "FeedForward", "LayerSpec", "Mixer", "Model", "ModelSpec", "Norm", "PagedTensor", "ParamSpec", "Part",
+    "PartSpec", "PendingNorm", "PositionEncoding", "RunSpec", "StateNeed", "StateView", "build_model", "make_part",
     "register_part",
 ]

@@ -57,7 +57,7 @@ class GQAttention(Mixer):
 
     # ------------------------------------------------------------------ declaration
     def cache_need(self):
-        return CacheNeed(self.n_kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.n_kv_heads, self.head_dim, self.window)
 
     def param_specs(self):
         p, h = self.prefix, self.hidden_size

@@ -20,16 +20,40 @@ from .spec import ParamSpec, PartSpec
 
 # --------------------------------------------------------------------------- needs
 @dataclass(frozen=True)
+class PagedTensor:
+    """One tensor of a paged cache: per token a block of `dims` numbers.  A page holds `page_size` tokens; its
+    block has the shape of `dims` with the token's offset in the page put in as axis `token_axis`.
+    dtype 'compute' is the engine's activation dtype, 'float32' stays."""
+
+    name: str
+    dims: tuple[int, ...]
+    token_axis: int = 0
+    dtype: str = "compute"
+
+    def page_shape(self, page_size: int) -> tuple[int, ...]:
+        if not 0 <= self.token_axis <= len(self.dims):
+            raise ValueError(f"paged tensor '{self.name}': token_axis {self.token_axis} is outside its {len(self.dims)} dims")
+        return (*self.dims[: self.token_axis], page_size, *self.dims[self.token_axis :])
+
+
+@dataclass(frozen=True)
 class CacheNeed:
-    """What a mixer asks of the paged cache: keys and values per token.
+    """What a mixer asks of the paged cache: which tensors it keeps per token, and for how long.
 
     window None: every earlier token stays readable.  window W: a token reads only
     the last W tokens (itself included); pages wholly behind that are given back.
+    Mixers with equal needs share a page pool and a block table per request.
     """
 
-    n_kv_heads: int
-    head_dim: int
+    tensors: tuple[PagedTensor, ...]
     window: int | None = None
+
+    @classmethod
+    def keys_and_values(cls, n_kv_heads: int, head_dim: int, window: int | None = None) -> "CacheNeed":
+        """Attention's cache: keys [n_kv_heads, page_size, head_dim] per page (a key's features contiguous) and
+        values [n_kv_heads, head_dim, page_size] (a feature's values over the page's tokens contiguous): each the
+        order in which the matrix cores take their operands."""
+        return cls((PagedTensor("k", (n_kv_heads, head_dim), 1), PagedTensor("v", (n_kv_heads, head_dim), 2)), window)
 
 
 @dataclass(frozen=True)
@@ -45,34 +69,45 @@ class StateNeed:
 class CacheView:
     """One cache slab as a mixer sees it during a step.
 
-    k            [num_pages, n_kv_heads, page_size, head_dim], act
-    v            [num_pages, n_kv_heads, head_dim, page_size], act (transposed within a page)
+    tensors      by the names of the mixer's `CacheNeed`: each [num_pages, *page_shape]; for attention
+                 k [num_pages, n_kv_heads, page_size, head_dim] and v [num_pages, n_kv_heads, head_dim, page_size]
     block_table  int32 [B, W]: page ids of each request in order (-1 where a page was given back)
     slots        int32 [T]: page * page_size + offset where each token of the step is stored
     """
 
-    k: torch.Tensor
-    v: torch.Tensor
+    tensors: dict[str, torch.Tensor]
     page_size: int
     block_table: torch.Tensor
     slots: torch.Tensor
     window: int | None
     writes: bool = True
 
+    @property
+    def k(self) -> torch.Tensor:
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.tensors["v"]
+
 
 @dataclass
 class StateView:
     """Per-request state records: `data[slot]` belongs to the request that holds `slot`.
 
-    data       [max_requests, *shape]
+    data       [max_requests + 1, *shape]; the last record belongs to no request (rows that pad a step use it)
     slots      int32 [B] slot of each request of the step (device); slots_host the same on the host
     fresh      list[bool]: True where the request has no tokens before this step (state must start anew)
+    fresh_device   the same as a bool tensor [B] on the device.  A mixer whose `forward` reads `slots` and
+               `fresh_device` and neither host list is `graph_safe`: its decode steps replay from a graph, in
+               which the host lists are those of the step that was captured.
     """
 
     data: torch.Tensor
     slots: torch.Tensor
     slots_host: list[int]
     fresh: list[bool]
+    fresh_device: torch.Tensor | None = None
 
 
 # --------------------------------------------------------------------------- part interfaces
@@ -205,20 +240,29 @@ class Block:
 
     forward(h, delta, ctx, cache, state) -> (h', delta'): `h` [T, H] is the residual stream (float32, or
     64-bit fixed point in steps of few tokens: parts never look into it, they hand it to the backend) and
-    `delta` the not-yet-added output of the previous layer (None for the first, or when that layer added it itself);
+    `delta` the not-yet-added output of the previous layer (None for the first, or when that layer added it itself;
+    act [T, H], or float32 partial sums [splits, T, H] of a split product: a norm's kernel adds either);
     h' is the residual stream after this layer's additions but one (it may be `h` updated in
     place, or a new tensor) and delta' this layer's not-yet-added output, so that the
     addition fuses with whatever norm comes next.
     """
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+    norm_slots: tuple[str, ...] = ()     # names of the norms this arrangement places
+    uses_mixer = True
+    uses_feed_forward = True
+
+    def __init__(self, mixer: Mixer | None, feed_forward: FeedForward | None, norms: dict[str, Norm]):
+        if set(norms) != set(self.norm_slots):
+            raise ValueError(f"{type(self).__name__} places the norms {sorted(self.norm_slots)}, the layer gives {sorted(norms)}")
+        if (mixer is not None) != self.uses_mixer or (feed_forward is not None) != self.uses_feed_forward:
+            raise ValueError(f"{type(self).__name__} arranges {'a' if self.uses_mixer else 'no'} mixer and "
+                             f"{'a' if self.uses_feed_forward else 'no'} feed-forward")
         self.mixer = mixer
         self.feed_forward = feed_forward
-        self.mixer_norm = mixer_norm
-        self.feed_forward_norm = feed_forward_norm
+        self.norms = dict(norms)
 
     def parts(self) -> list[Part]:
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        return [p for p in (*(self.norms[s] for s in self.norm_slots), self.mixer, self.feed_forward) if p is not None]
 
     def forward(self, h, delta, ctx, cache, state):
         raise NotImplementedError

@@ -12,7 +12,7 @@ import torch
 
 from .. import kernels
 
-from .base import CacheNeed, StateNeed, make_part
+from .base import BLOCKS, CacheNeed, StateNeed, make_part
 from .spec import ModelSpec, ParamSpec
 
 
@@ -31,15 +31,12 @@ class Model:
         self.embedding = make_part("embedding", spec.embedding, vocab_size=spec.vocab_size, **ctx)
         self.layers = []
         for ls in spec.layers:
-            mixer = make_part("mixer", ls.mixer, **ctx)
-            ff = make_part("feed_forward", ls.feed_forward, **ctx)
-            n1 = make_part("norm", ls.mixer_norm, **ctx)
-            n2 = make_part("norm", ls.feed_forward_norm, **ctx)
-            from .base import BLOCKS
-
             if ls.block not in BLOCKS:
-                raise KeyError(f"unknown block kind '{ls.block}'")
-            self.layers.append(BLOCKS[ls.block](mixer, ff, n1, n2))
+                raise KeyError(f"unknown block kind '{ls.block}' (registered: {', '.join(sorted(BLOCKS)) or 'none'})")
+            mixer = make_part("mixer", ls.mixer, **ctx) if ls.mixer is not None else None
+            ff = make_part("feed_forward", ls.feed_forward, **ctx) if ls.feed_forward is not None else None
+            norms = {slot: make_part("norm", ns, **ctx) for slot, ns in ls.norms.items()}
+            self.layers.append(BLOCKS[ls.block](mixer, ff, norms))
         self.final_norm = make_part("norm", spec.final_norm, **ctx)
         self.output_head = make_part("output_head", spec.output_head, vocab_size=spec.vocab_size, **ctx)
         self.dtype: torch.dtype | None = None
@@ -56,6 +53,10 @@ class Model:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"run order entry {i} names layer {run.layer}, the model has {len(self.layers)}")
             mixer = self.layers[run.layer].mixer
+            if mixer is None:
+                if run.cache is not None or run.state is not None:
+                    raise ValueError(f"run order entry {i}: layer {run.layer} has no mixer, so neither cache nor state")
+                continue
             need = mixer.cache_need()
             if need is None:
                 if run.cache is not None:

@@ -15,7 +15,8 @@ class ParamSpec:
     """One tensor of the weights file.
 
     role    how random weights draw it: 'matrix', 'embedding', 'bias' ~ N(0, 0.02);
-            'norm_scale' ~ 1 + N(0, 0.02); 'int_table' uniform integers
+            'norm_scale' ~ 1 + N(0, 0.02); 'int_table' uniform integers; or any role that was added
+            with `weights.register_role` (a decay in (0, 1), a table of a special form, ...)
     dtype   'compute' (cast to the engine's dtype), 'float32' or 'int32' (kept as stored)
     alt_shapes  other shapes accepted on load (the reference accepts [H, 1] for a
             norm weight, /root/reference/src/models/model_param_validation.cpp:62-74)
@@ -39,13 +40,18 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: a block arrangement with a mixer, a feed-forward and their norms."""
+    """One layer: a block arrangement with the parts it arranges.
+
+    norms   the layer's norms by the slot names that the block arrangement declares (`Block.norm_slots`:
+            'mixer' and 'feed_forward' for the pre-norm block; an arrangement with norms before and after each
+            branch declares four, one with a single shared norm one)
+    mixer, feed_forward   None where the arrangement has no such part (`Block.uses_mixer`, `uses_feed_forward`)
+    """
 
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    mixer: PartSpec | None
+    feed_forward: PartSpec | None
+    norms: Mapping[str, PartSpec] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

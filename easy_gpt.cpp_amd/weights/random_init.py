@@ -1,6 +1,7 @@
 """Random-weights mode: a model folder (config.json, model.safetensors) from a configuration and a seed.
 
-Distributions: matrices, embeddings and biases ~ N(0, 0.02); norm scales ~ 1 + N(0, 0.02).
+Distributions by a tensor's role (`ParamSpec.role`): matrices, embeddings and biases ~ N(0, 0.02); norm scales
+~ 1 + N(0, 0.02); integer tables uniform.  `register_role` adds a role with a distribution of its own.
 Each tensor is drawn from its own generator keyed by (seed, tensor name), so the
 values do not depend on the order in which tensors are made; they do depend on the
 device that draws them (the CPU unless asked otherwise: a GPU draws a large model's
@@ -12,7 +13,7 @@ from __future__ import annotations
 import hashlib
 import json
 import os
-from typing import Any, Mapping
+from typing import Any, Callable, Mapping
 
 import torch
 
@@ -31,15 +32,36 @@ def _generator(seed: int, name: str, device: str = "cpu") -> torch.Generator:
     return g
 
 
+def _normal(shape, g, device):
+    return torch.randn(shape, generator=g, dtype=torch.float32, device=device) * _STD
+
+
+# role -> draw(shape, generator, device): float32 (or, for tensors kept as integers, int32) values on `device`
+ROLES: dict[str, Callable[..., torch.Tensor]] = {
+    "matrix": _normal,
+    "embedding": _normal,
+    "bias": _normal,
+    "norm_scale": lambda shape, g, device: _normal(shape, g, device) + 1.0,
+    "int_table": lambda shape, g, device: torch.randint(0, 2**15, shape, generator=g, dtype=torch.int32, device=device),
+}
+
+
+def register_role(role: str, draw: Callable[..., torch.Tensor], replace: bool = False) -> None:
+    """Add a way to draw random weights: `draw(shape, generator, device)` returns the float32 values of a tensor
+    whose `ParamSpec.role` is `role` (say, decays within (0, 1)).  Parts of another architecture use it for tensors
+    that none of the built-in distributions suits."""
+    if role in ROLES and not replace:
+        raise ValueError(f"role '{role}' is already registered")
+    ROLES[role] = draw
+
+
 def random_tensor(spec: ParamSpec, seed: int, dtype: torch.dtype = torch.float32, device: str = "cpu") -> torch.Tensor:
     """The tensor that `spec` declares, drawn on `device` and returned in host memory."""
-    g = _generator(seed, spec.name, device)
-    if spec.role == "int_table":
-        return torch.randint(0, 2**15, spec.shape, generator=g, dtype=torch.int32, device=device).cpu()
-    t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * _STD
-    if spec.role == "norm_scale":
-        t = t + 1.0
-    if spec.dtype == "float32":
+    if spec.role not in ROLES:
+        raise KeyError(f"tensor '{spec.name}' has the role '{spec.role}', which has no distribution "
+                       f"(registered: {', '.join(sorted(ROLES))}; see register_role)")
+    t = ROLES[spec.role](tuple(spec.shape), _generator(seed, spec.name, device), device)
+    if spec.dtype != "compute" or not t.is_floating_point():
         return t.cpu()
     return t.to(dtype).cpu()
 

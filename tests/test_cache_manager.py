@@ -14,8 +14,8 @@ from easy_gpt.cpp_amd.cache import CacheManager, NoFreeSlot, OutOfPages
 from easy_gpt.cpp_amd.parts import CacheNeed
 from plain_cache import PagePool, SlotPool
 
-FULL = CacheNeed(n_kv_heads=2, head_dim=16, window=None)
-WIN = CacheNeed(n_kv_heads=1, head_dim=32, window=10)
+FULL = CacheNeed.keys_and_values(n_kv_heads=2, head_dim=16, window=None)
+WIN = CacheNeed.keys_and_values(n_kv_heads=1, head_dim=32, window=10)
 
 
 def test_page_pool_take_give_back_and_reuse_order():

@@ -125,13 +125,13 @@ def test_attention_part_whole_and_cut(dtype, nq, nkv, hd, hidden, window, bias, 
         one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
         ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(n), kv_len=one(pos + n), max_q_len=n,
                               max_kv_len=pos + n, shared={}, rows_independent=True)
-        cache = CacheView(kc, vc, ps, table, slots, window, True)
+        cache = CacheView({"k": kc, "v": vc}, ps, table, slots, window, True)
         outs.append(whole(att.forward(x[pos : pos + n].to(DEV), ctx, cache, None)))
         pos += n
     out = torch.cat(outs).cpu()
     assert float((out - ref).abs().max()) <= tol(dtype) * float(ref.abs().max())
     # a reader of the same cache that does not write (another layer's cache): same result for the last portion
-    cache_ro = CacheView(kc, vc, ps, table, slots, window, False)
+    cache_ro = CacheView({"k": kc, "v": vc}, ps, table, slots, window, False)
     kc_before = kc.clone()
     again = whole(att.forward(x[pos - n : pos].to(DEV), ctx, cache_ro, None))
     assert torch.equal(kc, kc_before) and torch.equal(again, outs[-1])
@@ -150,7 +150,7 @@ def test_pre_norm_block(dtype):
     w.update(weights_for(ff, dtype, 2, 0.2))
     w.update(weights_for(n1, dtype, 3))
     w.update(weights_for(n2, dtype, 4))
-    block = BLOCKS["pre_norm"](att, ff, n1, n2)
+    block = BLOCKS["pre_norm"](att, ff, {"mixer": n1, "feed_forward": n2})
     s, ps = 19, 8
     x = torch.randn(s, hidden, generator=torch.Generator().manual_seed(9))
     # plain: a = x + Attn(N1 x); y = a + MLP(N2 a)   (/root/reference/src/models/block.cpp:23-29)
@@ -166,7 +166,7 @@ def test_pre_norm_block(dtype):
     one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
     ctx = SimpleNamespace(positions=positions, q_start=one(0), q_len=one(s), kv_len=one(s), max_q_len=s, max_kv_len=s, shared={},
                           rows_independent=True)
-    h, delta = block.forward(x.to(DEV).clone(), None, ctx, CacheView(kc, vc, ps, table, slots, None, True), None)
+    h, delta = block.forward(x.to(DEV).clone(), None, ctx, CacheView({"k": kc, "v": vc}, ps, table, slots, None, True), None)
     got = h.double().cpu() + whole(delta).cpu()
     assert float((h.double().cpu() - a).abs().max()) <= tol(dtype) * float(a.abs().max())
     assert float((got - y).abs().max()) <= tol(dtype) * float(y.abs().max())

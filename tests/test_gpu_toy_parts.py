@@ -125,21 +125,24 @@ def toy_spec(c: ToyConfig) -> ModelSpec:
     def norm(p):
         return PartSpec("rmsnorm", dict(eps=c.eps), prefix=p)
 
+    def norms(p):
+        return {"mixer": norm(p + "n1."), "feed_forward": norm(p + "n2.")}
+
     def ff(p):
         return PartSpec("swiglu", dict(intermediate_size=2 * c.hidden_size), prefix=p)
 
     attn = dict(n_heads=c.n_heads, n_kv_heads=1, head_dim=c.head_dim, qkv_bias=False, out_bias=True, window=None)
     layers = (
-        LayerSpec("pre_norm", PartSpec("toy_decay", dict(decay=c.decay), "l0.mix."), ff("l0.ff."), norm("l0.n1."), norm("l0.n2.")),
+        LayerSpec("pre_norm", PartSpec("toy_decay", dict(decay=c.decay), "l0.mix."), ff("l0.ff."), norms("l0.")),
         LayerSpec("pre_norm",
                   PartSpec("gq_attention", dict(attn, position=PartSpec("toy_learned_offset", dict(max_position=c.max_position_embeddings), "l1.attn.")), "l1.attn."),
-                  ff("l1.ff."), norm("l1.n1."), norm("l1.n2.")),
+                  ff("l1.ff."), norms("l1.")),
         LayerSpec("pre_norm",
                   PartSpec("gq_attention", dict(attn, position=PartSpec("none", {})), "l2.attn."),
-                  ff("l2.ff."), norm("l2.n1."), norm("l2.n2.")),
+                  ff("l2.ff."), norms("l2.")),
         LayerSpec("pre_norm", PartSpec("toy_decay", dict(decay=c.decay), "l3.mix."),
                   PartSpec("toy_routed", dict(n_experts=c.n_experts, expert_size=c.expert_size, router_scale=c.router_scale), "l3.ff."),
-                  norm("l3.n1."), norm("l3.n2.")),
+                  norms("l3.")),
     )
     # layer 1 runs twice (second time with a cache of its own); layer 2 reads layer 1's first cache and writes none;
     # the routed feed-forward comes last, so that a token whose two best experts nearly tie changes only its own logits
@@ -247,7 +250,7 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_registered, tmp_pa
     d = write_random_model(str(tmp_path / "toy"), TOY_CONFIG, seed=3)
     eng = Engine.from_dir(d, dtype=dtype, device="cuda:0", page_size=4, max_tokens=256, max_requests=3)
     assert len(eng.model.cache_groups) == 1 and eng.model.cache_groups[0].cache_ids == (0, 1)
-    assert list(eng.model.state_needs) == [0, 1] and eng.states.data[0].shape == (3, 48)
+    assert list(eng.model.state_needs) == [0, 1] and eng.states.data[0].shape == (3 + 1, 48)
     w = plain.read_safetensors(os.path.join(d, "model.safetensors"))
     if dtype == "bfloat16":
         w = {k: v.float().to(torch.bfloat16).double() for k, v in w.items()}

@@ -28,7 +28,7 @@ class FakeEngine:
     next = (7 * sum of all tokens so far + position) mod VOCAB, so outputs depend on the whole history."""
 
     def __init__(self, num_pages, page_size=4, max_requests=8, max_position=1000, needs=None):
-        self.cache = CacheManager(needs or [CacheNeed(1, 8)], page_size, num_pages, max_requests)
+        self.cache = CacheManager(needs or [CacheNeed.keys_and_values(1, 8)], page_size, num_pages, max_requests)
         self.max_position = max_position
         self.device = "cpu"
         self.sums = {}
@@ -126,7 +126,7 @@ def test_admission_is_first_in_first_out_and_bounded():
 def test_a_first_portion_is_cut_to_the_free_pages_when_every_layer_has_a_window():
     # a pool of 4 pages of 4 tokens, far smaller than the chunk of 512: every group gives pages back as its window of
     # 6 tokens passes them, so the prompt gets through in portions that the free pages hold; nothing stalls or fails
-    eng = FakeEngine(num_pages=4, needs=[CacheNeed(1, 8, window=6)])
+    eng = FakeEngine(num_pages=4, needs=[CacheNeed.keys_and_values(1, 8, window=6)])
     s = Scheduler(eng, SchedulerConfig(max_active=2, prefill_chunk=512))
     r = s.add(Request("r", list(range(1, 41)), GREEDY, max_new_tokens=5))
     r2 = s.add(Request("r2", list(range(3, 30)), GREEDY, max_new_tokens=4))
@@ -136,7 +136,7 @@ def test_a_first_portion_is_cut_to_the_free_pages_when_every_layer_has_a_window(
     assert eng.log[0] == [("r", 16, [])]                   # the first portion: what four free pages hold
     assert eng.cache.free_pages() == [4]
     # a pool that cannot even hold what one window touches: the request fails alone, with a reason
-    eng = FakeEngine(num_pages=2, needs=[CacheNeed(1, 8, window=6)])
+    eng = FakeEngine(num_pages=2, needs=[CacheNeed.keys_and_values(1, 8, window=6)])
     s = Scheduler(eng, SchedulerConfig())
     r = s.add(Request("r", list(range(1, 41)), GREEDY, max_new_tokens=5))
     s.run()
