@@ -101,7 +101,8 @@ def link_floor() -> int:
     """What a chain of dependent kernels costs apart from its work: graphs of 125 links that each do next to nothing
     (every thread one load of what the link before wrote, `trips - 1` further loads that depend on each other, one
     store), replayed; microseconds per link by number of workgroups and of dependent round trips to memory, with
-    the further loads near (within the few kilobytes that the link before wrote: L2) or far (anywhere in 1 GiB: HBM)."""
+    the further loads near (within the few kilobytes that the link before wrote: L2) or far (anywhere in 1 GiB: HBM).
+    Then the same chain with flags in memory in place of kernel boundaries."""
     import torch
 
     from easy_gpt.cpp_amd import kernels
@@ -140,8 +141,53 @@ def link_floor() -> int:
                 table[key] = round((time.perf_counter() - t0) / reps / links * 1e6, 3)
                 print(f"[bench] {groups:5d} workgroups, {trips} dependent loads ({where}): {table[key]:.2f} us a link",
                       file=sys.stderr, flush=True)
+    # The same chain with its links handed over through flags in memory: the links alternate between two streams of
+    # one graph (two hardware queues), so a link is resident and waiting while the link before runs; its first thread
+    # polls the flag past the caches, then all threads read what the link before wrote past the caches.
+    del far_a, far_b
+    side = torch.cuda.Stream()
+    main = torch.cuda.Stream()
+    links = 124
+    for groups in (1, 64, 128, 256, 512):
+        n = groups * 256
+        a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+        flags = torch.zeros(links, dtype=torch.int32, device="cuda")
+        gave_up = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+        def chain():
+            first = torch.cuda.current_stream()
+            flags.zero_()
+            a.zero_()
+            side.wait_stream(first)
+            src, dst = a, b
+            for link in range(links):
+                k.probe_handoff(src, dst, n, flags[link - 1 : link] if link else None, groups, flags[link : link + 1], gave_up,
+                                first if link % 2 == 0 else side)
+                src, dst = dst, src
+            first.wait_stream(side)
+            return src
+
+        with torch.cuda.stream(main):
+            chain()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=main):
+                result = chain()
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            reps = 20
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                graph.replay()
+            torch.cuda.synchronize()
+            us = (time.perf_counter() - t0) / reps / links * 1e6
+        right = float(result.min()) == links and float(result.max()) == links and int(gave_up.item()) == 0
+        table[f"handoff_wg{groups}"] = round(us, 3)
+        print(f"[bench] {groups:5d} workgroups, handed over through a flag, links on two streams in turn: {us:.2f} us a link"
+              f"{'' if right else ' (WRONG RESULT or a wait ran out)'}", file=sys.stderr, flush=True)
     print(json.dumps({"metric": "microseconds per link of a replayed graph of 125 dependent near-empty kernels",
-                      "unit": "us", "links": links, "table": table}), flush=True)
+                      "unit": "us", "links": 125, "table": table}), flush=True)
     return 0
 
 

@@ -594,6 +594,51 @@ extern "C" int egpt_probe_link(const float* in, float* out, int n, int trips, in
     return EGPT_OK;
 }
 
+// Measurement only: the same link, handed over through a flag in memory instead of a kernel boundary, so that a
+// link can be resident (and could have its weights on the way) while the link before still runs.  The first thread of
+// every workgroup waits until `*wait_flag` has reached `wait_count` (the number of workgroups of the link before),
+// with loads that pass the caches and at most `spin_limit` of them: a wait that runs out adds one to `*gave_up` and
+// the workgroup goes on, so that every kernel ends whatever happens.  The threads then read what the link before
+// wrote with loads that pass the caches (one L2 per XCD: a cached copy may be stale), write through them, wait for
+// their stores and add one to `*signal_flag`.
+namespace egpt {
+__global__ __launch_bounds__(256) void probe_handoff_kernel(const float* __restrict__ in, float* __restrict__ out, int n,
+                                                            const unsigned* wait_flag, unsigned wait_count,
+                                                            unsigned* signal_flag, unsigned* gave_up, int spin_limit) {
+    if (threadIdx.x == 0 && wait_flag) {
+        int spins = 0;
+        while (__hip_atomic_load(wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < wait_count) {
+            if (++spins >= spin_limit) {
+                atomicAdd(gave_up, 1u);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+    }
+    __syncthreads();
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = __hip_atomic_load(in + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(out + i, v + 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (signal_flag) {
+        __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have arrived
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(signal_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+}  // namespace egpt
+
+// out[i] = in[i] + 1 for i < n.  wait_flag may be null (no wait), signal_flag may be null (no signal).
+extern "C" int egpt_probe_handoff(const float* in, float* out, int n, const unsigned* wait_flag, unsigned wait_count,
+                                  unsigned* signal_flag, unsigned* gave_up, int spin_limit, void* stream) {
+    if (!in || !out || n <= 0 || !gave_up || spin_limit < 1 || spin_limit > (1 << 22)) return EGPT_BAD_ARGUMENT;
+    probe_handoff_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(in, out, n, wait_flag, wait_count,
+                                                                                       signal_flag, gave_up, spin_limit);
+    EGPT_CHECK_LAUNCH();
+    return EGPT_OK;
+}
+
 #ifdef EGPT_TRACE
 static unsigned g_trace_next = 0;
 extern "C" unsigned egpt_trace_take(unsigned n_workgroups) {
@@ -618,4 +663,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 12; }
+extern "C" int egpt_abi_version(void) { return 13; }

@@ -28,7 +28,7 @@ def _load_library(trace: bool = False) -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 12:
+    if lib.egpt_abi_version() != 13:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -101,6 +101,7 @@ class HipKernels(KernelBackend):
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
             "egpt_probe_link": [vp, vp, i, i, i, vp],
+            "egpt_probe_handoff": [vp, vp, i, vp, ctypes.c_uint, vp, vp, i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -761,6 +762,20 @@ class HipKernels(KernelBackend):
         self._need(src, "src", _F32, (span,))
         self._need(dst, "dst", _F32, (span,))
         self._run("egpt_probe_link", src.data_ptr(), dst.data_ptr(), n, int(trips), span, self._stream())
+
+    def probe_handoff(self, src, dst, n, wait_flag, wait_count, signal_flag, gave_up, stream, spin_limit=200_000):
+        """Measurement only: dst[:n] = src[:n] + 1 on `stream`, started once `wait_flag` (uint32 [1] or None) has reached
+        `wait_count`, and adding one per workgroup to `signal_flag` (or None) when done.  A wait that runs out after
+        `spin_limit` looks adds to `gave_up` and goes on."""
+        self._need(src, "src", _F32)
+        self._need(dst, "dst", _F32)
+        for name, t in (("wait_flag", wait_flag), ("signal_flag", signal_flag), ("gave_up", gave_up)):
+            if t is not None:
+                self._need(t, name, _I32, (1,))
+        if n > min(src.shape[0], dst.shape[0]):
+            raise ValueError("n is beyond the tensors")
+        self._run("egpt_probe_handoff", src.data_ptr(), dst.data_ptr(), int(n), self._ptr(wait_flag), int(wait_count),
+                  self._ptr(signal_flag), gave_up.data_ptr(), int(spin_limit), stream.cuda_stream)
 
     def argmax(self, logits, out):
         r, v = logits.shape
