@@ -345,22 +345,28 @@ class HipKernels(KernelBackend):
     fused_rows = 16     # products with a computed x operand take at most this many rows
     normed_rows_cols = 400_000   # rows x columns beyond which the norm is not folded into a product
 
-    @staticmethod
-    def _normed_shape(n: int, k: int) -> tuple[int, int]:
+    # workgroups of the product with the norm folded in that the GPU holds at once, by wavefronts per workgroup: the
+    # kernel's 128 to 136 registers a lane leave a SIMD three wavefronts, so a CU holds three workgroups of four
+    # wavefronts or one wider one (seen in the kernels' own timestamps: of 504 workgroups of eight wavefronts, 280
+    # start at once and the others when those have ended)
+    _normed_resident = {4: 768, 8: 256, 16: 256}
+
+    @classmethod
+    def _normed_shape(cls, n: int, k: int) -> tuple[int, int]:
         """(splits of the k range, wavefronts per workgroup) of the product with the norm folded in.  Two steps of
         128 per workgroup are staged at once, which is the kernel's shortest chain of round trips; one step where
         the matrix is so small that this leaves the GPU short of workgroups.  Every workgroup computes its share
-        of x again, so where the columns allow it workgroups are wide (their wavefronts share the staged x)."""
+        of x again and waits for its first bytes once, so the workgroups should all be resident together: the
+        width whose workgroups need the fewest rounds, and among those the narrowest (measured: 4,608 x 3,584 at
+        8 rows takes 9.7 us with 252 workgroups of 16 wavefronts, 12.2 with 504 of 8; 17,920 x 1,536 is fastest
+        with 420 of 16; the matrices of the 0.5B sizes fit in one round at any width and are fastest at 4)."""
         steps = -(-k // 128)
         per = max(2, -(-steps // 20))
         if -(-n // 64) * -(-steps // per) < 192:
             per = max(1, -(-steps // 20))
         s = -(-steps // per)
-        waves = 4
-        for wide in (16, 8):
-            if -(-n // (16 * wide)) * s >= 400:
-                waves = wide
-                break
+        rounds = {w: -(-(-(-n // (16 * w)) * s) // cls._normed_resident[w]) for w in (4, 8, 16)}
+        waves = min((4, 8, 16), key=lambda w: (rounds[w], w))
         return s, waves
 
     def product_normed(self, h, delta, norm_weight, w, waves=None, splits=None):
