@@ -337,8 +337,10 @@ class HipKernels(KernelBackend):
         # a long k range is worth more workgroups: each one's stream is a chain of steps, one load ahead
         most = 2048 if steps >= 14 else 1024
         # more than one tile of rows: x weighs as much as w in every workgroup and the partial sums more than with
-        # few rows, so fewer, longer ranges (their x travels through registers a step ahead)
-        s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20 if m <= 16 else 10)
+        # few rows, so fewer, longer ranges (their x travels through registers a step ahead); a few more on a small
+        # matrix (measured inside the model at 896 x 4,864: 1.291 -> 1.260 ms a step at batch 24 and 1.790 -> 1.771 at 64
+        # with 13 ranges instead of 10, 1.853 with 19; at 1,536 x 8,960, 13 ranges cost 3 to 7 %)
+        s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20 if m <= 16 else 13 if n * k <= 8 << 20 else 10)
         per = -(-steps // s)
         return -(-steps // per)
 
