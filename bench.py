@@ -307,7 +307,7 @@ def further_points(args, model_dir: str, cfg: dict, g) -> dict:
         rids, last = fill_requests(engine, sampler, cfg["vocab_size"], prefix, 64, g)
         for b in (64, 8, 1):
             sub = last[:b]
-            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids[:b], sub, warm, steps, args.no_lookahead))
+            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids[:b], sub, warm, steps, args.no_lookahead)[0])
             last[:b] = sub
         for rid in rids:
             engine.finish(rid)
@@ -329,7 +329,7 @@ def further_points(args, model_dir: str, cfg: dict, g) -> dict:
         rate(label, "prefill", PREFILL_TOKENS, prefill_seconds(engine, other["vocab_size"], PREFILL_TOKENS, g, reps=5))
         for b in (1, 8, 64):
             rids, last = fill_requests(engine, sampler, other["vocab_size"], prefix, b, g)
-            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids, last, warm, steps, args.no_lookahead))
+            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids, last, warm, steps, args.no_lookahead)[0])
             for rid in rids:
                 engine.finish(rid)
         del engine, sampler
@@ -373,8 +373,9 @@ def fill_requests(engine, sampler, vocab: int, prefix: int, batch: int, g):
     return rids, last
 
 
-def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_lookahead: bool = False) -> float:
-    """Seconds of `steps` decode steps of the requests `rids` after `warmup` untimed ones.
+def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_lookahead: bool = False) -> tuple[float, float]:
+    """Seconds of `steps` decode steps of the requests `rids` after `warmup` untimed ones, and the median time between
+    the arrivals of two steps' tokens on the host.
 
     As the scheduler decodes: a step is launched before the host has seen the tokens of the step before it (its
     token ids go from the sampler to the step on the device), then the host waits for that earlier step's tokens.
@@ -404,16 +405,21 @@ def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_look
     if pending is not None:
         last[:] = pending.result()
     pending = None
+    arrivals = []                                  # when each step's tokens reached the host
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
         nxt = launch(pending, warmup + i)
         if pending is not None:
             pending.result()                       # the tokens of the step before, on the host
+            arrivals.append(time.perf_counter())
         pending = nxt
     last[:] = pending.result()
+    arrivals.append(time.perf_counter())
     torch.cuda.synchronize()
-    return time.perf_counter() - t0
+    sec = time.perf_counter() - t0
+    between = sorted(b - a for a, b in zip(arrivals, arrivals[1:]))
+    return sec, (between[len(between) // 2] if between else sec / steps)
 
 
 def main() -> int:
@@ -536,14 +542,14 @@ def main() -> int:
     # ---------------------------------------------------------------- decoding at each batch size
     def decode_run(batch: int, warmup: int, steps: int):
         rids, last = fill_requests(engine, sampler, vocab, PREFIX, batch, g)
-        sec = decode_seconds(engine, sampler, rids, last, warmup, steps, args.no_lookahead)
+        sec, medians[batch] = decode_seconds(engine, sampler, rids, last, warmup, steps, args.no_lookahead)
         for rid in rids:
             engine.finish(rid)
         mean_ctx = PREFIX + warmup + (steps + 1) / 2.0
         step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
         return sec, step_bytes
 
-    results = {}
+    results, medians = {}, {}
     for b in batches:
         sec, step_bytes = decode_run(b, args.warmup, args.steps)
         results[b] = (sec, step_bytes)
@@ -560,6 +566,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(sec / args.steps * 1e3, 4),
+        "ms_per_step_median": round(medians[args.batch] * 1e3, 4),      # between the arrivals of two steps' tokens on the host
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
