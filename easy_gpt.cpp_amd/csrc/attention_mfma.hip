@@ -925,6 +925,8 @@ static int launch_mfma(const void* qkv, void* out, float* part_o, float* part_ml
     return EGPT_OK;
 }
 
+constexpr int kDecodeLdsMost = 96 * 1024;       // bytes of LDS a workgroup of the decode kernel may ask for
+
 // PF: key blocks per round of loads of a wavefront.  More of them in flight is fewer round trips but more
 // registers; when there are so many workgroups that they must share CUs, fewer registers are worth more.
 template <int HD, int PF>
@@ -935,7 +937,19 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
     dim3 grid(n_seqs, nkv, n_splits);
     size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
     if (fused) lds += 18 * HD * sizeof(bf16_t);          // 16 query heads, the new key and value
-    if (lds > 64 * 1024) return EGPT_UNSUPPORTED_SIZE;
+    if (lds > kDecodeLdsMost) return EGPT_UNSUPPORTED_SIZE;
+    if (lds > 64 * 1024) {
+        // (eight wavefronts at head size 128: more than a kernel may take without being asked; once per instance)
+        static bool raised_fused = false, raised_plain = false;
+        bool& raised = fused ? raised_fused : raised_plain;
+        if (!raised) {
+            const void* fn = fused ? reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, true>)
+                                   : reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, false>);
+            if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsMost) != hipSuccess)
+                return EGPT_UNSUPPORTED_SIZE;
+            raised = true;
+        }
+    }
     FusedQkv fq = fused ? *fused : FusedQkv{};
     fq.trace_base = EGPT_TRACE_TAKE(grid);
     if (fused)

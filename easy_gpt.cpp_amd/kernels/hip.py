@@ -692,6 +692,12 @@ class HipKernels(KernelBackend):
                 n_waves = 0
         if not n_waves:
             n_splits, n_waves = splits_for(4), 4
+            # head size 128: eight wavefronts as well while every workgroup has a CU of its own (its 71 KB of LDS are
+            # asked for at the first launch): a wavefront then has one round of keys, and the fused variant's nine
+            # heads of 64 pairs are made in one pass (measured with 2,048- and 4,096-token contexts: 1.660 -> 1.600 ms
+            # a step at batch 8 and 1.505 -> 1.443 at batch 1 at the 1.5B sizes, 3 % at the 7B sizes)
+            if hd == 128 and pairs * n_splits <= 256:
+                n_waves = 8
         # The kernel's variant with half the loads in flight per round and fewer registers.  Head size 64: always,
         # unless a wavefront walks so many key blocks that the rounds' depth counts (measured: 0.954 -> 0.933 ms a step
         # at batch 8 and 2,048-token contexts, 0.872 -> 0.853 at batch 1, 1.135 -> 1.102 at batch 8 and 8,192 tokens,
