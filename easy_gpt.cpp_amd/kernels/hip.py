@@ -380,11 +380,13 @@ class HipKernels(KernelBackend):
         if w.dtype != _BF16 or not 0 < t <= self.fused_rows or k % 8 or not h.is_cuda:
             return None
         if splits is None and waves is None and (t * n > self.normed_rows_cols or n * k >= 64 << 20
-                                                 or (n * k >= 16 << 20 and t * n > 100_000)):
+                                                 or (n * k >= 16 << 20 and t * n > 150_000)):
             # every workgroup reads its k range of all rows of h and of delta's partial sums: on a matrix this large
             # (or with this many rows and columns) that costs more than a norm kernel of its own (measured on a
             # 37,888 x 3,584 product behind 14 partial sums: 80 us against 6 + 58; on a 17,920 x 1,536 one with 16 rows
-            # 26 us against 5 + 13, and from 6 rows on the separate kernels win there, which they never do on 9,728 x 896)
+            # 26 us against 5 + 13 when the norm still had 19 partial sums to add; with the stream in fixed point, which
+            # it reads as it is, folding wins there up to 8 rows: 1.597 -> 1.552 ms a step of the 1.5B sizes, and loses
+            # at 16: 1.819 -> 1.831; on 9,728 x 896 it always wins)
             return None
         if delta is not None and (delta.dim() != 3 or delta.dtype != _F32):
             return None
