@@ -59,6 +59,24 @@ class KernelBackend:
 
         return torch.float32
 
+    def residual_add(self, h, delta) -> None:
+        """h += delta in place, for a residual stream of either kind: delta act [T, H] or float32 partial sums
+        [S, T, H].  For norms other than the built-in one (whose kernel adds and normalises in one pass): plain
+        tensor arithmetic, so that such a norm need not know how the stream is kept."""
+        import torch
+
+        d = delta.sum(0, dtype=torch.float32) if delta.dim() == 3 else delta.float()
+        if h.dtype == torch.int64:
+            h += torch.round(d.double() * 4294967296.0).to(torch.int64)
+        else:
+            h += d
+
+    def residual_values(self, h):
+        """The residual stream as a float32 tensor [T, H] (a copy if it is kept in fixed point)."""
+        import torch
+
+        return (h.double() * (1.0 / 4294967296.0)).float() if h.dtype == torch.int64 else h
+
     def product(self, x, w, unrounded=False, residual=None):
         """x w^T as act [m, n], or as float32 partial sums [splits, m, n] for a consumer that adds them up; or, given
         a residual stream in fixed point that the backend can add the product into, that stream."""

@@ -135,9 +135,11 @@ class Part:
 
 
 class Norm(Part):
-    """forward(h, delta, out): h += delta (float32, in place, skipped when delta is None);
-    returns norm(h) as act [T, H].  forward_rows does the same for selected rows without
-    writing h back (used for the rows whose logits are wanted)."""
+    """forward(h, delta): h += delta (in place, skipped when delta is None; delta is act [T, H] or float32 partial
+    sums [S, T, H]); returns norm(h) as act [T, H].  forward_rows does the same for selected rows without
+    writing h back (used for the rows whose logits are wanted).  The stream h is float32 or 64-bit fixed point:
+    a norm hands it to the backend (`add_rmsnorm`; or `residual_add` and `residual_values` for a norm that the
+    backend has no kernel for) and never reads it by itself."""
 
     def rms_params(self) -> tuple[torch.Tensor, float] | None:
         """(weight, eps) if this norm is y = x / sqrt(mean(x^2) + eps) * weight, so that a part may fold it into its

@@ -7,7 +7,9 @@ here and run without a change to the framework's files.
     window (a page pool of its own beside attention's, pages given back behind the window);
   * a mixer with per-request state that is graph-safe (it reads the state's slots and freshness from device
     memory), so that its decode steps replay from captured graphs, padding rows included;
-  * a weight whose random values come from a distribution registered here (a decay within (0, 1)).
+  * a weight whose random values come from a distribution registered here (a decay within (0, 1));
+  * a norm that the backend has no kernel for (a layer norm with mean and bias), which reads and adds to the residual
+    stream through the backend whichever way the stream is kept, also inside replayed graphs.
 The toy parts compute with torch on the GPU; they are test equipment, not a model of anyone's."""
 import os
 from dataclasses import dataclass
@@ -18,10 +20,11 @@ import torch
 import helpers as H
 import plain_qwen2 as plain
 from easy_gpt.cpp_amd.config import Architecture, register_architecture, unregister_architecture
+from easy_gpt.cpp_amd import kernels
 from easy_gpt.cpp_amd.parts import (
-    Block, CacheNeed, LayerSpec, Mixer, ModelSpec, PagedTensor, ParamSpec, PartSpec, RunSpec, StateNeed, register_part,
+    Block, CacheNeed, LayerSpec, Mixer, ModelSpec, Norm, PagedTensor, ParamSpec, PartSpec, RunSpec, StateNeed, register_part,
 )
-from easy_gpt.cpp_amd.parts.base import BLOCKS, MIXERS
+from easy_gpt.cpp_amd.parts.base import BLOCKS, MIXERS, NORMS
 from easy_gpt.cpp_amd.weights import random_init, register_role
 
 pytestmark = pytest.mark.gpu
@@ -147,6 +150,46 @@ def channel_decay_plain(xn, w, rate):
     return torch.stack(outs)
 
 
+# --------------------------------------------------------------------------- a norm of another kind
+class MeanVarianceNorm(Norm):
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * w + b, computed in float32."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, hidden_size, eps):
+        self.prefix, self.hidden_size, self.eps = prefix, hidden_size, float(eps)
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + "weight", (self.hidden_size,), role="norm_scale"),
+                ParamSpec(self.prefix + "bias", (self.hidden_size,), role="bias")]
+
+    def load(self, get, dtype, device):
+        self.w = self._to(get(self.prefix + "weight"), "compute", dtype, device)
+        self.b = self._to(get(self.prefix + "bias"), "compute", dtype, device)
+
+    def _norm(self, x):
+        x = x - x.mean(-1, keepdim=True)
+        y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.w.float() + self.b.float()
+        return y.to(self.w.dtype)
+
+    def forward(self, h, delta):
+        k = kernels.backend()
+        if delta is not None:
+            k.residual_add(h, delta)
+        return self._norm(k.residual_values(h))
+
+    def forward_rows(self, h, delta, rows):
+        x = kernels.backend().residual_values(h)[rows.long()]
+        if delta is not None:
+            x = x + (delta.sum(0) if delta.dim() == 3 else delta.float())[rows.long()]
+        return self._norm(x)
+
+
+def mean_variance_norm_plain(x, w, b, eps):
+    x = x - x.mean(-1, keepdim=True)
+    return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w + b
+
+
 # --------------------------------------------------------------------------- two toy architectures
 @dataclass
 class ShapesConfig:
@@ -237,15 +280,17 @@ class GraphStateConfig:
 
 def graph_state_spec(c: GraphStateConfig) -> ModelSpec:
     norm = lambda p: PartSpec("rmsnorm", dict(eps=c.eps_pre), prefix=p)
+    other = lambda p: PartSpec("toy_mean_variance", dict(eps=c.eps_pre), prefix=p)
     ff = lambda p: PartSpec("swiglu", dict(intermediate_size=c.intermediate_size), p)
-    two = lambda p: {"mixer": norm(p + "n1."), "feed_forward": norm(p + "n2.")}
-    layers = (LayerSpec("pre_norm", PartSpec("toy_channel_decay", {}, "l0.mix."), ff("l0.ff."), two("l0.")),
-              LayerSpec("pre_norm", attention_spec(c, "l1.attn."), ff("l1.ff."), two("l1.")))
+    layers = (LayerSpec("pre_norm", PartSpec("toy_channel_decay", {}, "l0.mix."), ff("l0.ff."),
+                        {"mixer": norm("l0.n1."), "feed_forward": norm("l0.n2.")}),
+              LayerSpec("pre_norm", attention_spec(c, "l1.attn."), ff("l1.ff."),
+                        {"mixer": other("l1.n1."), "feed_forward": other("l1.n2.")}))
     return ModelSpec(
         hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
         embedding=PartSpec("token_embedding", {}, "emb."), layers=layers,
         run_order=(RunSpec(0, state=0), RunSpec(1, cache=0)),
-        final_norm=norm("final."), output_head=PartSpec("linear_head", dict(tied=False), "head."),
+        final_norm=other("final."), output_head=PartSpec("linear_head", dict(tied=False), "head."),
     )
 
 
@@ -263,9 +308,10 @@ def graph_state_plain(w, cfg, ids):
     ffn = lambda x, p: plain.swiglu_mlp(x, {k[len(p):]: v for k, v in w.items() if k.startswith(p)}, "")
     x = x + channel_decay_plain(plain.rms_norm(x, w["l0.n1.weight"], eps), w["l0.mix.w.weight"], w["l0.mix.rate"])
     x = x + ffn(plain.rms_norm(x, w["l0.n2.weight"], eps), "l0.ff.")
-    x = x + plain.self_attention_block(plain.rms_norm(x, w["l1.n1.weight"], eps), w, "l1.attn.", acfg, torch.arange(s))
-    x = x + ffn(plain.rms_norm(x, w["l1.n2.weight"], eps), "l1.ff.")
-    return plain.linear(plain.rms_norm(x, w["final.weight"], eps), w["head.weight"])
+    other = lambda x, p: mean_variance_norm_plain(x, w[p + "weight"], w[p + "bias"], eps)
+    x = x + plain.self_attention_block(other(x, "l1.n1."), w, "l1.attn.", acfg, torch.arange(s))
+    x = x + ffn(other(x, "l1.n2."), "l1.ff.")
+    return plain.linear(other(x, "final."), w["head.weight"])
 
 
 @pytest.fixture()
@@ -274,6 +320,7 @@ def toys_registered():
     register_part("block", "toy_mixer_only", MixerOnlyBlock)
     register_part("mixer", "toy_latent_mean", LatentMeanMixer)
     register_part("mixer", "toy_channel_decay", ChannelDecayMixer)
+    register_part("norm", "toy_mean_variance", MeanVarianceNorm)
     register_role("toy_decay_rate", lambda shape, g, device: 0.5 + 0.45 * torch.rand(shape, generator=g, device=device))
     register_architecture(Architecture("ToyShapesForCausalLM", ShapesConfig, shapes_spec, ("toyshapes",)))
     register_architecture(Architecture("ToyGraphStateForCausalLM", GraphStateConfig, graph_state_spec, ("toygraphstate",)))
@@ -284,6 +331,7 @@ def toys_registered():
     BLOCKS.pop("toy_mixer_only")
     MIXERS.pop("toy_latent_mean")
     MIXERS.pop("toy_channel_decay")
+    NORMS.pop("toy_mean_variance")
     random_init.ROLES.pop("toy_decay_rate")
 
 
