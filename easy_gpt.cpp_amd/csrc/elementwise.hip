@@ -144,11 +144,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
     const bool write_back = (rows == nullptr) && (delta != nullptr);
     // a row that the workgroup covers in one pass stays in registers for the second pass (one round trip less)
     const bool one_pass = hidden <= static_cast<int>(blockDim.x) * 8;
-    float kept[8] = {};
+    float kept[8] = {}, kept_w[8] = {};
     float ss = 0.f;
     for (int j = threadIdx.x * 8; j < hidden; j += blockDim.x * 8) {
         float v[8];
         load8_as_float(hrow + j, v);
+        if (one_pass) load8_as_float(weight + j, kept_w);     // with the row's loads, not behind the workgroup's sum
         if (drow) {
             float d[8];
             load8_as_float(drow + j, d);
@@ -172,7 +173,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
         float v[8], w[8];
         if (one_pass) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = kept[i];
+            for (int i = 0; i < 8; ++i) {
+                v[i] = kept[i];
+                w[i] = kept_w[i];
+            }
         } else {
             load8_as_float(hrow + j, v);
             if (drow && !write_back) {
@@ -181,8 +185,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec8_kernel(float* __restrict
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] += d[i];
             }
+            load8_as_float(weight + j, w);
         }
-        load8_as_float(weight + j, w);
         uint4 o;
         o.x = f32_to_bf16_bits(v[0] * inv * w[0]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[1] * inv * w[1])) << 16);
         o.y = f32_to_bf16_bits(v[2] * inv * w[2]) | (static_cast<uint32_t>(f32_to_bf16_bits(v[3] * inv * w[3])) << 16);
