@@ -111,9 +111,10 @@ class HipKernels(KernelBackend):
             fn.restype = i
 
     # ------------------------------------------------------------------ timestamps from inside kernels (trace build)
-    TRACED_FILES = ("gemm_skinny", "attention_mfma")
+    TRACED_FILES = ("gemm_skinny", "attention_mfma", "gemm_gate_up")
     TRACED_KERNELS = {0: "product", 1: "product, norm in front", 2: "product, SwiGLU in front",
-                      3: "product, attention parts combined in front", 5: "decode attention"}
+                      3: "product, attention parts combined in front", 5: "decode attention",
+                      6: "gate/up product with SwiGLU (first wavefront done, all done, stored)"}
 
     def trace_attach(self, capacity: int = 1 << 20) -> torch.Tensor:
         """Attach a buffer of `capacity` records (five int64 each) that the traced kernels write their workgroups'
