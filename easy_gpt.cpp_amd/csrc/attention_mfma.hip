@@ -868,6 +868,18 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __res
                                                               const float* __restrict__ part_ml,
                                                               bf16_t* __restrict__ out, int n_rows, int hd, int n_splits) {
     const int row = blockIdx.x, lane = threadIdx.x;
+    // the first eight splits' parts are asked for together with their weights' inputs, not behind them (a part of a
+    // split without visible keys may hold anything: it is read and then dropped)
+    float first[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const size_t pr = static_cast<size_t>(min(i, n_splits - 1)) * n_rows + row;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int d = lane + r * kWave;
+            first[i][r] = d < hd ? part_o[pr * hd + d] : 0.f;
+        }
+    }
     float m = -INFINITY, l = 0.f;
     if (lane < n_splits) {
         const size_t pr = static_cast<size_t>(lane) * n_rows + row;
@@ -889,7 +901,8 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __res
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int d = lane + r * kWave;
-                v[i][r] = (d < hd && w8[i] != 0.f) ? part_o[pr * hd + d] : 0.f;
+                if (s0 == 0) v[i][r] = w8[i] != 0.f ? first[i][r] : 0.f;
+                else v[i][r] = (d < hd && w8[i] != 0.f) ? part_o[pr * hd + d] : 0.f;
             }
         }
 #pragma unroll
