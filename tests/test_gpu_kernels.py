@@ -45,7 +45,7 @@ def test_embed(k, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hidden,eps,n_rows", [(72, 1e-6, 7), (896, 1e-5, 7), (3000, 1e-2, 7), (896, 1e-6, 70), (3000, 1e-5, 33),
                                                (100, 1e-6, 40), (896, 1e-6, 601), (1536, 1e-5, 512), (2000, 1e-6, 513),
-                                               (2056, 1e-6, 600)])
+                                               (2056, 1e-6, 600), (5000, 1e-6, 7), (4104, 1e-5, 33), (8192, 1e-6, 7)])
 def test_add_rmsnorm(k, dtype, hidden, eps, n_rows):
     h = rnd(n_rows, hidden, seed=1, scale=2.0)
     delta = rnd(n_rows, hidden, dtype=dtype, seed=2)
@@ -62,6 +62,7 @@ def test_add_rmsnorm(k, dtype, hidden, eps, n_rows):
     k.add_rmsnorm(h, None, w, eps, out)
     assert torch.equal(h, h1)
     # rows variant: gathers, adds, does not write back
+    assert n_rows >= 7                                            # the rows picked below exist
     picked = [6, 0, 3] + (list(range(n_rows - 1, -1, -1)) if n_rows >= 33 else [])
     rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
     out3 = torch.empty(len(picked), hidden, dtype=dtype, device=DEV)
