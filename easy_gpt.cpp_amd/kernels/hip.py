@@ -668,17 +668,24 @@ class HipKernels(KernelBackend):
         output projection combines are read by every column of workgroups there, so they stay few."""
         key_blocks = -(-max_kv_len // 32)
         pairs = b * nkv
+        self_most = 64                    # parts that the output projection (or the combining kernel) takes
 
         def splits_for(n_waves, blocks=None):
             per_round = n_waves * (1 if pairs * key_blocks <= 2048 else (blocks or (4 if hd == 64 else 2)))
             wanted = -(-key_blocks // per_round)
-            # the output projection combines up to 8 parts in registers; more only for few requests with contexts
-            # so long that 8 parts would leave every wavefront four rounds or more
-            most = 16 if (combine or (pairs <= 8 and wanted >= 32)) else 8
-            # head size 128: at most two workgroups per CU, beyond which the kernel's variant with fewer loads in
-            # flight runs (measured at the 1.5B sizes, 2,048-token contexts: 2.42 ms a step with 512 workgroups at
-            # batch 32 against 2.63 with 576, 3.20 with 512 at batch 64 against 3.48 with 1,152)
-            room = 2048 if hd == 64 else 512
+            # the output projection combines up to 8 parts in registers; more only behind contexts so long that 8
+            # parts would leave every wavefront four rounds or more, and then up to some 512 workgroups in all: a CU
+            # has only so many bytes on their way, so a long context wants many CUs more than it minds many parts
+            # (measured at the 0.5B sizes with 32,000-token contexts: batch 1 takes 1.119 ms a step with 16 parts,
+            # 0.991 with 32, 0.976 with 64; batch 8 takes 1.919 with 8, 1.588 with 16, 1.513 with 32, 1.673 with 64;
+            # with 8,192-token contexts batch 1 takes 0.888 with 16 and 0.854 with 32, batch 8 is fastest with 8)
+            most = max(8, min(self_most, 512 // pairs)) if wanted >= 32 else 8
+            # as many workgroups as this at most (head size 64, 8,192-token contexts, batch 64: 2.821 ms a step with
+            # 2,048 workgroups, 2.698 with 1,024).  Head size 128: at most two workgroups per CU, beyond which the
+            # kernel's variant with fewer loads in flight runs (measured at the 1.5B sizes, 2,048-token contexts:
+            # 2.42 ms a step with 512 workgroups at batch 32 against 2.63 with 576, 3.20 with 512 at batch 64 against
+            # 3.48 with 1,152)
+            room = 1024 if hd == 64 else 512
             return max(1, min(wanted, most, max(1, room // pairs)))
 
         n_splits = n_waves = 0

@@ -21,7 +21,7 @@ DTYPES = ["float32", "bfloat16"]
 SIZES_0P5B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 896,
     "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
-    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 4096,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 16384,
     "use_sliding_window": False, "hidden_act": "silu", "torch_dtype": "bfloat16",
 }
 VOCAB = SIZES_0P5B["vocab_size"]
@@ -151,4 +151,49 @@ def test_the_benchmarks_shape_decoding_behind_long_prefixes(models_0p5b, dtype):
     for rid in list(reqs):
         eng.finish(rid)
     compare(rows, cfg, w, reqs, tol_of(dtype), f"0.5B sizes {dtype} decoding behind 2,100 tokens")
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_behind_a_long_prefix_splits_the_keys_many_times(models_0p5b, dtype):
+    # one request behind 9,000 tokens decodes alone: its keys are split over more workgroups than the output
+    # projection combines in registers (its wide path); then beside two requests with 3,000-token prefixes
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    model_dir, cfg, w = models_0p5b(dtype)
+    lens = {"long": 9000, "b": 3011, "c": 2990}
+    n_new = 9
+    reqs = {rid: H.make_requests(VOCAB, [n + n_new], seed=64 + i)["r0"] for i, (rid, n) in enumerate(lens.items())}
+    eng = engine_for(model_dir, dtype, max_tokens=9216 + 2 * 3072, max_requests=3)
+    if dtype == "bfloat16":
+        assert kernels.backend()._decode_shape(1, 2, 64, 9216, False)[0] > 16
+    rows, fed = {}, {}
+
+    def prefill(rid):
+        eng.add_request(rid)
+        ids, n, pos = reqs[rid], lens[rid], 0
+        while pos < n:
+            step = min(2048, n - pos)
+            out = eng.step([StepEntry(rid, ids[pos : pos + step], [step - 1] if pos + step == n else [])])
+            pos += step
+        rows[(rid, n - 1)] = out.float().cpu()[0]
+        fed[rid] = n
+
+    def decode(which):
+        out = eng.step([StepEntry(rid, [reqs[rid][fed[rid]]], [0]) for rid in which]).float().cpu()
+        for j, rid in enumerate(which):
+            rows[(rid, fed[rid])] = out[j].clone()
+            fed[rid] += 1
+
+    prefill("long")
+    for _ in range(5):
+        decode(["long"])
+    prefill("b")
+    prefill("c")
+    for _ in range(4):
+        decode(["long", "b", "c"])
+    for rid in reqs:
+        eng.finish(rid)
+    compare(rows, cfg, w, reqs, tol_of(dtype), f"0.5B sizes {dtype} decoding behind 9,000 tokens")
     assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
