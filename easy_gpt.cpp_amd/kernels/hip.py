@@ -706,8 +706,9 @@ class HipKernels(KernelBackend):
             # asked for at the first launch): a wavefront then has one round of keys, and the fused variant's nine
             # heads of 64 pairs are made in one pass (measured with 2,048- and 4,096-token contexts: 1.660 -> 1.600 ms
             # a step at batch 8 and 1.505 -> 1.443 at batch 1 at the 1.5B sizes, 3 % at the 7B sizes)
-            if hd == 128 and pairs * n_splits <= 256:
-                n_waves = 8
+            # (with a key block per wavefront at least: 1.270 -> 1.243 ms a step of eight layers of the 7B sizes at batch 1)
+            if hd == 128 and pairs * min(n_splits, -(-key_blocks // 8)) <= 256:
+                n_splits, n_waves = min(n_splits, -(-key_blocks // 8)), 8
         # The kernel's variant with half the loads in flight per round and fewer registers.  Head size 64: always,
         # unless a wavefront walks so many key blocks that the rounds' depth counts (measured: 0.954 -> 0.933 ms a step
         # at batch 8 and 2,048-token contexts, 0.872 -> 0.853 at batch 1, 1.135 -> 1.102 at batch 8 and 8,192 tokens,
