@@ -36,7 +36,8 @@ def _load_library(trace: bool = False) -> ctypes.CDLL:
 class _FirstChoice:
     """Within it the library's products are its own first choice even where products are chosen by measurement:
     for the products with float32 output, which that measurement does not cover and which run another, slower
-    way while it is on (the 2,048 x 1,152 x 896 product: 32 us against 12)."""
+    way while it is on (the 2,048 x 1,152 x 896 product: 32 us against 12), and for products of a few dozen rows,
+    where it gains nothing and errs now and then."""
 
     def __enter__(self):
         from . import library_tuning
@@ -305,6 +306,16 @@ class HipKernels(KernelBackend):
                     torch.mm(x, w.t(), out_dtype=_F32, out=out)
                 if bias is not None:
                     out += bias
+            elif m <= 64 and n * k < 64 << 20:
+                # a few dozen rows of a matrix that is not large: the library's first choice streams the weights well,
+                # and a measurement of candidates that all take a few microseconds picks a poor one now and then (a
+                # 64 x 17,920 x 1,536 product at 35 us instead of 18, once in a few runs); on 37,888 x 3,584 the
+                # measured choice is the better one every time (51 us against 60)
+                with _FirstChoice():
+                    if bias is None:
+                        torch.mm(x, w.t(), out=out)
+                    else:
+                        torch.addmm(bias, x, w.t(), out=out)
             elif bias is None:
                 torch.mm(x, w.t(), out=out)
             else:
