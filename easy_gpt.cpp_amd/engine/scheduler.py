@@ -129,6 +129,7 @@ class Scheduler:
         self._serial = 0
         self.lookahead = bool(getattr(engine, "supports_lookahead", False))
         self._ahead: _Launched | None = None      # the step after the one being waited for, already launched
+        self._last_end = 0.0                      # when the last step's tokens were there
 
     # ------------------------------------------------------------------ submitting
     def add(self, request: Request) -> Request:
@@ -325,11 +326,14 @@ class Scheduler:
         return _Launched(entries, tokens, samplers, t0)
 
     def _launch_ahead(self, now: _Launched) -> _Launched | None:
-        """The step after `now`, if it is certain to be `now`'s requests decoding one token each: nobody waits,
+        """The step after `now`, if it is certain to be `now`'s requests decoding one token each: nobody waits (or
+        whoever waits cannot be admitted before a running request ends: every slot is taken),
         every running request is sampled in `now`, none of them ends with that token for a reason known before the
         token is (its limit of new tokens, max_position_embeddings), and the pages their next tokens need are free.
         Its token ids are `now`'s sampled tokens, taken on the device."""
-        if not self.lookahead or self.waiting or now.tokens is None:
+        if not self.lookahead or now.tokens is None:
+            return None
+        if self.waiting and len(self.running) < self.config.max_active:
             return None
         entries = now.entries
         if len(now.samplers) != len(entries) or len(entries) != len(self.running):
@@ -373,6 +377,7 @@ class Scheduler:
                 r = e.request
                 if r.status != "running":
                     self.stats.discarded += 1           # launched ahead of the end token that finished the request
+                    self.stats.decode_tokens -= 1       # (counted when it was launched)
                     continue
                 r.output.append(int(tok))
                 self.stats.generated += 1
@@ -391,7 +396,11 @@ class Scheduler:
                     self.done.append(r)
                     finished.append(r)
         self.stats.steps += 1
-        self.stats.step_seconds += time.perf_counter() - now.t0
+        # a step launched ahead starts while the step before it is still being waited for: its time counts from
+        # that step's end, so that the steps' times add up to the time that passed
+        t_end = time.perf_counter()
+        self.stats.step_seconds += t_end - max(now.t0, self._last_end)
+        self._last_end = t_end
         self.stats.pages_high_water = max(self.stats.pages_high_water, max(p.high_water for p in self.cache.pools))
         return finished
 

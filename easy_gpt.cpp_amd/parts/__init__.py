@@ -8,9 +8,11 @@ from .base import (
     Block,
     CacheNeed,
     CacheView,
+    Embedding,
     FeedForward,
     Mixer,
     Norm,
+    OutputHead,
     PagedTensor,
     Part,
     PendingNorm,
@@ -25,7 +27,7 @@ from .spec import LayerSpec, ModelSpec, ParamSpec, PartSpec, RunSpec
 
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block", "CacheGroup", "CacheNeed",
-    "CacheView", "FeedForward", "LayerSpec", "Mixer", "Model", "ModelSpec", "Norm", "PagedTensor", "ParamSpec", "Part",
+    "CacheView", "Embedding", "FeedForward", "LayerSpec", "Mixer", "Model", "ModelSpec", "Norm", "OutputHead", "PagedTensor", "ParamSpec", "Part",
     "PartSpec", "PendingNorm", "PositionEncoding", "RunSpec", "StateNeed", "StateView", "build_model", "make_part",
     "register_part",
 ]

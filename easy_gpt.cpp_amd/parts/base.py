@@ -237,6 +237,34 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Turns a step's tokens into the residual stream.
+
+    forward(ctx) -> [T, H] residual stream (of the type `kernels.residual_dtype` names for this many tokens).  It is
+    handed the whole step context, so an embedding may use more than `ctx.token_ids` (int32 [T]): a learned vector
+    per position would look up `ctx.positions`.  `output_matrix()` is the [V, H] matrix that an output head may tie
+    itself to, or None if this embedding has none to share."""
+
+    def output_matrix(self) -> torch.Tensor | None:
+        return None
+
+    def forward(self, ctx: Any) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class OutputHead(Part):
+    """forward(x) -> float32 logits [R, V] for the normed rows x act [R, H].  `tied` True: the head declares no
+    matrix of its own and is given the embedding's (`tie`) after the weights are loaded."""
+
+    tied = False
+
+    def tie(self, matrix: torch.Tensor) -> None:
+        raise NotImplementedError
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block:
     """Arrangement of one layer's parts around the residual stream.
 

@@ -11,11 +11,11 @@ from __future__ import annotations
 import torch
 
 from .. import kernels
-from .base import Part, register_part
+from .base import Embedding, OutputHead, register_part
 from .spec import ParamSpec
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int):
@@ -30,15 +30,19 @@ class TokenEmbedding(Part):
     def load(self, get, dtype, device):
         self.table = self._to(get(self.prefix + "weight"), "compute", dtype, device)
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def output_matrix(self) -> torch.Tensor:
+        return self.table
+
+    def forward(self, ctx) -> torch.Tensor:
         k = kernels.backend()
+        token_ids = ctx.token_ids
         out = torch.empty((token_ids.shape[0], self.hidden_size), device=token_ids.device,
                           dtype=k.residual_dtype(token_ids.shape[0], self.table.dtype))     # the residual stream
         k.embed(token_ids, self.table, out)
         return out
 
 
-class OutputHead(Part):
+class LinearHead(OutputHead):
     graph_safe = True
 
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied: bool):
@@ -57,8 +61,11 @@ class OutputHead(Part):
         if not self.tied:
             self.weight = self._to(get(self.prefix + "weight"), "compute", dtype, device)
 
-    def tie(self, table: torch.Tensor) -> None:
-        self.weight = table
+    def tie(self, matrix: torch.Tensor) -> None:
+        if tuple(matrix.shape) != (self.vocab_size, self.hidden_size):
+            raise ValueError(f"a tied output head needs a [{self.vocab_size}, {self.hidden_size}] matrix, "
+                             f"got {tuple(matrix.shape)}")
+        self.weight = matrix
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out = torch.empty((x.shape[0], self.vocab_size), dtype=torch.float32, device=x.device)
@@ -67,4 +74,4 @@ class OutputHead(Part):
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)
-register_part("output_head", "linear_head", OutputHead)
+register_part("output_head", "linear_head", LinearHead)

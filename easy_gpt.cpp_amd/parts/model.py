@@ -109,11 +109,14 @@ class Model:
 
     def load(self, get, dtype: torch.dtype, device) -> None:
         """Take every declared tensor through `get(name)` (a checked weights source)."""
-        device = torch.device(device)
+        device = resolve_device(device)
         for p in self.parts():
             p.load(get, dtype, device)
         if getattr(self.output_head, "tied", False):
-            self.output_head.tie(self.embedding.table)
+            matrix = self.embedding.output_matrix()
+            if matrix is None:
+                raise ValueError(f"the output head is tied, but {type(self.embedding).__name__} has no matrix to share")
+            self.output_head.tie(matrix)
         self.dtype, self.device = dtype, device
 
     # ------------------------------------------------------------------ one step
@@ -124,7 +127,7 @@ class Model:
             return self._forward(ctx)
 
     def _forward(self, ctx) -> torch.Tensor | None:
-        h = self.embedding.forward(ctx.token_ids)
+        h = self.embedding.forward(ctx)
         delta = None
         for run in self.spec.run_order:
             block = self.layers[run.layer]
@@ -135,6 +138,15 @@ class Model:
             return None
         x = self.final_norm.forward_rows(h, delta, ctx.want_rows)
         return self.output_head.forward(x)
+
+
+def resolve_device(device) -> torch.device:
+    """`device` as a torch.device with its index spelled out: "cuda" names the current GPU, and tensors made there
+    report "cuda:<index>", which does not compare equal to the unindexed name."""
+    device = torch.device(device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    return device
 
 
 def build_model(spec: ModelSpec) -> Model:

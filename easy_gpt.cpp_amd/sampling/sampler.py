@@ -79,7 +79,9 @@ class PendingTokens:
 
 class Sampler:
     def __init__(self, device):
-        self.device = torch.device(device)
+        from ..parts.model import resolve_device
+
+        self.device = resolve_device(device)
 
     def sample(self, logits: torch.Tensor, params: list[SamplingParams], serials: list[int], counts: list[int]) -> list[int]:
         """One token per row of `logits` [R, V]; row r belongs to request serials[r], which has
@@ -97,11 +99,16 @@ class Sampler:
         if all(p.greedy for p in params):
             k.argmax(logits, out)
         else:
-            # one row per option, so that each is a contiguous view of one upload
-            host = torch.tensor(
-                [[0.0 if p.greedy else p.temperature for p in params], [p.top_p for p in params],
-                 [uniform_for(p.seed, s, n) for p, s, n in zip(params, serials, counts)]], dtype=torch.float32)
-            topk = torch.tensor([p.top_k for p in params], dtype=torch.int32)
-            host = host.to(logits.device)
-            k.sample(logits, host[0], topk.to(logits.device), host[1], host[2], out)
+            # one row per option, so that each is a contiguous view of one upload; from pinned memory, so that the
+            # copy is queued behind the step instead of making the host wait for it (a copy from pageable memory
+            # would: with a step launched ahead, that is the step whose tokens are not needed yet)
+            pinned = logits.is_cuda
+            host = torch.empty((4, r), dtype=torch.float32, pin_memory=pinned)
+            rows = host.numpy()
+            rows[0] = [0.0 if p.greedy else p.temperature for p in params]
+            rows[1] = [p.top_p for p in params]
+            rows[2] = [uniform_for(p.seed, s, n) for p, s, n in zip(params, serials, counts)]
+            rows[3].view("int32")[:] = [p.top_k for p in params]
+            dev = host.to(logits.device, non_blocking=pinned)
+            k.sample(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], out)
         return PendingTokens(out)

@@ -73,19 +73,21 @@ def test_embedding_and_output_head(dtype):
     ids = torch.tensor([0, 332, 7], dtype=torch.int32, device=DEV)
     # the embedding's output is the step's residual stream: float32, or for few tokens in bfloat16 the 64-bit fixed
     # point (units of 2^-32) that products add themselves into; for many tokens float32 in either precision
-    stream = emb.forward(ids)
+    from types import SimpleNamespace
+
+    stream = emb.forward(SimpleNamespace(token_ids=ids))
     assert stream.dtype == (torch.int64 if dtype == torch.bfloat16 else torch.float32)
     values = stream.double().cpu() / (2.0 ** 32 if stream.dtype == torch.int64 else 1.0)
     assert torch.equal(values, w["e.weight"][[0, 332, 7]])
     many = torch.arange(40, dtype=torch.int32, device=DEV)
-    assert emb.forward(many).dtype == torch.float32
-    assert torch.equal(emb.forward(many).double().cpu(), w["e.weight"][:40])
+    assert emb.forward(SimpleNamespace(token_ids=many)).dtype == torch.float32
+    assert torch.equal(emb.forward(SimpleNamespace(token_ids=many)).double().cpu(), w["e.weight"][:40])
     for tied in (True, False):
         head = make_part("output_head", PartSpec("linear_head", dict(tied=tied), prefix="o."), hidden_size=40, vocab_size=333)
         wh = weights_for(head, dtype, seed=5, scale=1.0)
         assert (len(head.param_specs()) == 0) == tied
         if tied:
-            head.tie(emb.table)
+            head.tie(emb.output_matrix())
         x = torch.randn(4, 40, generator=torch.Generator().manual_seed(6)).to(dtype)
         ref = plain.linear(x.double(), w["e.weight"] if tied else wh["o.weight"])
         out = head.forward(x.to(DEV))

@@ -160,9 +160,12 @@ def test_decoding_runs_one_step_ahead_of_the_host():
         outs = {k: r.output for k, r in reqs.items()}
         if engine_class is FakeEngine:
             plain_outputs = outs
+            plain_stats = s.stats
             assert s.stats.steps_ahead == 0
             continue
         assert outs == plain_outputs
+        # the token that was computed past b's end is not counted as decoded
+        assert (s.stats.decode_tokens, s.stats.prompt_tokens) == (plain_stats.decode_tokens, plain_stats.prompt_tokens)
         assert outs["b"] == expected_output(prompts["b"], 12, eos=eos) and reqs["b"].finish_reason == "eos"
         assert reqs["a"].finish_reason == reqs["c"].finish_reason == "length"
         assert s.stats.steps_ahead == eng.ahead_steps > 8 and s.stats.discarded == 1
@@ -188,6 +191,30 @@ def test_looking_ahead_stops_where_pages_or_the_batch_change():
         outs.append([r.output for r in reqs])
         assert all(r.output == expected_output(r.prompt, 10 + i) for i, r in enumerate(reqs))
         assert eng.cache.free_pages() == [24]
+    assert outs[0] == outs[1]
+
+
+def test_looking_ahead_while_requests_wait_for_a_slot():
+    # more requests than slots: those that wait cannot be admitted before a running one ends, so decoding still runs
+    # ahead of the host; with a slot free (and somebody waiting for it) it does not
+    prompts = [[3 + i, 4, 5] for i in range(5)]
+    outs = []
+    for engine_class in (FakeEngine, FakeAheadEngine):
+        eng = engine_class(num_pages=100)
+        s = Scheduler(eng, SchedulerConfig(max_active=2, max_admit_per_step=2))
+        reqs = [s.add(Request(i, p, GREEDY, max_new_tokens=12)) for i, p in enumerate(prompts)]
+        ahead_while_waiting = 0
+        while s.has_work():
+            before = s.stats.steps_ahead
+            s.step()
+            if s.waiting and s.stats.steps_ahead > before:
+                assert len(s.running) == 2
+                ahead_while_waiting += 1
+        outs.append([r.output for r in reqs])
+        assert all(r.output == expected_output(r.prompt, 12) for r in reqs)
+        if engine_class is FakeAheadEngine:
+            assert ahead_while_waiting >= 12 and s.stats.discarded == 0
+            assert eng.cache.free_pages() == [100]
     assert outs[0] == outs[1]
 
 
