@@ -81,6 +81,20 @@ int egpt_attention_decode_fused(const float* qkv_prod, int in_splits, const floa
                                 void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                                 const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
                                 int window, int n_splits, int n_waves, int combine, int lean, void* stream);
+// Paged attention on the matrix cores for every head size that is a multiple of 16 up to 256 and page sizes that are
+// multiples of 16, bfloat16 or float32 (true float32: v_mfma_f32_16x16x4_f32); see attention_any.hip.  The tiled entry
+// takes prompt portions and mixed batches (operands as egpt_paged_attention).  The decode entry takes one token per
+// request (token q_start[b] belongs to request b): part_o [n_segments][n_seqs][nq][hd] and part_ml
+// [n_segments][n_seqs][nq][2] (float32) take the results of the segments of 64 keys, n_segments >= ceil(longest
+// context / 64), which a second kernel folds into out.  In float32 a row's result is the same bits from either.
+int egpt_attention_any_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                             const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
+                             const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int hd, int page_size,
+                             float scale, int window, int dtype, void* stream);
+int egpt_attention_any_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
+                              const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
+                              const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
+                              int window, int n_segments, int dtype, void* stream);
 int egpt_attention_combine(const float* part_o, const float* part_ml, void* out, int n_rows, int hd, int n_splits,
                            void* stream);
 // Products for m <= 16 rows whose x operand is computed while it is staged (see gemm_skinny.hip).

@@ -17,7 +17,8 @@ import tempfile
 import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_gate_up.hip", "attention.hip", "attention_mfma.hip", "sampling.hip"]
+SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_gate_up.hip", "attention.hip", "attention_mfma.hip", "attention_any.hip",
+           "sampling.hip"]
 HEADERS = ["api.h", "common.h"]
 LIB_NAME = "libeasygpt_hip.so"
 ARCH = "gfx950"

@@ -98,12 +98,12 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
     // lane (li, lg) of a load takes the lg-th 16 bytes of each 64 of row li: an instruction reads 64 contiguous bytes
     // of each of its 16 rows; the j-th of its four values goes into the j-th product instruction, x likewise
     const float* wp = w + static_cast<size_t>(min(n0 + li, n - 1)) * k + lg * 4;
-    auto load_w = [&](float4* av, int step) {
+    auto load_w = [&](f32x4* av, int step) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int k0 = step * kStepF + q * 16 + lg * 4;
-            av[q] = k0 < k ? *reinterpret_cast<const float4*>(wp + static_cast<size_t>(step) * kStepF + q * 16)
-                           : float4{0.f, 0.f, 0.f, 0.f};
+            av[q] = k0 < k ? *reinterpret_cast<const f32x4*>(wp + static_cast<size_t>(step) * kStepF + q * 16)
+                           : f32x4{0.f, 0.f, 0.f, 0.f};
         }
     };
     float4 xr[MT];
@@ -125,34 +125,42 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
     f32x4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float4 a_cur[4], a_next[4];
+    // w runs kAhead steps ahead of the products (16 KB per wavefront on their way: with few rows the kernel is a
+    // stream of w, and a stream one step deep was a chain of round trips, 1.1 TB/s on a 17 MB matrix); the order of
+    // the products, and so every bit of the result, is that of the steps
+    constexpr int kAhead = 4;
+    f32x4 a[kAhead][4];     // (a native vector type: arrays of it stay in registers across the loop's back edge)
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u)
+        if (step_begin + u < step_end) load_w(a[u], step_begin + u);
     if (step_begin < step_end) {
-        load_w(a_cur, step_begin);
         x_load(step_begin);
-        if (step_begin + 1 < step_end) load_w(a_next, step_begin + 1);
         x_store(0);
         if (step_begin + 1 < step_end) x_load(step_begin + 1);
     }
     __syncthreads();
-    for (int step = step_begin; step < step_end; ++step) {
-        const int buf = (step - step_begin) & 1;
-        if (step > step_begin && step + 1 < step_end) load_w(a_next, step + 1);
+    for (int step0 = step_begin; step0 < step_end; step0 += kAhead) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const float av[4] = {a_cur[q].x, a_cur[q].y, a_cur[q].z, a_cur[q].w};
+        for (int u = 0; u < kAhead; ++u) {
+            const int step = step0 + u;
+            if (step >= step_end) break;
+            const int buf = u & 1;                  // (step - step_begin) & 1: kAhead is even
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const float4 b4 = *reinterpret_cast<const float4*>(&xs[buf][t * 16 + li][q * 16 + lg * 4]);
-                const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+            for (int q = 0; q < 4; ++q) {
+                const float av[4] = {a[u][q][0], a[u][q][1], a[u][q][2], a[u][q][3]};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j], acc[t], 0, 0, 0);
+                for (int t = 0; t < MT; ++t) {
+                    const float4 b4 = *reinterpret_cast<const float4*>(&xs[buf][t * 16 + li][q * 16 + lg * 4]);
+                    const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j], acc[t], 0, 0, 0);
+                }
             }
+            if (step + kAhead < step_end) load_w(a[u], step + kAhead);
+            if (step + 1 < step_end) x_store(buf ^ 1);
+            if (step + 2 < step_end) x_load(step + 2);
+            __syncthreads();
         }
-        if (step + 1 < step_end) x_store(buf ^ 1);
-        if (step + 2 < step_end) x_load(step + 2);
-        __syncthreads();
-#pragma unroll
-        for (int q = 0; q < 4; ++q) a_cur[q] = a_next[q];
     }
     // D layout: lane (li, lg) holds rows lg*4 + v of the 16 x 16 tile (an n index) at column li (an m index)
 #pragma unroll

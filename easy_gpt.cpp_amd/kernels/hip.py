@@ -28,7 +28,7 @@ def _load_library(trace: bool = False) -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 13:
+    if lib.egpt_abi_version() != 14:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -97,6 +97,8 @@ class HipKernels(KernelBackend):
             "egpt_gemm_skinny": [vp, vp, vp, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_paged_attention": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
             "egpt_paged_attention_mfma": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, i, vp],
+            "egpt_attention_any_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
+            "egpt_attention_any_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, vp],
             "egpt_argmax": [vp, vp, vp, i, i, vp],
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
@@ -666,9 +668,27 @@ class HipKernels(KernelBackend):
                       float(scale), int(window), n_splits, 16, 1 if combine else 0,
                       self._stream())
             return (part_o, part_ml) if (n_splits > 1 and not combine) else None
+        if hd % 16 == 0 and page_size % 16 == 0:
+            # every other head size in steps of 16, and all of float32: the matrix-core kernels that take any of them
+            if max_q_len == 1 and t == b:
+                n_segments = -(-max_kv_len // self.attention_segment)
+                part_o = torch.empty((n_segments, t, nq, hd), dtype=_F32, device=qkv.device)
+                part_ml = torch.empty((n_segments, t, nq, 2), dtype=_F32, device=qkv.device)
+                self._run("egpt_attention_any_decode", qkv.data_ptr(), out.data_ptr(), part_o.data_ptr(),
+                          part_ml.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), width,
+                          q_start.data_ptr(), kv_len.data_ptr(), b, nq, nkv, hd, page_size, float(scale), int(window),
+                          n_segments, dt, self._stream())
+                return None
+            self._run("egpt_attention_any_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                      block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
+                      nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())
+            return None
+        # head or page sizes that are no multiples of 16: the general kernel
         self._run("egpt_paged_attention", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
                   nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())
+
+    attention_segment = 64       # keys per segment of the decode kernel for any head size (kSegment in attention_any.hip)
 
     @staticmethod
     def _decode_shape(b, nkv, hd, max_kv_len, combine):

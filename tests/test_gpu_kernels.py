@@ -636,6 +636,64 @@ def test_paged_attention_window(k, dtype, window, hd):
     assert err <= (2e-6 if dtype == torch.float32 else 1.2e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 2, 16, 16), (6, 2, 32, 32), (6, 3, 48, 16), (14, 2, 64, 16), (10, 5, 80, 48),
+                                           (8, 2, 96, 16), (7, 1, 112, 16), (12, 2, 128, 64), (4, 1, 144, 16),
+                                           (5, 5, 160, 32), (3, 1, 192, 16), (2, 2, 224, 16), (20, 1, 256, 16)])
+def test_attention_for_any_head_size_on_the_matrix_cores(k, dtype, nq, nkv, hd, ps):
+    # every head size in steps of 16, both precisions (bfloat16 heads of 64 and 128 have kernels of their own, float32
+    # ones do not): prompt portions with and without a prefix, lengths around the chunks of 32 and 64 keys and the
+    # segments of 256, and a group of more than 16 heads
+    seqs = [(1, 1), (9, 9), (1, 130), (7, 71), (2, 64), (1, 65), (33, 33), (3, 200), (70, 300), (40, 520), (5, 1029)]
+    err = run_paged(k, seqs, nq, nkv, hd, ps, dtype)
+    assert err <= (3e-6 if dtype == torch.float32 else 1.2e-2)
+    # only decoded tokens: the kernel that gives every segment of 256 keys a wavefront, and the fold
+    seqs = [(1, max(1, 1500 - 211 * i)) for i in range(8)] + [(1, 256), (1, 257), (1, 512), (1, 2113)]
+    err = run_paged(k, seqs, nq, nkv, hd, ps, dtype, seed=2)
+    assert err <= (3e-6 if dtype == torch.float32 else 1.2e-2)
+    # peaked scores, where a skipped or misplaced key shows
+    err = run_paged(k, [(1, 700), (4, 513), (1, 17), (60, 260)], nq, nkv, hd, ps, dtype, q_scale=5.0, seed=3)
+    assert err <= (3e-5 if dtype == torch.float32 else 5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,window", [(32, 7), (96, 64), (96, 300), (64, 257), (160, 1000)])
+def test_attention_for_any_head_size_with_a_window(k, dtype, hd, window):
+    seqs = [(1, 100), (20, 90), (5, 5), (1, window), (1, window + 1), (3, 66), (40, 300), (1, 900), (70, 1400)]
+    assert run_paged(k, seqs, 6, 2, hd, 16, dtype, window=window) <= (3e-6 if dtype == torch.float32 else 1.2e-2)
+    seqs = [(1, 100), (1, window), (1, window + 1), (1, 900), (1, 1400), (1, 2000)]
+    assert run_paged(k, seqs, 6, 2, hd, 16, dtype, window=window) <= (3e-6 if dtype == torch.float32 else 1.2e-2)
+
+
+@pytest.mark.parametrize("hd,ps,window", [(64, 16, 0), (48, 16, 0), (128, 32, 0), (256, 16, 0), (80, 16, 100), (64, 16, 300)])
+def test_float32_attention_gives_the_same_bits_however_the_rows_are_cut(k, hd, ps, window):
+    # a token's float32 result from the prompt kernel (as a row of a portion, beside other rows and requests) and
+    # from the decode kernel (alone behind its context, in a batch of other lengths) are the same bits: both take
+    # the keys in chunks and segments at fixed positions and fold them with the same operations
+    nq, nkv, dtype = 6, 2, torch.float32
+    n, kv = 70, 700
+    seqs = [(3, 40), (n, kv), (1, 9)]
+    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed=21)
+    t = sum(q for q, _ in seqs)
+    qkv = rnd(t, (nq + 2 * nkv) * hd, seed=22, scale=2.0)
+    ints = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    whole = torch.empty(t, nq * hd, device=DEV)
+    k.paged_attention(qkv, whole, kc, vc, table, ints([0, 3, 3 + n]), ints([3, n, 1]), ints([40, kv, 9]), nq, nkv, hd, ps,
+                      scale, window, n, kv)
+    # the same portion cut in two, the second part alone in its step
+    cut = torch.empty(n - 33, nq * hd, device=DEV)
+    k.paged_attention(qkv[3 + 33 : 3 + n].contiguous(), cut, kc, vc, table[1:2].contiguous(), ints([0]), ints([n - 33]),
+                      ints([kv]), nq, nkv, hd, ps, scale, window, n - 33, kv)
+    assert torch.equal(cut, whole[3 + 33 : 3 + n])
+    # every token of the portion as a decoded token behind its own context, all of them in one batch
+    lens = [kv - n + i + 1 for i in range(n)]
+    single = torch.empty(n, nq * hd, device=DEV)
+    k.paged_attention(qkv[3 : 3 + n].contiguous(), single, kc, vc, table[1:2].expand(n, -1).contiguous(),
+                      ints(list(range(n))), ints([1] * n), ints(lens), nq, nkv, hd, ps, scale, window, 1, kv)
+    assert torch.equal(single, whole[3 : 3 + n])
+
+
 @pytest.mark.parametrize("hd,shape", [(64, 41), (64, 42), (64, 44), (64, 22), (64, 24), (128, 41), (128, 42), (128, 22)])
 @pytest.mark.parametrize("window,ps", [(0, 16), (0, 64), (100, 32), (300, 16)])
 def test_paged_attention_tiled_workgroup_shapes(k, hd, shape, window, ps):
