@@ -4,12 +4,13 @@ and a 2,048-token prefill, for the Qwen2.5-0.5B layer sizes with random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step is one decode step of the whole batch: the engine's step function on one token per request, greedy
-sampling on the device, and the sampled tokens brought to the host (a server needs them there to detect the
-end of a request).  Steps are launched as the scheduler launches them: one step ahead of the host, the token ids
-going from the sampler to the next step on the device (--no-lookahead waits for every step's tokens first).
-Prints one JSON line.  The default run adds the same quantities at further context lengths and at the 1.5B and 7B
-layer sizes to `points` (see FURTHER_CONTEXTS below; --no-further-points skips them).
+A step is one decode step of the whole batch, run by the scheduler (`Scheduler.step`): the engine's step function on
+one token per request, greedy sampling on the device, the sampled tokens brought to the host (a server needs them
+there to detect the end of a request) and the scheduler's bookkeeping.  The scheduler launches a step one step ahead
+of the host, the token ids going from the sampler to the next step on the device (--no-lookahead waits for every
+step's tokens first).  Prints one JSON line.  The default run adds to `points`: the same quantities at further
+context lengths and batch sizes, in float32, at a head size of 96, at the 1.5B, 3B, 7B and 14B layer sizes, and the
+mixed serving workload (see FURTHER_* below; --no-further-points skips them).
 """
 import argparse
 import json
@@ -38,22 +39,29 @@ NEW_TOKENS = 128
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 
-# The larger Qwen2.5 layer sizes, for --shape (the default run and its record stay the 0.5B ones):
-# (config changes, layers of the model, prefix length of the decode runs)
+# The larger Qwen2.5 layer sizes, for --shape and for the further points (the default run and its record stay the
+# 0.5B ones): (config changes, layers of the model, prefix length of the decode runs)
 OTHER_SHAPES = {
     "1.5b": (dict(hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
                   vocab_size=151936, tie_word_embeddings=True), 28, 2048),
+    "3b": (dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, intermediate_size=11008,
+                vocab_size=151936, tie_word_embeddings=True), 36, 4096),
     "7b": (dict(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
                 vocab_size=152064, tie_word_embeddings=False), 28, 4096),
+    "14b": (dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=13824,
+                 vocab_size=152064, tie_word_embeddings=False), 48, 4096),
+    # the 1.5B sizes with 16 heads of 96 instead of 12 of 128: the same products and attention FLOPs, another head size
+    "1.5b-hd96": (dict(hidden_size=1536, num_attention_heads=16, num_key_value_heads=2, head_dim=96,
+                       intermediate_size=8960, vocab_size=151936, tie_word_embeddings=True), 28, 2048),
 }
 
 
 SERVE_REQUESTS, SERVE_NEW_TOKENS, SERVE_CHUNK = 64, 256, 512
 
 
-def serve_workload(engine, name: str, args, vocab: int) -> int:
+def serve_workload(engine, args, vocab: int, name: str = "Qwen2.5-0.5B") -> dict:
     """64 requests, submitted together, prompt lengths uniform in [128, 2048], 256 new tokens each (greedy, end token
-    ignored), through the scheduler with prompts in portions of 512 tokens: total tokens a second."""
+    ignored), through the scheduler with prompts in portions of 512 tokens: total tokens a second, as a record."""
     import random
 
     import torch
@@ -83,7 +91,7 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
         print(f"[bench] serve pass {rep}: {results[-1][0]:.2f} s, {sched.stats.steps} steps", file=sys.stderr, flush=True)
     sec, st = results[-1]
     total = sum(lens) + SERVE_REQUESTS * SERVE_NEW_TOKENS
-    print(json.dumps({
+    return {
         "metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(total / sec, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(sec / st.steps * 1e3, 3),
         "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
@@ -93,184 +101,26 @@ def serve_workload(engine, name: str, args, vocab: int) -> int:
                    "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": min(SERVE_CHUNK, args.serve_budget),
                    "max_tokens_per_step": args.serve_budget,
                    "preemptions": st.preemptions, "steps_launched_ahead": st.steps_ahead, "sampling": "greedy"},
-    }), flush=True)
-    return 0
+    }
 
 
-def link_floor() -> int:
-    """What a chain of dependent kernels costs apart from its work: graphs of 125 links that each do next to nothing
-    (every thread one load of what the link before wrote, `trips - 1` further loads that depend on each other, one
-    store), replayed; microseconds per link by number of workgroups and of dependent round trips to memory, with
-    the further loads near (within the few kilobytes that the link before wrote: L2) or far (anywhere in 1 GiB: HBM).
-    Then the same chain with flags in memory in place of kernel boundaries."""
-    import torch
-
-    from easy_gpt.cpp_amd import kernels
-
-    k = kernels.backend()
-    links, table = 125, {}
-    far = 1 << 28                                       # floats: dependent loads that range over 1 GiB miss every cache
-    far_a, far_b = torch.zeros(far, device="cuda"), torch.zeros(far, device="cuda")
-    for where in ("near", "far"):
-        for groups in (1, 64, 256, 1024, 4096):
-            n = groups * 256
-            if where == "near":
-                a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
-            else:
-                a, b = far_a, far_b
-            for trips in (1, 2, 3, 5):
-                def chain():
-                    src, dst = a, b
-                    for _ in range(links):
-                        k.probe_link(src, dst, trips, n)
-                        src, dst = dst, src
-                chain()
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    chain()
-                for _ in range(3):
-                    graph.replay()
-                torch.cuda.synchronize()
-                reps = 20
-                t0 = time.perf_counter()
-                for _ in range(reps):
-                    graph.replay()
-                torch.cuda.synchronize()
-                key = f"{where}_wg{groups}_trips{trips}"
-                table[key] = round((time.perf_counter() - t0) / reps / links * 1e6, 3)
-                print(f"[bench] {groups:5d} workgroups, {trips} dependent loads ({where}): {table[key]:.2f} us a link",
-                      file=sys.stderr, flush=True)
-    # The same chain with its links handed over through flags in memory: the links alternate between two streams of
-    # one graph (two hardware queues), so a link is resident and waiting while the link before runs; its first thread
-    # polls the flag past the caches, then all threads read what the link before wrote past the caches.
-    del far_a, far_b
-    side = torch.cuda.Stream()
-    main = torch.cuda.Stream()
-    links = 124
-    for groups in (1, 64, 128, 256, 512):
-        n = groups * 256
-        a, b = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
-        flags = torch.zeros(links, dtype=torch.int32, device="cuda")
-        gave_up = torch.zeros(1, dtype=torch.int32, device="cuda")
-
-        def chain():
-            first = torch.cuda.current_stream()
-            flags.zero_()
-            a.zero_()
-            side.wait_stream(first)
-            src, dst = a, b
-            for link in range(links):
-                k.probe_handoff(src, dst, n, flags[link - 1 : link] if link else None, groups, flags[link : link + 1], gave_up,
-                                first if link % 2 == 0 else side)
-                src, dst = dst, src
-            first.wait_stream(side)
-            return src
-
-        with torch.cuda.stream(main):
-            chain()
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=main):
-                result = chain()
-            for _ in range(3):
-                graph.replay()
-            torch.cuda.synchronize()
-            reps = 20
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                graph.replay()
-            torch.cuda.synchronize()
-            us = (time.perf_counter() - t0) / reps / links * 1e6
-        right = float(result.min()) == links and float(result.max()) == links and int(gave_up.item()) == 0
-        table[f"handoff_wg{groups}"] = round(us, 3)
-        print(f"[bench] {groups:5d} workgroups, handed over through a flag, links on two streams in turn: {us:.2f} us a link"
-              f"{'' if right else ' (WRONG RESULT or a wait ran out)'}", file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "microseconds per link of a replayed graph of 125 dependent near-empty kernels",
-                      "unit": "us", "links": 125, "table": table}), flush=True)
-    return 0
-
-
-def anatomy(args, base: dict, name: str) -> int:
-    """What the kernels of one decode step spend their time on, seen from inside: the step is replayed from its graph
-    with the library's trace build, whose product and decode-attention kernels write the wall clock of four phases per
-    workgroup (start; operands staged or queries made; matrix products done; results stored).  Per kind of kernel,
-    medians over the layers, in microseconds: the gap from the end of the kernel before to the first workgroup's
-    start, the ramp until the last workgroup has started, the phases of the median workgroup, and the span from the
-    first start to the last end.  Timestamps cost a little: the step takes a few per cent longer than in bench runs."""
-    import statistics
-    import tempfile
-
-    import torch
-
-    from easy_gpt.cpp_amd import kernels
-    from easy_gpt.cpp_amd.engine import Engine, StepEntry
-    from easy_gpt.cpp_amd.kernels.hip import HipKernels
-    from easy_gpt.cpp_amd.weights import write_random_model
-
-    k = HipKernels(trace=True)
-    kernels.use_backend(k)
-    batch, prefix = args.batch, PREFIX
-    tmp = tempfile.mkdtemp(prefix="egpt_bench_")
-    write_random_model(tmp, base, seed=0, dtype=torch.bfloat16)
-    engine = Engine.from_dir(tmp, dtype="bfloat16", device="cuda:0", page_size=args.page_size,
-                             max_tokens=batch * (prefix + 256) + 2048, max_requests=batch + 1)
-    g = torch.Generator().manual_seed(0)
-    rids = [f"d{i}" for i in range(batch)]
-    for rid in rids:
-        engine.add_request(rid)
-        engine.step([StepEntry(rid, torch.randint(0, base["vocab_size"], (prefix,), generator=g).tolist(), [prefix - 1])])
-    for i in range(6):
-        engine.step([StepEntry(rid, [5 + i], [0]) for rid in rids])
-    buf = k.trace_attach()
-    for rep in range(3):
-        buf.zero_()
-        torch.cuda.synchronize()
-        engine.step([StepEntry(rid, [77 + rep], [0]) for rid in rids])
-        torch.cuda.synchronize()
-    launches = k.trace_records(buf)
-    kinds: dict = {}
-    prev_end, rates = None, []
-    for launch in launches:
-        wgs = [w["us"] for w in launch["workgroups"]]
-        first, last_start = min(w[0] for w in wgs), max(w[0] for w in wgs)
-        end = max(w[3] for w in wgs)
-        med = lambda j: statistics.median(w[j] - w[0] for w in wgs if w[j]) if any(w[j] for w in wgs) else None
-        key = (k.TRACED_KERNELS.get(launch["kernel"], str(launch["kernel"])), len(wgs))
-        kinds.setdefault(key, []).append((first - prev_end if prev_end is not None else 0.0, last_start - first,
-                                          med(1), med(2), med(3), end - first))
-        prev_end = end
-        for w in launch["workgroups"]:
-            if w["us"][3] > w["us"][0] + 0.5:
-                rates.append(((w["cycles"][3] - w["cycles"][0]) & 0xffffffff) / (w["us"][3] - w["us"][0]))
-    rows = []
-    print(f"{'kernel':46s} {'wgs':>5s} {'calls':>5s} | {'gap':>5s} {'ramp':>5s} {'staged':>6s} {'mfma':>5s} {'stored':>6s} {'span':>5s}",
-          file=sys.stderr)
-    for (kind, n_wgs), v in kinds.items():
-        m = [None if any(x[i] is None for x in v) else round(statistics.median(x[i] for x in v), 2) for i in range(6)]
-        rows.append({"kernel": kind, "workgroups": n_wgs, "calls": len(v), "gap": m[0], "ramp": m[1], "staged": m[2],
-                     "mfma": m[3], "stored": m[4], "span": m[5]})
-        f = lambda x: "    -" if x is None else f"{x:5.2f}"
-        print(f"{kind:46s} {n_wgs:5d} {len(v):5d} | {f(m[0])} {f(m[1])} {f(m[2]):>6s} {f(m[3])} {f(m[4]):>6s} {f(m[5])}", file=sys.stderr)
-    marks = [w["us"] for launch in launches for w in launch["workgroups"]]
-    total = max(w[3] for w in marks) - min(w[0] for w in marks)
-    rates.sort()
-    print(json.dumps({"metric": f"anatomy of a decode step at batch {batch} ({name}, prefix {prefix}), microseconds",
-                      "first_start_to_last_end_us": round(total, 1), "shader_clock_mhz": round(rates[len(rates) // 2]),
-                      "kernels": rows}), flush=True)
-    return 0
-
-
-# The further points of the default run, beside decode_b1 and decode_b64.  Each name starts with what differs from the
-# headline shape, then the quantity as there (decode_b<batch>: decoded tokens a second; prefill: tokens a second):
-#   ctx8k_, ctx32k_  the 0.5B sizes with prefixes of 8,192 and 32,640 tokens (prefill: one prompt of that length in one step)
-#   q1p5b_           Qwen2.5-1.5B layer sizes (28 layers, hidden 1536, 12 / 2 heads of 128, intermediate 8960, vocabulary
-#                    151936, tied), prefixes of 2,048 tokens, a 2,048-token prefill
-#   q7b_             Qwen2.5-7B layer sizes (28 layers, hidden 3584, 28 / 4 heads of 128, intermediate 18944, vocabulary
-#                    152064, untied), prefixes of 4,096 tokens, a 2,048-token prefill
-FURTHER_CONTEXTS = (("ctx8k", 8192), ("ctx32k", 32640))
-FURTHER_SHAPES = (("q1p5b", "1.5b"), ("q7b", "7b"))
+# What the default run measures beside its record (all layers of each model, random weights drawn on the GPU):
+# at the 0.5B sizes (the record's model) prefixes of 8k and 32k tokens with a prefill of that length, and batches of
+# 128 and 256 behind 2k and 8k;
+FURTHER_CONTEXTS = (("ctx8k", 8192, (256, 128, 64, 8, 1)), ("ctx32k", 32640, (64, 8, 1)))
+FURTHER_BATCHES = (128, 256)
+# at other layer sizes a 2,048-token prefill and decode runs (label, shape, dtype, ((prefix, batches), ...)); the
+# first prefix is the shape's own and its points are named without it
+FURTHER_SHAPES = (
+    ("fp32", "0.5b", "float32", ((2048, (8,)),)),
+    ("hd96", "1.5b-hd96", "bfloat16", ()),
+    ("q1p5b", "1.5b", "bfloat16", ((2048, (1, 8, 64)),)),
+    ("q3b", "3b", "bfloat16", ((4096, (1, 8, 64)),)),
+    ("q7b", "7b", "bfloat16", ((4096, (1, 8, 64)), (2048, (128, 256)), (8192, (128,)))),
+    ("q14b", "14b", "bfloat16", ((4096, (1, 8, 64)),)),
+)
 FURTHER_WARMUP, FURTHER_STEPS = 4, 32
+FILL_TOKENS = 65536         # prompts are put into the cache several to a step, up to this many tokens
 
 
 def remove_folder(path: str) -> None:
@@ -279,60 +129,78 @@ def remove_folder(path: str) -> None:
     os.rmdir(path)
 
 
+def shape_config(shape: str) -> tuple[dict, int]:
+    if shape == "0.5b":
+        return dict(QWEN25_05B), PREFIX
+    changes, n_layers, prefix = OTHER_SHAPES[shape]
+    return dict(QWEN25_05B, **changes, num_hidden_layers=n_layers), prefix
+
+
 def further_points(args, model_dir: str, cfg: dict, g) -> dict:
-    """Decode at batch 1 / 8 / 64 and a prefill at further context lengths (the model in `model_dir`) and at the larger
-    layer sizes (random weights drawn on the GPU), all layers of each model: a flat dict of tokens a second."""
+    """The points beside the record: a flat dict of tokens a second."""
     import torch
 
     from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.engine.engine import load_random_model
     from easy_gpt.cpp_amd.sampling import Sampler
-    from easy_gpt.cpp_amd.weights import write_random_model
 
     points, page = {}, args.page_size
     warm, steps = FURTHER_WARMUP, FURTHER_STEPS
-    room = 3 * (warm + steps) + page                    # the first request decodes in all three runs
 
-    def rate(label, what, tokens, sec):
-        points[f"{label}_{what}"] = round(tokens / sec, 1)
-        print(f"[bench] {label} {what}: {tokens / sec:.1f} tok/s, {sec / (steps if what != 'prefill' else 1) * 1e3:.3f} ms",
+    def rate(name, tokens, sec, per_step=True):
+        points[name] = round(tokens / sec, 1)
+        print(f"[bench] {name}: {tokens / sec:.1f} tok/s, {sec / (steps if per_step else 1) * 1e3:.3f} ms",
               file=sys.stderr, flush=True)
 
-    longest = max(p for _, p in FURTHER_CONTEXTS)
-    engine = Engine.from_dir(model_dir, dtype=args.dtype, device="cuda:0", page_size=page,
-                             max_tokens=65 * (-(-(longest + room) // page) * page), max_requests=66,
-                             tune_products=not args.no_tune)
-    sampler = Sampler(engine.device)
-    for label, prefix in FURTHER_CONTEXTS:              # the prefixes are filled once and decoded as 64, 8 and 1
-        rate(label, "prefill", prefix, prefill_seconds(engine, cfg["vocab_size"], prefix, g, reps=3))
-        rids, last = fill_requests(engine, sampler, cfg["vocab_size"], prefix, 64, g)
-        for b in (64, 8, 1):
+    def decode_runs(engine, sampler, vocab, label, prefix, batches):
+        """Prefixes of `prefix` tokens for the largest batch, filled once and decoded as each of `batches`
+        (largest first: every run's first requests have decoded in the runs before it)."""
+        batches = sorted(batches, reverse=True)
+        rids, last = fill_requests(engine, sampler, vocab, prefix, batches[0], g)
+        for b in batches:
             sub = last[:b]
-            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids[:b], sub, warm, steps, args.no_lookahead)[0])
+            sec = decode_seconds(engine, sampler, rids[:b], sub, warm, steps, args.no_lookahead)[0]
+            rate(f"{label}_decode_b{b}" if label else f"decode_b{b}", b * steps, sec)
             last[:b] = sub
         for rid in rids:
             engine.finish(rid)
+
+    def room(prefix, batches):        # tokens the runs of one prefix hold: every run decodes the first requests further
+        return max(batches) * (-(-(prefix + len(batches) * (warm + steps) + 1) // page) * page)
+
+    # ---- the record's model: further contexts and batches
+    tokens = max([room(p, b) for _, p, b in FURTHER_CONTEXTS] + [room(PREFIX, FURTHER_BATCHES)])
+    engine = Engine.from_dir(model_dir, dtype=args.dtype, device="cuda:0", page_size=page,
+                             max_tokens=tokens + FILL_TOKENS, max_requests=max(FURTHER_BATCHES) + 2,
+                             tune_products=not args.no_tune)
+    sampler = Sampler(engine.device)
+    decode_runs(engine, sampler, cfg["vocab_size"], "", PREFIX, FURTHER_BATCHES)
+    for label, prefix, batches in FURTHER_CONTEXTS:
+        rate(f"{label}_prefill", prefix, prefill_seconds(engine, cfg["vocab_size"], prefix, g, reps=3), per_step=False)
+        decode_runs(engine, sampler, cfg["vocab_size"], label, prefix, batches)
+    # ---- the mixed serving workload through the scheduler (what `--serve` prints)
+    serve = serve_workload(engine, args, cfg["vocab_size"])
+    points["serve_tokens_per_s"] = serve["value"]
+    print(f"[bench] serve: {serve['value']} tok/s (prompts and generated), {serve['steps']} steps", file=sys.stderr, flush=True)
     del engine, sampler
     torch.cuda.empty_cache()
 
-    for label, shape in FURTHER_SHAPES:
-        changes, n_layers, prefix = OTHER_SHAPES[shape]
-        other = dict(QWEN25_05B, **changes, num_hidden_layers=n_layers)
+    # ---- other layer sizes, head sizes and float32
+    for label, shape, dtype, runs in FURTHER_SHAPES:
+        other, _ = shape_config(shape)
         t0 = time.time()
-        tmp = tempfile.mkdtemp(prefix="egpt_bench_")
-        write_random_model(tmp, other, seed=0, dtype=torch.bfloat16, device="cuda:0")
-        engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page,
-                                 max_tokens=64 * (-(-(prefix + warm + steps) // page) * page) + PREFILL_TOKENS,
-                                 max_requests=65, tune_products=not args.no_tune)
-        remove_folder(tmp)
+        model = load_random_model(other, seed=0, dtype=dtype, device="cuda:0")
+        tokens = max([room(p, b) for p, b in runs] + [0]) + max(FILL_TOKENS, PREFILL_TOKENS)
+        engine = Engine(model, page_size=page, max_tokens=tokens, max_requests=max([max(b) for _, b in runs] + [1]) + 2,
+                        tune_products=not args.no_tune)
         sampler = Sampler(engine.device)
         print(f"[bench] {label} model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
-        rate(label, "prefill", PREFILL_TOKENS, prefill_seconds(engine, other["vocab_size"], PREFILL_TOKENS, g, reps=5))
-        for b in (1, 8, 64):
-            rids, last = fill_requests(engine, sampler, other["vocab_size"], prefix, b, g)
-            rate(label, f"decode_b{b}", b * steps, decode_seconds(engine, sampler, rids, last, warm, steps, args.no_lookahead)[0])
-            for rid in rids:
-                engine.finish(rid)
-        del engine, sampler
+        rate(f"{label}_prefill", PREFILL_TOKENS, prefill_seconds(engine, other["vocab_size"], PREFILL_TOKENS, g, reps=5),
+             per_step=False)
+        for i, (prefix, batches) in enumerate(runs):
+            decode_runs(engine, sampler, other["vocab_size"], label if i == 0 else f"{label}_ctx{prefix // 1024}k",
+                        prefix, batches)
+        del engine, sampler, model
         torch.cuda.empty_cache()
     return points
 
@@ -357,7 +225,8 @@ def prefill_seconds(engine, vocab: int, tokens: int, g, reps: int = 10) -> float
 
 
 def fill_requests(engine, sampler, vocab: int, prefix: int, batch: int, g):
-    """`batch` requests with prefixes of `prefix` random tokens in the cache (untimed); their ids and next tokens."""
+    """`batch` requests with prefixes of `prefix` random tokens in the cache (untimed, several prompts to a step); their
+    ids and next tokens."""
     import torch
 
     from easy_gpt.cpp_amd.engine import StepEntry
@@ -365,12 +234,66 @@ def fill_requests(engine, sampler, vocab: int, prefix: int, batch: int, g):
 
     greedy = SamplingParams(greedy=True)
     rids, last = [f"d{i}" for i in range(batch)], []
-    for rid in rids:
-        engine.add_request(rid)
-        p = torch.randint(0, vocab, (prefix,), generator=g).tolist()
-        out = engine.step([StepEntry(rid, p, [prefix - 1])])
-        last.append(sampler.sample(out, [greedy], [0], [0])[0])
+    per_step = max(1, FILL_TOKENS // prefix)
+    from easy_gpt.cpp_amd import kernels
+
+    tuned = kernels.library_tuning
+    if tuned and per_step > 1:
+        kernels.tune_library_products(False)       # (no measurements for the shapes of these untimed steps)
+    for first in range(0, batch, per_step):
+        group = rids[first : first + per_step]
+        entries = []
+        for rid in group:
+            engine.add_request(rid)
+            entries.append(StepEntry(rid, torch.randint(0, vocab, (prefix,), generator=g).tolist(), [prefix - 1]))
+        out = engine.step(entries)
+        last.extend(sampler.sample(out, [greedy] * len(group), [0] * len(group), [0] * len(group)))
+    if tuned and per_step > 1:
+        kernels.tune_library_products(True)
     return rids, last
+
+
+def scheduler_decode_seconds(engine, vocab: int, prefix: int, batch: int, warmup: int, steps: int, g,
+                             no_lookahead: bool = False) -> tuple[float, float]:
+    """Seconds of `steps` decode steps of `batch` requests through `Scheduler.step` after `warmup` untimed ones, and the
+    median time between two steps' returns.  The requests are admitted together and their prompts (the prefixes) run
+    in one step, so that all of them decode from the same context length on."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    sched = Scheduler(engine, SchedulerConfig(max_active=batch, max_admit_per_step=batch,
+                                              max_tokens_per_step=batch * prefix, prefill_chunk=prefix), eos_token_id=-1)
+    if no_lookahead:
+        sched.lookahead = False
+    for i in range(batch):
+        sched.add(Request(f"d{i}", torch.randint(0, vocab, (prefix,), generator=g).tolist(), SamplingParams(greedy=True),
+                          max_new_tokens=warmup + steps + 8, ignore_eos=True))
+    from easy_gpt.cpp_amd import kernels
+
+    tuned = kernels.library_tuning
+    if tuned:
+        kernels.tune_library_products(False)       # (no measurements for the shapes of this one untimed step)
+    sched.step()                                   # the prompts
+    if tuned:
+        kernels.tune_library_products(True)
+    assert len(sched.running) == batch and all(len(r.output) == 1 for r in sched.running)
+    for _ in range(warmup):
+        sched.step()
+    arrivals = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sched.step()                               # returns when the step's tokens are on the host
+        arrivals.append(time.perf_counter())
+    torch.cuda.synchronize()                       # (with the step that was launched ahead of the last return)
+    sec = time.perf_counter() - t0
+    assert sched.stats.generated == batch * (1 + warmup + steps) and not sched.stats.preemptions
+    for r in list(sched.running):
+        engine.finish(r.request_id)
+    between = sorted(b - a for a, b in zip(arrivals, arrivals[1:]))
+    return sec, (between[len(between) // 2] if between else sec / steps)
 
 
 def decode_seconds(engine, sampler, rids, last, warmup: int, steps: int, no_lookahead: bool = False) -> tuple[float, float]:
@@ -429,7 +352,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     ap.add_argument("--shape", default="0.5b", choices=["0.5b"] + sorted(OTHER_SHAPES),
-                    help="layer sizes: Qwen2.5-0.5B (the default, which the headline numbers are quoted on), 1.5B or 7B")
+                    help="layer sizes: Qwen2.5-0.5B (the default, which the headline numbers are quoted on) or a larger one")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prefix", type=int, default=None,
                     help="tokens each request holds before decoding starts (default: 2,048; 4,096 at the 7B sizes)")
@@ -448,14 +371,9 @@ def main() -> int:
     ap.add_argument("--no-lookahead", action="store_true",
                     help="wait for a step's tokens on the host before the next step is launched (the scheduler with --serve, "
                          "the decode loop otherwise)")
-    ap.add_argument("--anatomy", action="store_true",
-                    help="instead of timing: one decode step at --batch seen from inside its kernels (the library's trace "
-                         "build, compiled at the first call)")
-    ap.add_argument("--link-floor", action="store_true",
-                    help="instead of the model: what a link of a chain of dependent, near-empty kernels costs in a graph")
+    ap.add_argument("--direct-loop", action="store_true",
+                    help="decode with the engine's step function in a loop of the benchmark's own instead of Scheduler.step")
     args = ap.parse_args()
-    if args.link_floor:
-        return link_floor()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path, --gpus {args.gpus} is not run")
         return 2
@@ -473,8 +391,6 @@ def main() -> int:
         PREFIX, CONTEXT = args.prefix, args.prefix + 2048
     if args.layers is None:
         args.layers = FULL_LAYERS
-    if args.anatomy:
-        return anatomy(args, dict(base, num_hidden_layers=args.layers), name)
     if args.warmup + args.steps > CONTEXT - PREFIX:
         print(f"--warmup + --steps must stay within the context of {CONTEXT} after a prefix of {PREFIX}")
         return 2
@@ -490,7 +406,7 @@ def main() -> int:
     elem = 2 if args.dtype == "bfloat16" else 4
     h, nq, nkv, inter, vocab = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                                 cfg["intermediate_size"], cfg["vocab_size"])
-    hd = h // nq
+    hd = cfg.get("head_dim", h // nq)
     layers = args.layers
     page_size = args.page_size
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
@@ -512,7 +428,8 @@ def main() -> int:
 
     if args.serve:
         remove_folder(tmp)
-        return serve_workload(engine, name, args, vocab)
+        print(json.dumps(serve_workload(engine, args, vocab, name)), flush=True)
+        return 0
     # the further points stand beside the default run's record only
     further = not (args.no_points or args.no_further_points or args.shape != "0.5b" or args.prefix is not None
                    or args.layers != FULL_LAYERS or args.dtype != "bfloat16" or args.batch != 8)
@@ -541,10 +458,13 @@ def main() -> int:
 
     # ---------------------------------------------------------------- decoding at each batch size
     def decode_run(batch: int, warmup: int, steps: int):
-        rids, last = fill_requests(engine, sampler, vocab, PREFIX, batch, g)
-        sec, medians[batch] = decode_seconds(engine, sampler, rids, last, warmup, steps, args.no_lookahead)
-        for rid in rids:
-            engine.finish(rid)
+        if args.direct_loop:
+            rids, last = fill_requests(engine, sampler, vocab, PREFIX, batch, g)
+            sec, medians[batch] = decode_seconds(engine, sampler, rids, last, warmup, steps, args.no_lookahead)
+            for rid in rids:
+                engine.finish(rid)
+        else:
+            sec, medians[batch] = scheduler_decode_seconds(engine, vocab, PREFIX, batch, warmup, steps, g, args.no_lookahead)
         mean_ctx = PREFIX + warmup + (steps + 1) / 2.0
         step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
         return sec, step_bytes
@@ -577,7 +497,8 @@ def main() -> int:
             "heads": nq, "kv_heads": nkv, "head_dim": hd, "intermediate": inter, "vocab": vocab, "tied": bool(cfg["tie_word_embeddings"]),
             "global_batch": args.batch, "seq_len": CONTEXT, "prefix_len": PREFIX, "new_tokens": new_tokens,
             "page_size": page_size, "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "sampling": "greedy", "parallelism": "single GPU", "library_products": "first choice" if args.no_tune else "measured",
+            "sampling": "greedy", "library_products": "first choice" if args.no_tune else "measured",
+            "parallelism": "single GPU, decode steps run by " + ("a loop over Engine.step" if args.direct_loop else "Scheduler.step"),
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 5)},

@@ -134,13 +134,6 @@ size_t egpt_sample_workspace(int n_rows, int vocab);
 int egpt_sample_wide(const float* logits, const float* temperature, const int32_t* top_k, const float* top_p,
                      const float* uniform, int32_t* out, void* workspace, int n_rows, int vocab, void* stream);
 
-// Measurement only: one link of a chain of dependent kernels that does next to nothing (see elementwise.hip);
-// in, out float32 [span] (in all zeros), one workgroup per 256 of the first n elements, `trips` dependent loads per
-// thread, all but the first anywhere in the span.
-int egpt_probe_link(const float* in, float* out, int n, int trips, int span, void* stream);
-int egpt_probe_handoff(const float* in, float* out, int n, const unsigned* wait_flag, unsigned wait_count,
-                       unsigned* signal_flag, unsigned* gave_up, int spin_limit, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -520,7 +520,6 @@ struct FusedQkv {
     const int32_t* slots;     // [n_tokens] page * page_size + offset of the token's key and value
     bf16_t* k_cache_w;        // the caches again, writable
     bf16_t* v_cache_w;
-    unsigned trace_base;      // builds with EGPT_TRACE: the first record of this launch's workgroups
 };
 
 // Decoded tokens only (one query token per request, its heads of one kv group in one 16-row tile): a
@@ -550,7 +549,6 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     const int lj = lane % 16, lg = lane / 16;
     const int b = blockIdx.x, kh = blockIdx.y, split = blockIdx.z;
     const int group_size = nq / nkv;
-    EGPT_MARK(f.trace_base, 5, 0);
     const int kv = kv_len[b], tok = q_start[b];
     const int p = kv - 1;
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
@@ -742,7 +740,6 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
         load_round(kb0);
         if (kb0 == w_begin) {
             make_q();
-            EGPT_MARK(f.trace_base, 5, 1);
         }
         if constexpr (FUSED) {
             // the new token's key and value come from LDS, not from the cache line that was just written
@@ -819,7 +816,6 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
         }
         kb0 += PF;
     } while (kb0 < w_end);
-    EGPT_MARK(f.trace_base, 5, 2);
     float l = l_run;
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
@@ -858,7 +854,6 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
             }
         }
     }
-    EGPT_MARK(f.trace_base, 5, 3);
 }
 
 // out[row, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s over the splits; one wavefront per row.
@@ -964,7 +959,6 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
         }
     }
     FusedQkv fq = fused ? *fused : FusedQkv{};
-    fq.trace_base = EGPT_TRACE_TAKE(grid);
     if (fused)
         attention_decode_kernel<HD, PF, true><<<grid, n_waves * kWave, lds, s>>>(
             nullptr, static_cast<bf16_t*>(out), part_o, part_ml, static_cast<const bf16_t*>(k_cache),
@@ -1001,7 +995,6 @@ static int dispatch_decode(const void* qkv, void* out, float* part_o, float* par
 }  // namespace egpt
 
 using namespace egpt;
-EGPT_TRACE_ATTACH(attention_mfma)
 
 // Prompt portions (and mixed batches) with keys and values shared through LDS by the wavefronts of a
 // workgroup.  Same operands and meaning as egpt_paged_attention_mfma with n_splits == 1; page sizes that are

@@ -87,26 +87,19 @@ def _log(msg: str, verbose: bool) -> None:
         print(f"[easy_gpt.cpp_amd build] {msg}", file=sys.stderr, flush=True)
 
 
-TRACE_LIB_NAME = "libeasygpt_hip_trace.so"
-
-
-def build(verbose: bool = True, trace: bool = False) -> str:
-    """Compile every source for gfx950 and link the library.  Always compiles.  trace=True: the variant with
-    timestamps from inside the kernels (-DEGPT_TRACE, see common.h), a library of its own beside the other, for
-    measurements only."""
+def build(verbose: bool = True) -> str:
+    """Compile every source for gfx950 and link the library.  Always compiles."""
     hipcc = _hipcc()
     if hipcc is None:
         raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
     lib, stamp = _paths()
-    if trace:
-        lib, stamp = os.path.join(os.path.dirname(lib), TRACE_LIB_NAME), os.path.join(os.path.dirname(lib), "libeasygpt_hip_trace.stamp")
     obj_dir = tempfile.mkdtemp(prefix="egpt_build_")
     t0 = time.time()
     try:
         procs = []
         for src in SOURCES:
             obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
-            cmd = [hipcc, *FLAGS, *(["-DEGPT_TRACE"] if trace else []), "-I", HERE, "-c", os.path.join(HERE, src), "-o", obj]
+            cmd = [hipcc, *FLAGS, "-I", HERE, "-c", os.path.join(HERE, src), "-o", obj]
             _log(f"compiling {src} for {ARCH}", verbose)
             procs.append((src, obj, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs = []
@@ -136,18 +129,6 @@ def build(verbose: bool = True, trace: bool = False) -> str:
         return lib
     finally:
         shutil.rmtree(obj_dir, ignore_errors=True)
-
-
-def ensure_trace_built(verbose: bool = True) -> str:
-    """Path of the library with timestamps from inside the kernels; builds it if there is none that matches the sources."""
-    lib, _ = _paths()
-    d = os.path.dirname(lib)
-    lib, stamp = os.path.join(d, TRACE_LIB_NAME), os.path.join(d, "libeasygpt_hip_trace.stamp")
-    if os.path.isfile(lib) and os.path.isfile(stamp):
-        with open(stamp) as f:
-            if f.read().strip() == source_hash():
-                return lib
-    return build(verbose, trace=True)
 
 
 def ensure_built(verbose: bool = True) -> str:

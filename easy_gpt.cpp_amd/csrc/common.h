@@ -97,46 +97,6 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 
 }  // namespace egpt
 
-// Timestamps from inside kernels, for builds with -DEGPT_TRACE only (an ordinary build has none of this).
-// EGPT_MARK(base, kernel, phase): the first thread of a workgroup stores the wall clock (units of 10 ns) of `phase`
-// (0 to 3) into record `base + workgroup` of a buffer that the host attached with
-// egpt_trace_attach_<file>(buffer, capacity); a launcher takes `base` for its grid from egpt_trace_take, so a
-// captured graph's nodes keep their records over replays.  A decode step is a chain of short dependent kernels;
-// what a link's time is made of (launch, the first load's way from memory, arithmetic, the tail) shows only
-// from inside.  A record is five words: (kernel << 48 | workgroup), then the four phases' clocks.
-#ifdef EGPT_TRACE
-extern "C" unsigned egpt_trace_take(unsigned n_workgroups);
-namespace egpt {
-static __device__ unsigned long long* trace_buf = nullptr;
-static __device__ unsigned int trace_cap = 0;
-__device__ __forceinline__ void trace_mark(unsigned base, unsigned kernel, unsigned phase) {
-    __builtin_amdgcn_sched_barrier(0);
-    if (threadIdx.x == 0 && trace_buf) {
-        const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-        if (base + wg < trace_cap) {
-            unsigned long long* rec = trace_buf + static_cast<size_t>(base + wg) * 5;
-            if (phase == 0) rec[0] = (static_cast<unsigned long long>(kernel) << 48) | wg;
-            // low words of the wall clock (10 ns) and of the shader clock (cycles): the two together give the clock rate
-            rec[1 + phase] = (wall_clock64() & 0xffffffffull) | (static_cast<unsigned long long>(clock64()) << 32);
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-}
-}  // namespace egpt
-#define EGPT_MARK(base, kernel, phase) egpt::trace_mark(base, kernel, phase)
-#define EGPT_TRACE_TAKE(grid) egpt_trace_take((grid).x * (grid).y * (grid).z)
-#define EGPT_TRACE_ATTACH(file)                                                                          \
-    extern "C" int egpt_trace_attach_##file(void* buf, unsigned cap) {                                   \
-        if (hipMemcpyToSymbol(HIP_SYMBOL(egpt::trace_buf), &buf, sizeof(buf)) != hipSuccess) return 1;   \
-        if (hipMemcpyToSymbol(HIP_SYMBOL(egpt::trace_cap), &cap, sizeof(cap)) != hipSuccess) return 1;   \
-        return 0;                                                                                        \
-    }
-#else
-#define EGPT_MARK(base, kernel, phase) do {} while (0)
-#define EGPT_TRACE_TAKE(grid) 0u
-#define EGPT_TRACE_ATTACH(file)
-#endif
-
 // Error codes returned by every entry point (0 = launched).
 #define EGPT_OK 0
 #define EGPT_BAD_ARGUMENT 1

@@ -602,88 +602,6 @@ extern "C" int egpt_rope_table(const int32_t* positions, const float* inv_freq, 
     return EGPT_OK;
 }
 
-// ---- a link of a chain of dependent kernels that does next to nothing: what the runtime and the memory system
-// charge a decode step per kernel and per dependent round trip, apart from any useful work.  Thread i reads in[i]
-// (written by the link before), then makes `trips - 1` further loads, each at an address that depends on the value
-// loaded before, and writes out[i].  The further loads range over `span` elements of `in`: a span as small as the
-// grid keeps them in L2, a span of hundreds of megabytes sends every one to another page of HBM.
-namespace egpt {
-__global__ __launch_bounds__(256) void probe_link_kernel(const float* __restrict__ in, float* __restrict__ out, int n,
-                                                         int trips, int span) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    float v = in[i];
-    long at = i;
-    for (int r = 1; r < trips; ++r) {
-        at = (at * 16 + 1048583 + static_cast<long>(v)) % span;       // v is zero throughout, but only the load can tell
-        v += __builtin_nontemporal_load(in + at);
-    }
-    out[i] = v;
-}
-}  // namespace egpt
-
-extern "C" int egpt_probe_link(const float* in, float* out, int n, int trips, int span, void* stream) {
-    if (!in || !out || n <= 0 || trips < 1 || span < n) return EGPT_BAD_ARGUMENT;
-    probe_link_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(in, out, n, trips, span);
-    EGPT_CHECK_LAUNCH();
-    return EGPT_OK;
-}
-
-// Measurement only: the same link, handed over through a flag in memory instead of a kernel boundary, so that a
-// link can be resident (and could have its weights on the way) while the link before still runs.  The first thread of
-// every workgroup waits until `*wait_flag` has reached `wait_count` (the number of workgroups of the link before),
-// with loads that pass the caches and at most `spin_limit` of them: a wait that runs out adds one to `*gave_up` and
-// the workgroup goes on, so that every kernel ends whatever happens.  The threads then read what the link before
-// wrote with loads that pass the caches (one L2 per XCD: a cached copy may be stale), write through them, wait for
-// their stores and add one to `*signal_flag`.
-namespace egpt {
-__global__ __launch_bounds__(256) void probe_handoff_kernel(const float* __restrict__ in, float* __restrict__ out, int n,
-                                                            const unsigned* wait_flag, unsigned wait_count,
-                                                            unsigned* signal_flag, unsigned* gave_up, int spin_limit) {
-    if (threadIdx.x == 0 && wait_flag) {
-        int spins = 0;
-        while (__hip_atomic_load(wait_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < wait_count) {
-            if (++spins >= spin_limit) {
-                atomicAdd(gave_up, 1u);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-        }
-    }
-    __syncthreads();
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
-        const float v = __hip_atomic_load(in + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(out + i, v + 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (signal_flag) {
-        __builtin_amdgcn_s_waitcnt(0);          // this thread's stores have arrived
-        __syncthreads();
-        if (threadIdx.x == 0) __hip_atomic_fetch_add(signal_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-}
-}  // namespace egpt
-
-// out[i] = in[i] + 1 for i < n.  wait_flag may be null (no wait), signal_flag may be null (no signal).
-extern "C" int egpt_probe_handoff(const float* in, float* out, int n, const unsigned* wait_flag, unsigned wait_count,
-                                  unsigned* signal_flag, unsigned* gave_up, int spin_limit, void* stream) {
-    if (!in || !out || n <= 0 || !gave_up || spin_limit < 1 || spin_limit > (1 << 22)) return EGPT_BAD_ARGUMENT;
-    probe_handoff_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(in, out, n, wait_flag, wait_count,
-                                                                                       signal_flag, gave_up, spin_limit);
-    EGPT_CHECK_LAUNCH();
-    return EGPT_OK;
-}
-
-#ifdef EGPT_TRACE
-static unsigned g_trace_next = 0;
-extern "C" unsigned egpt_trace_take(unsigned n_workgroups) {
-    const unsigned base = g_trace_next;
-    g_trace_next += n_workgroups;
-    return base;
-}
-extern "C" void egpt_trace_reset(void) { g_trace_next = 0; }
-#endif
-
 extern "C" const char* egpt_error_string(int code) {
     switch (code) {
         case EGPT_OK: return "ok";

@@ -29,10 +29,8 @@ __device__ __forceinline__ uint4 load16_if(const bf16_t* p, bool ok) {
 template <int MT, int KC, int NG>
 __global__ __launch_bounds__(64 * kGuWaves) void gemm_gate_up_kernel(const bf16_t* __restrict__ x,
                                                                      const bf16_t* __restrict__ w,
-                                                                     bf16_t* __restrict__ out, int m, int inter, int k,
-                                                                     [[maybe_unused]] unsigned trace_base) {
+                                                                     bf16_t* __restrict__ out, int m, int inter, int k) {
     __shared__ f32x4 part[kGuWaves][MT][NG][2][kWave];
-    EGPT_MARK(trace_base, 6, 0);
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int li = lane % 16, lg = lane / 16;
@@ -98,7 +96,6 @@ __global__ __launch_bounds__(64 * kGuWaves) void gemm_gate_up_kernel(const bf16_
             }
         }
     }
-    EGPT_MARK(trace_base, 6, 1);            // this wavefront's products are done: everything it loads has arrived
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -107,7 +104,6 @@ __global__ __launch_bounds__(64 * kGuWaves) void gemm_gate_up_kernel(const bf16_
             part[wave][t][g][1][lane] = acc[t][g][1];
         }
     __syncthreads();
-    EGPT_MARK(trace_base, 6, 2);            // all wavefronts' products are done
     // the wavefronts share the (row tile, column group) pairs: sums in wavefront order, the activation, one rounding
     for (int job = wave; job < MT * NG; job += kGuWaves) {
         const int t = job / NG, cg = job % NG;
@@ -131,7 +127,6 @@ __global__ __launch_bounds__(64 * kGuWaves) void gemm_gate_up_kernel(const bf16_
                 out[static_cast<size_t>(row) * inter + column] = from_float<bf16_t>(u[v] * (g[v] / (1.0f + expf(-g[v]))));
         }
     }
-    EGPT_MARK(trace_base, 6, 3);
 }
 
 template <int MT, int NG>
@@ -139,18 +134,16 @@ static void launch_gate_up(const bf16_t* x, const bf16_t* w, bf16_t* out, int m,
     const int blocks = (inter + kGuCols * NG - 1) / (kGuCols * NG);
     const int per_wave = ((k + 31) / 32 + kGuWaves - 1) / kGuWaves;
     [[maybe_unused]] const dim3 grid(blocks);
-    const unsigned trace_base = EGPT_TRACE_TAKE(grid);
     // rounds of 7 or 8 chunks: the fewer rounds, and of those the fewer registers
     if ((per_wave + 7) / 8 < (per_wave + 6) / 7)
-        gemm_gate_up_kernel<MT, 8, NG><<<blocks, 64 * kGuWaves, 0, s>>>(x, w, out, m, inter, k, trace_base);
+        gemm_gate_up_kernel<MT, 8, NG><<<blocks, 64 * kGuWaves, 0, s>>>(x, w, out, m, inter, k);
     else
-        gemm_gate_up_kernel<MT, 7, NG><<<blocks, 64 * kGuWaves, 0, s>>>(x, w, out, m, inter, k, trace_base);
+        gemm_gate_up_kernel<MT, 7, NG><<<blocks, 64 * kGuWaves, 0, s>>>(x, w, out, m, inter, k);
 }
 
 }  // namespace egpt
 
 using namespace egpt;
-EGPT_TRACE_ATTACH(gemm_gate_up)
 
 // out bfloat16 [m][inter] = SwiGLU of x w^T; x bfloat16 [m][k], w bfloat16 [2 * inter][k] (gate rows, then up rows);
 // m <= 64, k % 8 == 0.

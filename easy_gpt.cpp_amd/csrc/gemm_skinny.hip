@@ -64,7 +64,6 @@ struct SkinnyArgs {
     const float* part_o;
     const float* part_ml;
     int a_splits, nq, hd;
-    unsigned trace_base;       // builds with EGPT_TRACE: the first record of this launch's workgroups
 };
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p, bool ok) {
@@ -132,7 +131,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
     const int li = lane % 16, lg = lane / 16;
     const int split = blockIdx.y;
     const int m = a.m, n = a.n, k = a.k;
-    EGPT_MARK(a.trace_base, PRO, 0);
     const int n0 = (blockIdx.x * NW + wave) * kRowsPerWave;
     const int total_steps = (k + kStep - 1) / kStep;
     const int step_begin = split * a.steps_per_split;
@@ -378,10 +376,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
             }
         }
         __syncthreads();
-        EGPT_MARK(a.trace_base, PRO, 1);
         if (n_steps > 0) products(0, a_cur);
         if (n_steps > 1) products(1, a_next);
-        EGPT_MARK(a.trace_base, PRO, 2);
         if constexpr (PRO == kNorm) {
             if (blockIdx.x == 0 && tid < m)
                 a.ss_out[split * m + tid] = (n_steps > 0 ? ss_part[0][tid] : 0.f) + (n_steps > 1 ? ss_part[1][tid] : 0.f);
@@ -470,7 +466,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
                 if (col0 + c < n) fixed_add(a.acc_fixed + static_cast<size_t>(r) * n + col0 + c, turned[r][c]);
             }
         }
-        EGPT_MARK(a.trace_base, PRO, 3);
         return;
     }
 #pragma unroll
@@ -489,7 +484,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_skinny_kernel(SkinnyArgs a) {
                 a.out_f32[(static_cast<size_t>(split) * m + mm) * n + nn] = val;
         }
     }
-    EGPT_MARK(a.trace_base, PRO, 3);
 }
 
 // The product for 17 to 64 rows and many columns: x stays in LDS for the workgroup's whole k range (up to
@@ -595,7 +589,6 @@ static dim3 skinny_grid(int n, int n_splits, int waves) {
     do {                                                                                                     \
         const dim3 grid = skinny_grid(a.n, n_splits, waves);                                                 \
         hipStream_t s_ = static_cast<hipStream_t>(stream);                                                   \
-        a.trace_base = EGPT_TRACE_TAKE(grid);                                                                \
         if (waves == 4) gemm_skinny_kernel<MT_, PRO_, INF_, 4><<<grid, 256, 0, s_>>>(a);                     \
         else if (waves == 8) gemm_skinny_kernel<MT_, PRO_, INF_, 8><<<grid, 512, 0, s_>>>(a);                \
         else gemm_skinny_kernel<MT_, PRO_, INF_, 16><<<grid, 1024, 0, s_>>>(a);                              \
@@ -604,7 +597,6 @@ static dim3 skinny_grid(int n, int n_splits, int waves) {
 }  // namespace egpt
 
 using namespace egpt;
-EGPT_TRACE_ATTACH(gemm_skinny)
 
 // out_f32 != null: float32 [n_splits][m][n] partial sums (bias only allowed with n_splits == 1).
 // out_bf16 != null: bfloat16 [m][n], n_splits must be 1.

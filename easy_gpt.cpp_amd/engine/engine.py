@@ -60,6 +60,23 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0", allow_unexpect
     return model
 
 
+def load_random_model(config: dict, seed: int, dtype="bfloat16", device="cuda:0") -> Model:
+    """A model with the random weights that `weights.write_random_model(folder, config, seed)` would write, drawn on
+    the device and taken by the parts without a file in between (the values are the file's: a tensor's elements are
+    a function of seed, tensor name and index).  `config` is a config.json mapping."""
+    from ..config.registry import resolve_architecture
+    from ..weights.random_init import RandomWeights
+
+    arch = resolve_architecture(config)
+    cfg = arch.config_class.from_dict(config, where="config")
+    model = build_model(arch.build_spec(cfg))
+    torch_dtype = DTYPES[dtype] if isinstance(dtype, str) else dtype
+    stored = torch.bfloat16 if torch_dtype == torch.bfloat16 else torch.float32
+    model.load(RandomWeights(model.param_specs(), seed, stored, device).get, torch_dtype, torch.device(device))
+    model.config = cfg
+    return model
+
+
 class Engine:
     PAD_TO = 64          # steps that run from a padded graph are padded to a multiple of this many tokens
 

@@ -46,6 +46,7 @@ class KernelBackend:
     fuses nothing.  `kernels.hip.HipKernels` overrides them where its kernels cover the shapes."""
 
     name = "abstract"
+    max_head_dim = 256      # the widest attention head the kernels take: a part refuses more when it is built
     fused_rows = 0          # products whose x operand is computed while it is staged take at most this many rows
 
     def pinned_stream(self):

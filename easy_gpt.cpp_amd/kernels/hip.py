@@ -16,7 +16,7 @@ _F32, _BF16, _I32, _I64 = torch.float32, torch.bfloat16, torch.int32, torch.int6
 _DT = {_F32: 0, _BF16: 1}
 
 
-def _load_library(trace: bool = False) -> ctypes.CDLL:
+def _load_library() -> ctypes.CDLL:
     if not torch.cuda.is_available():
         raise KernelsUnavailable(
             "no GPU is visible to torch; this engine has no CPU path (its kernels are HIP code for gfx950)"
@@ -24,7 +24,7 @@ def _load_library(trace: bool = False) -> ctypes.CDLL:
     from ..csrc import build
 
     try:
-        path = build.ensure_trace_built() if trace else build.ensure_built()
+        path = build.ensure_built()
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
@@ -68,12 +68,9 @@ class _PinnedStream:
 class HipKernels(KernelBackend):
     name = "hip-gfx950"
 
-    def __init__(self, trace: bool = False):
-        """trace=True loads the library's variant with timestamps from inside the kernels (measurements only:
-        `trace_attach`, `trace_records`)."""
-        lib = _load_library(trace)
+    def __init__(self):
+        lib = _load_library()
         self.lib = lib
-        self.trace = bool(trace)
         self._pinned = None
         vp, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
         lib.egpt_error_string.restype = ctypes.c_char_p
@@ -103,8 +100,6 @@ class HipKernels(KernelBackend):
             "egpt_sample": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_sample_wide": [vp, vp, vp, vp, vp, vp, vp, i, i, vp],
             "egpt_gemm_gate_up_swiglu": [vp, vp, vp, i, i, i, i, vp],
-            "egpt_probe_link": [vp, vp, i, i, i, vp],
-            "egpt_probe_handoff": [vp, vp, i, vp, ctypes.c_uint, vp, vp, i, vp],
         }
         lib.egpt_sample_workspace.restype = ctypes.c_size_t
         lib.egpt_sample_workspace.argtypes = [i, i]
@@ -112,45 +107,6 @@ class HipKernels(KernelBackend):
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = i
-
-    # ------------------------------------------------------------------ timestamps from inside kernels (trace build)
-    TRACED_FILES = ("gemm_skinny", "attention_mfma", "gemm_gate_up")
-    TRACED_KERNELS = {0: "product", 1: "product, norm in front", 2: "product, SwiGLU in front",
-                      3: "product, attention parts combined in front", 5: "decode attention",
-                      6: "gate/up product with SwiGLU (first wavefront done, all done, stored)"}
-
-    def trace_attach(self, capacity: int = 1 << 20) -> torch.Tensor:
-        """Attach a buffer of `capacity` records (five int64 each) that the traced kernels write their workgroups'
-        timestamps into; returns it.  Records are numbered in the order of launches since the library was loaded,
-        so a captured graph's kernels keep their records over replays."""
-        if not self.trace:
-            raise RuntimeError("this is not the library's trace build (HipKernels(trace=True))")
-        buf = torch.zeros((capacity, 5), dtype=torch.int64, device="cuda")
-        for name in self.TRACED_FILES:
-            fn = getattr(self.lib, f"egpt_trace_attach_{name}")
-            fn.argtypes, fn.restype = [ctypes.c_void_p, ctypes.c_uint], ctypes.c_int
-            if fn(buf.data_ptr(), capacity) != 0:
-                raise RuntimeError("the trace buffer could not be attached")
-        return buf
-
-    @staticmethod
-    def trace_records(buf: torch.Tensor) -> list[dict]:
-        """The kernel launches that wrote into `buf` since it was last cleared, in order of time: for each its kernel
-        id, and per workgroup the wall clock (microseconds) and shader clock (cycles) of its four phases."""
-        rec = buf.cpu()
-        live = (rec[:, 1] != 0).nonzero().flatten().tolist()
-        rows = rec.tolist()
-        launches, cur = [], None
-        for i in live:
-            tag, *marks = rows[i]
-            kid, wg = (tag >> 48) & 0xffff, tag & 0xffffffff
-            if cur is None or wg == 0 or kid != cur["kernel"]:
-                cur = {"kernel": kid, "workgroups": []}
-                launches.append(cur)
-            cur["workgroups"].append({"us": [(m & 0xffffffff) / 100.0 for m in marks],
-                                      "cycles": [(m >> 32) & 0xffffffff for m in marks]})
-        launches.sort(key=lambda l: min(w["us"][0] for w in l["workgroups"]))
-        return launches
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -809,29 +765,6 @@ class HipKernels(KernelBackend):
             self._need(row_ss, "row_ss", _F32, (ss_splits, t))
         self._run("egpt_swiglu", gate_up.data_ptr(), splits, self._ptr(row_ss), ss_splits, int(hidden), float(eps),
                   out.data_ptr(), t, inter, dt, self._stream())
-
-    def probe_link(self, src, dst, trips=1, n=None):
-        """Measurement only: dst[:n] = src[:n] through a kernel that does next to nothing but `trips` dependent loads
-        per thread, the later ones anywhere in src."""
-        span = src.shape[0]
-        n = span if n is None else int(n)
-        self._need(src, "src", _F32, (span,))
-        self._need(dst, "dst", _F32, (span,))
-        self._run("egpt_probe_link", src.data_ptr(), dst.data_ptr(), n, int(trips), span, self._stream())
-
-    def probe_handoff(self, src, dst, n, wait_flag, wait_count, signal_flag, gave_up, stream, spin_limit=200_000):
-        """Measurement only: dst[:n] = src[:n] + 1 on `stream`, started once `wait_flag` (uint32 [1] or None) has reached
-        `wait_count`, and adding one per workgroup to `signal_flag` (or None) when done.  A wait that runs out after
-        `spin_limit` looks adds to `gave_up` and goes on."""
-        self._need(src, "src", _F32)
-        self._need(dst, "dst", _F32)
-        for name, t in (("wait_flag", wait_flag), ("signal_flag", signal_flag), ("gave_up", gave_up)):
-            if t is not None:
-                self._need(t, name, _I32, (1,))
-        if n > min(src.shape[0], dst.shape[0]):
-            raise ValueError("n is beyond the tensors")
-        self._run("egpt_probe_handoff", src.data_ptr(), dst.data_ptr(), int(n), self._ptr(wait_flag), int(wait_count),
-                  self._ptr(signal_flag), gave_up.data_ptr(), int(spin_limit), stream.cuda_stream)
 
     def argmax(self, logits, out):
         r, v = logits.shape

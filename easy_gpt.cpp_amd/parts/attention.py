@@ -40,6 +40,9 @@ class GQAttention(Mixer):
     ):
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads ({n_heads}) must be a multiple of n_kv_heads ({n_kv_heads})")
+        if not 0 < int(head_dim) <= kernels.KernelBackend.max_head_dim:
+            raise ValueError(f"head size {head_dim} is not supported by the attention kernels "
+                             f"(1 to {kernels.KernelBackend.max_head_dim})")
         self.prefix = prefix
         self.hidden_size = int(hidden_size)
         self.n_heads = int(n_heads)

@@ -21,7 +21,7 @@ DTYPES = ["float32", "bfloat16"]
 SIZES_0P5B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 896,
     "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
-    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 16384,
+    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,
     "use_sliding_window": False, "hidden_act": "silu", "torch_dtype": "bfloat16",
 }
 VOCAB = SIZES_0P5B["vocab_size"]
@@ -196,4 +196,63 @@ def test_decoding_behind_a_long_prefix_splits_the_keys_many_times(models_0p5b, d
     for rid in reqs:
         eng.finish(rid)
     compare(rows, cfg, w, reqs, tol_of(dtype), f"0.5B sizes {dtype} decoding behind 9,000 tokens")
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_behind_32000_tokens(models_0p5b, dtype):
+    # the longest context of the benchmark's record: a request of 32,000 tokens, its prompt fed in one step of that
+    # many tokens (no graph covers it) and, again, in portions of 2,048 (replayed from the graph of that size); then
+    # decoded alone (the keys split over dozens of workgroups) and beside seven requests behind 4,000 tokens
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    model_dir, cfg, w = models_0p5b(dtype)
+    n_long, n_short, n_alone, n_beside = 32000, 4000, 3, 3
+    reqs = {"long": H.make_requests(VOCAB, [n_long + n_alone + n_beside], seed=70)["r0"]}
+    for i in range(7):
+        reqs[f"s{i}"] = H.make_requests(VOCAB, [n_short - 11 * i + n_beside], seed=71 + i)["r0"]
+    eng = engine_for(model_dir, dtype, max_tokens=2 * 32768 + 7 * 4096, max_requests=9)
+    rows, fed = {}, {}
+
+    def decode(which):
+        out = eng.step([StepEntry(rid, [reqs[rid][fed[rid]]], [0]) for rid in which]).float().cpu()
+        for j, rid in enumerate(which):
+            rows[(rid, fed[rid])] = out[j].clone()
+            fed[rid] += 1
+
+    # in portions of 2,048 (a second request with the same tokens), logits at the last place and inside
+    eng.add_request("portions")
+    ids, pos = reqs["long"], 0
+    while pos < n_long:
+        step = min(2048, n_long - pos)
+        out = eng.step([StepEntry("portions", ids[pos : pos + step], [step - 1] if pos + step == n_long else [])])
+        pos += step
+    in_portions = out.float().cpu()[0].clone()
+    assert any(p.graph is not None for p in eng._padded_plans.values())
+    eng.finish("portions")
+    # in one step
+    eng.add_request("long")
+    out = eng.step([StepEntry("long", ids[:n_long], [999, n_long - 1])]).float().cpu()
+    rows[("long", 999)], rows[("long", n_long - 1)] = out[0].clone(), out[1].clone()
+    fed["long"] = n_long
+    scale = float(rows[("long", n_long - 1)].abs().max())
+    assert float((in_portions - rows[("long", n_long - 1)]).abs().max()) <= 2 * tol_of(dtype) * scale
+    for _ in range(n_alone):
+        decode(["long"])
+    for i in range(7):
+        rid = f"s{i}"
+        n = len(reqs[rid]) - n_beside
+        eng.add_request(rid)
+        for pos in range(0, n, 2048):
+            step = min(2048, n - pos)
+            out = eng.step([StepEntry(rid, reqs[rid][pos : pos + step], [step - 1] if pos + step == n else [])])
+        rows[(rid, n - 1)] = out.float().cpu()[0].clone()
+        fed[rid] = n
+    for _ in range(n_beside):
+        decode(["long"] + [f"s{i}" for i in range(7)])
+    for rid in reqs:
+        eng.finish(rid)
+    rows[("long2", n_long - 1)] = in_portions
+    reqs["long2"] = reqs["long"][:n_long]
+    compare(rows, cfg, w, reqs, tol_of(dtype), f"0.5B sizes {dtype} decoding behind 32,000 tokens")
     assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]

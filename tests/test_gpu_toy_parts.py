@@ -247,7 +247,7 @@ def test_toy_architecture_is_registered_built_and_stepped(toy_registered, tmp_pa
     from easy_gpt.cpp_amd.weights import write_random_model
 
     kernels.use_backend(None)
-    d = write_random_model(str(tmp_path / "toy"), TOY_CONFIG, seed=3)
+    d = write_random_model(str(tmp_path / "toy"), TOY_CONFIG, seed=4)
     eng = Engine.from_dir(d, dtype=dtype, device="cuda:0", page_size=4, max_tokens=256, max_requests=3)
     assert len(eng.model.cache_groups) == 1 and eng.model.cache_groups[0].cache_ids == (0, 1)
     assert list(eng.model.state_needs) == [0, 1] and eng.states.data[0].shape == (3 + 1, 48)

@@ -8,6 +8,8 @@ here and run without a change to the framework's files.
   * a mixer with per-request state that is graph-safe (it reads the state's slots and freshness from device
     memory), so that its decode steps replay from captured graphs, padding rows included;
   * a weight whose random values come from a distribution registered here (a decay within (0, 1));
+  * an embedding that adds a learned vector per position to the token's (it is handed the step context, so it finds
+    the positions there) and shares its token matrix with a tied output head;
   * a norm that the backend has no kernel for (a layer norm with mean and bias), which reads and adds to the residual
     stream through the backend whichever way the stream is kept, also inside replayed graphs.
 The toy parts compute with torch on the GPU; they are test equipment, not a model of anyone's."""
@@ -22,7 +24,7 @@ import plain_qwen2 as plain
 from easy_gpt.cpp_amd.config import Architecture, register_architecture, unregister_architecture
 from easy_gpt.cpp_amd import kernels
 from easy_gpt.cpp_amd.parts import (
-    Block, CacheNeed, LayerSpec, Mixer, ModelSpec, Norm, PagedTensor, ParamSpec, PartSpec, RunSpec, StateNeed, register_part,
+    Block, CacheNeed, Embedding, LayerSpec, Mixer, ModelSpec, Norm, PagedTensor, ParamSpec, PartSpec, RunSpec, StateNeed, register_part,
 )
 from easy_gpt.cpp_amd.parts.base import BLOCKS, MIXERS, NORMS
 from easy_gpt.cpp_amd.weights import random_init, register_role
@@ -407,3 +409,104 @@ def test_a_graph_safe_state_replays_from_graphs(toys_registered, tmp_path, dtype
     assert {key[0] for key in plans} >= {24, 3, 1} and all(p.graph is not None for key, p in plans.items() if key[0] in (24, 3))
     # the padding rows wrote the record that belongs to no request, and only that one beyond the requests' own
     assert float(eng.states.data[0][n_req].abs().max()) > 0
+
+
+# --------------------------------------------------------------------------- an embedding that looks at positions
+class PositionalEmbedding(Embedding):
+    """x_t = E[id_t] + P[position_t]; the output head may tie itself to E."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, hidden_size, vocab_size, max_position):
+        self.prefix, self.hidden_size, self.vocab_size, self.max_position = prefix, hidden_size, vocab_size, max_position
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + "tokens.weight", (self.vocab_size, self.hidden_size), role="embedding"),
+                ParamSpec(self.prefix + "positions.weight", (self.max_position, self.hidden_size), role="embedding")]
+
+    def load(self, get, dtype, device):
+        self.tokens = self._to(get(self.prefix + "tokens.weight"), "compute", dtype, device)
+        self.positions = self._to(get(self.prefix + "positions.weight"), "compute", dtype, device)
+
+    def output_matrix(self):
+        return self.tokens
+
+    def forward(self, ctx):
+        k = kernels.backend()
+        t = ctx.token_ids.shape[0]
+        out = torch.empty((t, self.hidden_size), device=ctx.token_ids.device, dtype=k.residual_dtype(t, self.tokens.dtype))
+        k.embed(ctx.token_ids, self.tokens, out)
+        k.residual_add(out, self.positions.index_select(0, ctx.positions.long()))
+        return out
+
+
+@dataclass
+class PosConfig:
+    hidden_size: int
+    vocab_size: int
+    max_position_embeddings: int
+    eps: float
+
+    @classmethod
+    def from_dict(cls, d, where="config.json"):
+        return cls(**{k: d[k] for k in cls.__dataclass_fields__})
+
+
+def pos_spec(c: PosConfig) -> ModelSpec:
+    norm = lambda p: PartSpec("rmsnorm", dict(eps=c.eps), prefix=p)
+    attn = PartSpec("gq_attention", dict(n_heads=2, n_kv_heads=1, head_dim=16, qkv_bias=True, out_bias=False, window=None,
+                                         position=PartSpec("none", {})), "l0.attn.")
+    layer = LayerSpec("pre_norm", attn, PartSpec("swiglu", dict(intermediate_size=72), prefix="l0.ff."),
+                      {"mixer": norm("l0.n1."), "feed_forward": norm("l0.n2.")})
+    return ModelSpec(hidden_size=c.hidden_size, vocab_size=c.vocab_size, max_position=c.max_position_embeddings,
+                     embedding=PartSpec("toy_positional", dict(max_position=c.max_position_embeddings), "emb."),
+                     layers=(layer,), run_order=(RunSpec(0, cache=0),), final_norm=norm("final."),
+                     output_head=PartSpec("linear_head", dict(tied=True), "head."))
+
+
+POS_CONFIG = {"architectures": ["ToyPositionalForCausalLM"], "hidden_size": 40, "vocab_size": 97,
+              "max_position_embeddings": 80, "eps": 1e-5}
+
+
+def pos_plain(w, cfg, ids):
+    s = len(ids)
+    x = w["emb.tokens.weight"][torch.tensor(ids)] + w["emb.positions.weight"][:s]
+    xn = plain.rms_norm(x, w["l0.n1.weight"], cfg["eps"])
+    p = "l0.attn."
+    q = plain.linear(xn, w[p + "q_proj.weight"], w[p + "q_proj.bias"]).reshape(s, 2, 16)
+    k = plain.linear(xn, w[p + "k_proj.weight"], w[p + "k_proj.bias"]).reshape(s, 1, 16)
+    v = plain.linear(xn, w[p + "v_proj.weight"], w[p + "v_proj.bias"]).reshape(s, 1, 16)
+    x = x + plain.linear(plain.attention(q, k, v, 2, 1).reshape(s, 32), w[p + "o_proj.weight"])
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["l0.n2.weight"], cfg["eps"]), w, "l0.ff.")
+    return plain.linear(plain.rms_norm(x, w["final.weight"], cfg["eps"]), w["emb.tokens.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_embedding_that_reads_positions_and_ties_the_output_head(tmp_path, dtype):
+    # without position encoding in the attention, the logits depend on positions through the embedding alone: tokens
+    # decoded one by one (from graphs) and in portions must get the positions they stand at
+    from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.parts.base import EMBEDDINGS
+    from easy_gpt.cpp_amd.weights import write_random_model
+
+    kernels.use_backend(None)
+    register_part("embedding", "toy_positional", PositionalEmbedding)
+    register_architecture(Architecture("ToyPositionalForCausalLM", PosConfig, pos_spec, ("toypos",)))
+    try:
+        d = write_random_model(str(tmp_path / "pos"), POS_CONFIG, seed=6)
+        eng = Engine.from_dir(d, dtype=dtype, device="cuda:0", page_size=16, max_tokens=256, max_requests=4)
+        assert eng.model.output_head.weight is eng.model.embedding.tokens and eng.model.graph_safe
+        w = plain.read_safetensors(os.path.join(d, "model.safetensors"))
+        if dtype == "bfloat16":
+            w = {k: v.float().to(torch.bfloat16).double() for k, v in w.items()}
+        reqs = H.make_requests(POS_CONFIG["vocab_size"], [50, 9, 70], seed=7)
+        ref = {rid: pos_plain(w, POS_CONFIG, ids) for rid, ids in reqs.items()}
+        shifted = pos_plain(w, POS_CONFIG, [0] + reqs["r1"])[1:]                 # the same tokens one place further on
+        assert float((shifted - ref["r1"]).abs().max()) > 1e-3 * float(ref["r1"].abs().max())
+        tol = H.FP32_TOL if dtype == "float32" else H.BF16_TOL_RANDOM
+        for trace in (H.trace_whole(reqs), H.trace_last_decoded(reqs, 32), H.trace_mixed(reqs, seed=5, max_live=3)):
+            H.assert_rows_match(H.replay(eng, trace), ref, tol, f"positional embedding {dtype}")
+        assert any(p.graph is not None for p in eng._decode_plans.values())
+    finally:
+        unregister_architecture("ToyPositionalForCausalLM")
+        EMBEDDINGS.pop("toy_positional")

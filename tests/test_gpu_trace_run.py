@@ -15,9 +15,11 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def run_trace(model_dir, dtype, trace, out_dir, max_tokens, vocab):
+def run_trace(model_dir, dtype, trace, out_dir, max_tokens, vocab, page_size=None):
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
            "--out", out_dir, "--max-tokens", str(max_tokens)]
+    if page_size is not None:
+        cmd += ["--page-size", str(page_size)]
     p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     rows, fed = {}, {}
     for rec in trace:
@@ -40,6 +42,13 @@ def run_trace(model_dir, dtype, trace, out_dir, max_tokens, vocab):
             fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
     p.stdin.close()
     assert p.wait(timeout=60) == 0
+    # the index written at the end names the same rows by (request, position)
+    with open(os.path.join(out_dir, "index.json")) as f:
+        index = json.load(f)
+    assert index["vocab"] == vocab and len(index["rows"]) == len(rows)
+    for item in index["rows"]:
+        data = np.fromfile(os.path.join(out_dir, item["file"]), dtype="<f4").reshape(-1, vocab)
+        assert torch.equal(torch.from_numpy(data[item["row"]].copy()), rows[(item["id"], item["position"])])
     return rows
 
 
@@ -53,6 +62,10 @@ def test_trace_run_mixed_trace(tiny_models, tmp_path, dtype):
     rows = run_trace(tiny_models[name], dtype, trace, str(tmp_path / "out"), H.max_live_tokens(trace, 64), cfg["vocab_size"])
     assert len(rows) > 150
     H.assert_rows_match(rows, ref, H.FP32_TOL if dtype == "float32" else H.BF16_TOL_RANDOM, f"trace_run {dtype}")
+    # a page size that is no divisor of 64 (requests counted in whole pages of it)
+    rows = run_trace(tiny_models[name], dtype, trace, str(tmp_path / "out48"), H.max_live_tokens(trace, 48), cfg["vocab_size"],
+                     page_size=48)
+    H.assert_rows_match(rows, ref, H.FP32_TOL if dtype == "float32" else H.BF16_TOL_RANDOM, f"trace_run {dtype}, pages of 48")
 
 
 def test_trace_run_whole_and_last32(tiny_models, tmp_path):

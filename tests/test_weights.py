@@ -248,3 +248,35 @@ def test_random_weights_folder(tmp_path):
     bf = write_random_model(str(tmp_path / "m4"), TINY_A, seed=0, dtype=torch.bfloat16)
     with SafetensorsFile(os.path.join(bf, "model.safetensors")) as f:
         assert f.read("model.embed_tokens.weight").dtype == torch.bfloat16
+
+
+def test_random_values_are_a_function_of_seed_name_and_index():
+    # element i of a tensor depends on (seed, tensor name, i) and on nothing else: not on the tensor's shape, not on how
+    # many elements are drawn at a time, and (integer arithmetic only) not on the device; pinned by a few values, so
+    # that a change of the generator shows
+    from easy_gpt.cpp_amd.parts.spec import ParamSpec
+    from easy_gpt.cpp_amd.weights import RandomWeights, random_init, random_tensor
+
+    a = random_tensor(ParamSpec("w", (7, 11)), seed=3, device="cpu")
+    b = random_tensor(ParamSpec("w", (77,)), seed=3, device="cpu")
+    assert torch.equal(a.flatten(), b)
+    assert not torch.equal(b, random_tensor(ParamSpec("v", (77,)), seed=3, device="cpu"))
+    chunk = random_init._CHUNK
+    try:
+        random_init._CHUNK = 13
+        assert torch.equal(b, random_tensor(ParamSpec("w", (77,)), seed=3, device="cpu"))
+    finally:
+        random_init._CHUNK = chunk
+    big = random_tensor(ParamSpec("m", (400, 500)), seed=1, device="cpu").double()
+    assert abs(float(big.mean())) < 2e-4 and abs(float(big.std()) - 0.02) < 2e-4
+    kurtosis = float((big ** 4).mean() / (big ** 2).mean() ** 2)
+    assert 2.7 < kurtosis < 3.0 and float(big.abs().max()) < 4.9 * 0.02        # a sum of eight uniforms: nearly normal
+    assert [round(v, 6) for v in big[0, :4].tolist()] == [0.03894, -0.020119, 0.008327, 0.003933]
+    table = random_tensor(ParamSpec("t", (5,), role="int_table", dtype="int32"), seed=1, device="cpu")
+    assert table.tolist() == [14619, 23638, 5612, 9413, 15729]
+    # the source without a file hands out the same tensors, in the stored dtype
+    specs = [ParamSpec("w", (7, 11)), ParamSpec("s", (9,), role="norm_scale")]
+    src = RandomWeights(specs, seed=3, dtype=torch.bfloat16, device="cpu")
+    assert torch.equal(src.get("w"), a.to(torch.bfloat16)) and src.get("s").dtype == torch.bfloat16
+    with pytest.raises(KeyError):
+        src.get("missing")
