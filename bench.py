@@ -363,7 +363,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--no-further-points", action="store_true",
                     help="skip the points at 8k and 32k prefixes and at the 1.5B and 7B layer sizes")
-    ap.add_argument("--prefill-only", action="store_true", help="only the 2,048-token prefill (for profiling)")
+    ap.add_argument("--prefill-only", action="store_true", help="only the prefill (for profiling)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="tokens of the prompt that --prefill-only feeds in one step (the record's prefill is 2,048)")
     ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
     ap.add_argument("--serve", action="store_true",
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
@@ -420,8 +422,8 @@ def main() -> int:
     if args.serve:
         max_batch, tokens_per_request = SERVE_REQUESTS, -(-(2048 + SERVE_NEW_TOKENS) // page_size) * page_size
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
-                             max_tokens=max_batch * tokens_per_request + PREFILL_TOKENS, max_requests=max_batch + 1,
-                             tune_products=not args.no_tune)
+                             max_tokens=max_batch * tokens_per_request + max(PREFILL_TOKENS, args.prefill_tokens),
+                             max_requests=max_batch + 1, tune_products=not args.no_tune)
     sampler = Sampler(engine.device)
     g = torch.Generator().manual_seed(0)
     print(f"[bench] model ready in {time.time() - t_setup:.1f} s", file=sys.stderr, flush=True)
@@ -447,12 +449,13 @@ def main() -> int:
     # ---------------------------------------------------------------- prefill of 2,048 tokens, one request, one step
     prefill = None
     if not args.no_points or args.prefill_only:
-        sec = prefill_seconds(engine, vocab, PREFILL_TOKENS, g)
-        prefill = {"value": round(PREFILL_TOKENS / sec, 1), "tokens": PREFILL_TOKENS, "ms": round(sec * 1e3, 3),
-                   "frac": round(prefill_flops(PREFILL_TOKENS) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
+        n_prompt = args.prefill_tokens if args.prefill_only else PREFILL_TOKENS
+        sec = prefill_seconds(engine, vocab, n_prompt, g, reps=10 if n_prompt <= 8192 else 3)
+        prefill = {"value": round(n_prompt / sec, 1), "tokens": n_prompt, "ms": round(sec * 1e3, 3),
+                   "frac": round(prefill_flops(n_prompt) / sec / (PEAK_TFLOPS[dtype_key] * 1e12), 5)}
         print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     if args.prefill_only:
-        print(json.dumps({"metric": f"prefill tok/s at 2,048 tokens ({name})", "prefill": prefill}), flush=True)
+        print(json.dumps({"metric": f"prefill tok/s at {n_prompt:,} tokens ({name})", "prefill": prefill}), flush=True)
         remove_folder(tmp)
         return 0
 

@@ -14,6 +14,8 @@
 // (as /root/reference/src/cuda/ops/self_attn_detail.cuh:299-383); P is rounded to bfloat16 for the
 // second product.  With n_splits > 1 each split of the key range writes an unnormalised partial result
 // and its (maximum, sum), which attention_reduce_kernel combines.
+#include <type_traits>
+
 #include "api.h"
 #include "common.h"
 
@@ -335,7 +337,15 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
     f32x4 o[DT];
 #pragma unroll
     for (int d = 0; d < DT; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;     // the maximum in units of the raw scores
+    float m_run = -INFINITY;                  // the maximum in units of the raw scores
+    // The rows' sums of probabilities are left to the matrix cores: one more tile of "values" whose first feature is
+    // all ones (lanes lj == 0 hold it, the other features are zeros) gives sum_key P[key, row] as feature 0 of a
+    // 17th output tile, in element 0 of the lanes lg == 0.  (Sixteen additions per step on the vector pipe, which is
+    // what this kernel waits for, against two matrix instructions on a pipe that is idle seven eighths of the time.)
+    f32x4 o_sum = f32x4{0.f, 0.f, 0.f, 0.f};
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(lj == 0 ? 1.0f : 0.0f);
 
     // The loads of a tile go through three stages, each one iteration ahead of the next, so that no load
     // waits for another inside an iteration: page numbers (tile + 2), keys and values into registers
@@ -372,21 +382,22 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
             for (int u = 0; u < CH; ++u) v_regs[u] = uint4{0u, 0u, 0u, 0u};
         }
     };
-    auto stash = [&](int stage) {
+    // Where this thread puts its chunks, and where this lane reads its operands, in either stage: the loop below is
+    // unrolled over the two stages, so that every LDS access is one of these registers plus an immediate offset.
+    bf16_t* const k_put[2] = {ks_at(0, k_row, k_col), ks_at(1, k_row, k_col)};
+    bf16_t* const v_put[2] = {vs_at(0, v_row, v_key), vs_at(1, v_row, v_key)};
+    const bf16_t* const k_get[2] = {ks_at(0, ksi * 64 + lj, lg * 8), ks_at(1, ksi * 64 + lj, lg * 8)};
+    const bf16_t* const v_get[2] = {vs_at(0, lj, ksi * 64 + lg * 4), vs_at(1, lj, ksi * 64 + lg * 4)};
+    auto stash = [&](auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
-            *reinterpret_cast<uint4*>(ks_at(stage, k_row, k_col + u * 8)) = k_regs[u];
-            *reinterpret_cast<uint4*>(vs_at(stage, v_row + u * 8 * RT, v_key)) = v_regs[u];
+            *reinterpret_cast<uint4*>(k_put[stage] + u * 8) = k_regs[u];
+            *reinterpret_cast<uint4*>(v_put[stage] + u * 8 * RT * VROW) = v_regs[u];
         }
     };
-
-    lookup(t_begin);
-    fetch(t_begin);
-    lookup(t_begin + 1);
-    stash(0);
-    __syncthreads();
-    for (int tile = t_begin; tile < t_end; ++tile) {
-        const int stage = (tile - t_begin) & 1;
+    auto walk = [&](auto stage_c, int tile) {
+        constexpr int stage = decltype(stage_c)::value;
         fetch(tile + 1);           // past the last tile every page number is -1: nothing is read
         lookup(tile + 2);
         const int key0 = tile * KT + ksi * 64;       // this wavefront's 64 keys
@@ -398,7 +409,7 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
                 acc[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
-                    const uint4 kk = *reinterpret_cast<const uint4*>(ks_at(stage, ksi * 64 + kt * 16 + lj, kd * 32 + lg * 8));
+                    const uint4 kk = *reinterpret_cast<const uint4*>(k_get[stage] + kt * 16 * KROW + kd * 32);
                     acc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kk), q[kd], acc[kt], 0, 0, 0);
                 }
             }
@@ -420,7 +431,7 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
             if (__any(m_new != m_run)) {             // some row's maximum moved: rescale what is accumulated
                 const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
-                l_run *= alpha;
+                o_sum[0] *= alpha;
 #pragma unroll
                 for (int d = 0; d < DT; ++d) {
                     o[d][0] *= alpha; o[d][1] *= alpha; o[d][2] *= alpha; o[d][3] *= alpha;
@@ -428,34 +439,40 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
                 m_run = m_new;
             }
             const float shift = -m_use * scale2;
-            float sum = 0.f;
             bf16x8 pb[2];
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float pv = __builtin_amdgcn_exp2f(fmaf(acc[kt][v], scale2, shift));
-                    sum += pv;
-                    pb[kt / 2][(kt % 2) * 4 + v] = static_cast<__bf16>(pv);
-                }
-            l_run += sum;
-            // O^T += V^T P^T, two products of 32 keys per 16 features
+                for (int v = 0; v < 4; ++v)
+                    pb[kt / 2][(kt % 2) * 4 + v] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(acc[kt][v], scale2, shift)));
+            // O^T += V^T P^T, two products of 32 keys per 16 features, and the tile of ones for the rows' sums
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) o_sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[kb], o_sum, 0, 0, 0);
 #pragma unroll
             for (int d = 0; d < DT; ++d)
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
-                    const uint2 v0 = *reinterpret_cast<const uint2*>(vs_at(stage, d * 16 + lj, ksi * 64 + kb * 32 + lg * 4));
-                    const uint2 v1 = *reinterpret_cast<const uint2*>(vs_at(stage, d * 16 + lj, ksi * 64 + kb * 32 + 16 + lg * 4));
+                    const uint2 v0 = *reinterpret_cast<const uint2*>(v_get[stage] + d * 16 * VROW + kb * 32);
+                    const uint2 v1 = *reinterpret_cast<const uint2*>(v_get[stage] + d * 16 * VROW + kb * 32 + 16);
                     const uint4 a = uint4{v0.x, v0.y, v1.x, v1.y};
                     o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), pb[kb], o[d], 0, 0, 0);
                 }
         }
-        stash(stage ^ 1);
+        stash(std::integral_constant<int, stage ^ 1>{});
         __syncthreads();
+    };
+
+    lookup(t_begin);
+    fetch(t_begin);
+    lookup(t_begin + 1);
+    stash(std::integral_constant<int, 0>{});
+    __syncthreads();
+    for (int tile = t_begin; tile < t_end; tile += 2) {
+        walk(std::integral_constant<int, 0>{}, tile);
+        if (tile + 1 < t_end) walk(std::integral_constant<int, 1>{}, tile + 1);
     }
-    float l = l_run;
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
+    // the row's sum: feature 0 of the tile of ones, which the lane lj of the first quarter holds
+    float l = __shfl(o_sum[0], lj, kWave);
     if constexpr (KS > 1) {
         // The wavefronts of one row tile hold partial results over their keys: those with ks > 0 leave
         // theirs in LDS (the tiles are no longer read: the loop ended with a barrier), ks == 0 adds them up.
@@ -504,6 +521,294 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
             packed.y = f32_to_bf16_bits(o[d][2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[d][3] * inv)) << 16);
             *reinterpret_cast<uint2*>(op + d * 16) = packed;
         }
+    }
+}
+
+// Prompt portions, 32 rows to a wavefront.  The same arithmetic as attention_tiled_kernel with the 32 x 32 x 16 matrix
+// instruction: a wavefront takes a block of 32 rows and 64 keys of each tile, S^T[32 keys, 32 rows] = K Q^T leaves a lane
+// 16 scores of one row (row = lane % 32; the lane's half h = lane / 32 holds keys 8b + 4h + v of a block of 32, b and v
+// in 0..3), and the probabilities are again the second product's operand as they lie: for its step over 16 keys a lane
+// supplies eight of them, the same eight that it holds, so a page's values are staged into LDS in that order (within 16
+// keys: [h][b % 2][v]).  Against the kernel of 16-row tiles, a score costs half the matrix instructions, half the LDS
+// reads and half the staging and loop instructions; what is left per score is its exponential, a multiply-add, a
+// maximum and half a conversion, which is the vector pipe's floor for a softmax in float32.  A workgroup takes RB blocks
+// of rows; KS wavefronts per block split each tile of 64 * KS keys and are combined through LDS at the end.
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// max(a, b, c) in one instruction.  (fmaxf quiets signalling NaNs first, which costs an instruction per operand that
+// comes from the matrix cores; scores are never NaN here.)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+template <int HD, int RB, int KS>
+__global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
+    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window) {
+    constexpr int NQ = HD / 16;                  // steps of 16 features of the score product
+    constexpr int FB = HD / 32;                  // blocks of 32 output features
+    constexpr int ROWS = 32 * RB;
+    constexpr int KT = 64 * KS;                  // keys per LDS tile
+    constexpr int KROW = HD + 8, VROW = KT + 8;  // padded rows (bf16 elements)
+    constexpr int THREADS = 64 * RB * KS;
+    constexpr int CH = HD / (8 * RB);            // 16-byte chunks per thread and tile, of keys and of values
+    constexpr int STAGE = KT * KROW + HD * VROW;
+    constexpr int PER_LANE = FB * 16 + 2;        // floats a lane leaves for the combination
+    constexpr int COMBINE = (KS - 1) * RB * 64 * PER_LANE * 2;    // in bf16 elements
+    static_assert(CH >= 1 && HD % (8 * RB) == 0, "a thread takes whole chunks");
+    __shared__ __attribute__((aligned(16))) bf16_t smem[(2 * STAGE > COMBINE) ? 2 * STAGE : COMBINE];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int rb = wave % RB, ksi = wave / RB;
+    const int lr = lane % 32, lh = lane / 32;
+    const int kh = blockIdx.y;
+    const int group_size = nq / nkv;
+
+    int b = 0, grp = blockIdx.x;
+    for (; b < n_seqs; ++b) {
+        const int groups = (q_len[b] * group_size + ROWS - 1) / ROWS;
+        if (grp < groups) {
+            grp = groups - 1 - grp;          // the last rows first: they have the most keys to walk
+            break;
+        }
+        grp -= groups;
+    }
+    if (b >= n_seqs) return;
+    const int n = q_len[b], kv = kv_len[b], qs = q_start[b];
+    const int rows = n * group_size;
+    const int width = (nq + 2 * nkv) * HD;
+    const int32_t* table = block_table + static_cast<size_t>(b) * table_width;
+
+    // the workgroup's rows and the keys they need
+    const int blk_first = grp * ROWS, blk_last = min(rows, blk_first + ROWS) - 1;
+    const int blk_p_hi = kv - n + blk_last / group_size;
+    const int blk_first_pos = kv - n + blk_first / group_size;
+    const int blk_lo = window > 0 ? max(0, blk_first_pos - window + 1) : 0;
+    const int t_begin = blk_lo / KT, t_end = blk_p_hi / KT + 1;
+
+    // this wavefront's block of 32 rows, this lane's row
+    const int row_base = blk_first + rb * 32;
+    const int r = row_base + lr;
+    const bool valid = r < rows;
+    const int i_tok = valid ? r / group_size : 0;
+    const int tok = qs + i_tok;
+    const int head = kh * group_size + (valid ? r % group_size : 0);
+    const int p_row = valid ? kv - n + i_tok : -1;
+    const int lo_row = (window > 0 && valid) ? max(0, p_row - window + 1) : 0;
+    const bool wave_any = row_base < rows;
+    const int w_last = min(rows, row_base + 32) - 1;
+    const int w_p_hi = wave_any ? kv - n + w_last / group_size : -1;       // largest causal limit in the block
+    const int w_p_min = wave_any ? kv - n + row_base / group_size : -1;    // smallest
+    const int w_lo_first = (window > 0 && wave_any) ? max(0, w_p_min - window + 1) : 0;
+    const int w_lo_max = (window > 0 && wave_any) ? max(0, w_p_hi - window + 1) : 0;
+    bf16x8 q[NQ];
+    {
+        const bf16_t* qp = qkv + static_cast<size_t>(tok) * width + head * HD + lh * 8;
+#pragma unroll
+        for (int j = 0; j < NQ; ++j) {
+            const uint4 v = valid ? *reinterpret_cast<const uint4*>(qp + j * 16) : uint4{0u, 0u, 0u, 0u};
+            q[j] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    const float scale2 = scale * 1.4426950408889634f;
+
+    f32x16 o[FB];
+#pragma unroll
+    for (int f = 0; f < FB; ++f)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[f][e] = 0.f;
+    float m_run = -INFINITY;                  // the maximum in units of the raw scores
+    // the rows' sums of probabilities come from the matrix cores: a block of "values" whose first feature is all ones
+    // (the lanes lane % 32 == 0 hold it) gives them as feature 0 of one more output block, element 0 of the lanes of
+    // half 0 (32 additions per step on the vector pipe, which this kernel waits for, against four matrix instructions)
+    f32x16 o_sum;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_sum[e] = 0.f;
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = static_cast<__bf16>(lr == 0 ? 1.0f : 0.0f);
+    f32x16 zero16;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) zero16[e] = 0.f;
+
+    const int page_mask = page_size - 1;             // page sizes here are powers of two
+    const int k_row = tid / RB, k_col = (tid % RB) * CH * 8;                 // key within the tile, first feature
+    const int v_key = (tid % (KT / 8)) * 8, v_row = tid / (KT / 8);          // first of eight keys, feature (+ 8 RB u)
+    // where a run of eight keys goes within its 16 keys of a value row: the first four to half 0, the others to half 1
+    const int v_pos = (v_key / 16) * 16 + ((v_key % 16) / 8) * 4;
+    uint4 k_regs[CH], v_regs[CH];
+    int k_page, v_page;                              // -1: nothing to read (zeros)
+    auto lookup = [&](int tile) {
+        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
+        k_page = (kk <= blk_p_hi && kk >= blk_lo) ? table[kk >> page_shift] : -1;
+        v_page = (vk <= blk_p_hi && vk + 7 >= blk_lo) ? table[vk >> page_shift] : -1;
+    };
+    auto fetch = [&](int tile) {
+        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
+        if (k_page >= 0) {
+            const bf16_t* src = k_cache + ((static_cast<long>(k_page) * nkv + kh) * page_size + (kk & page_mask)) * HD + k_col;
+#pragma unroll
+            for (int u = 0; u < CH; ++u) k_regs[u] = *reinterpret_cast<const uint4*>(src + u * 8);
+        } else {
+#pragma unroll
+            for (int u = 0; u < CH; ++u) k_regs[u] = uint4{0u, 0u, 0u, 0u};
+        }
+        if (v_page >= 0) {
+            const bf16_t* src = v_cache + ((static_cast<long>(v_page) * nkv + kh) * HD + v_row) * page_size + (vk & page_mask);
+#pragma unroll
+            for (int u = 0; u < CH; ++u)
+                v_regs[u] = *reinterpret_cast<const uint4*>(src + static_cast<long>(u) * (8 * RB) * page_size);
+        } else {
+#pragma unroll
+            for (int u = 0; u < CH; ++u) v_regs[u] = uint4{0u, 0u, 0u, 0u};
+        }
+    };
+    bf16_t* const k_put[2] = {smem + k_row * KROW + k_col, smem + STAGE + k_row * KROW + k_col};
+    bf16_t* const v_put[2] = {smem + KT * KROW + v_row * VROW + v_pos, smem + STAGE + KT * KROW + v_row * VROW + v_pos};
+    const bf16_t* const k_get[2] = {smem + (ksi * 64 + lr) * KROW + lh * 8, smem + STAGE + (ksi * 64 + lr) * KROW + lh * 8};
+    const bf16_t* const v_get[2] = {smem + KT * KROW + lr * VROW + ksi * 64 + lh * 8,
+                                    smem + STAGE + KT * KROW + lr * VROW + ksi * 64 + lh * 8};
+    auto stash = [&](auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+            *reinterpret_cast<uint4*>(k_put[stage] + u * 8) = k_regs[u];
+            bf16_t* vp = v_put[stage] + u * 8 * RB * VROW;
+            *reinterpret_cast<uint2*>(vp) = uint2{v_regs[u].x, v_regs[u].y};
+            *reinterpret_cast<uint2*>(vp + 8) = uint2{v_regs[u].z, v_regs[u].w};
+        }
+    };
+    auto walk = [&](auto stage_c, int tile) {
+        constexpr int stage = decltype(stage_c)::value;
+        fetch(tile + 1);           // past the last tile every page number is -1: nothing is read
+        lookup(tile + 2);
+        const int key0 = tile * KT + ksi * 64;       // this wavefront's 64 keys
+        if (wave_any && key0 <= w_p_hi && key0 + 63 >= w_lo_first) {     // else nothing visible to these rows
+            f32x16 acc[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int j = 0; j < NQ; ++j) {
+                    const uint4 kk = *reinterpret_cast<const uint4*>(k_get[stage] + kb * 32 * KROW + j * 16);
+                    acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), q[j],
+                                                                      j == 0 ? zero16 : acc[kb], 0, 0, 0);
+                }
+            }
+            if (!(key0 + 63 <= w_p_min && key0 >= w_lo_max)) {           // on the diagonal or the window's edge
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = key0 + kb * 32 + (e / 4) * 8 + lh * 4 + e % 4;
+                        if (!(key <= p_row && key >= lo_row)) acc[kb][e] = -INFINITY;
+                    }
+            }
+            float mx = max3(acc[0][0], acc[0][1], acc[0][2]), mx1 = max3(acc[1][0], acc[1][1], acc[1][2]);
+#pragma unroll
+            for (int e = 3; e < 15; e += 2) {
+                mx = max3(mx, acc[0][e], acc[0][e + 1]);
+                mx1 = max3(mx1, acc[1][e], acc[1][e + 1]);
+            }
+            mx = max3(mx, mx1, acc[0][15]);
+            mx = fmaxf(mx, acc[1][15]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+            const float m_new = fmaxf(m_run, mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            if (__any(m_new != m_run)) {             // some row's maximum moved: rescale what is accumulated
+                const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
+                o_sum[0] *= alpha;
+#pragma unroll
+                for (int f = 0; f < FB; ++f)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[f][e] *= alpha;
+                m_run = m_new;
+            }
+            const float shift = -m_use * scale2;
+            // the second product's steps of 16 keys: step t takes elements 8 (t % 2) .. + 7 of block t / 2 from a lane
+            bf16x8 pb[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    pb[t][e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(acc[t / 2][(t % 2) * 8 + e], scale2, shift)));
+#pragma unroll
+            for (int t = 0; t < 4; ++t) o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[t], o_sum, 0, 0, 0);
+#pragma unroll
+            for (int f = 0; f < FB; ++f)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const uint4 a = *reinterpret_cast<const uint4*>(v_get[stage] + f * 32 * VROW + t * 16);
+                    o[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb[t], o[f], 0, 0, 0);
+                }
+        }
+        stash(std::integral_constant<int, stage ^ 1>{});
+        __syncthreads();
+    };
+
+    lookup(t_begin);
+    fetch(t_begin);
+    lookup(t_begin + 1);
+    stash(std::integral_constant<int, 0>{});
+    __syncthreads();
+    for (int tile = t_begin; tile < t_end; tile += 2) {
+        walk(std::integral_constant<int, 0>{}, tile);
+        if (tile + 1 < t_end) walk(std::integral_constant<int, 1>{}, tile + 1);
+    }
+    // the row's sum: feature 0 of the block of ones, which lane lr of half 0 holds
+    float l = __shfl(o_sum[0], lr, kWave);
+    if constexpr (KS > 1) {
+        // The wavefronts of one block of rows hold partial results over their keys: those with ks > 0 leave
+        // theirs in LDS (the tiles are no longer read: the loop ended with a barrier), ks == 0 adds them up.
+        float* comb = reinterpret_cast<float*>(smem);
+        if (ksi > 0) {
+            float* dst = comb + (static_cast<size_t>((ksi - 1) * RB + rb) * PER_LANE) * 64 + lane;
+#pragma unroll
+            for (int f = 0; f < FB; ++f)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) dst[(f * 16 + e) * 64] = o[f][e];
+            dst[(FB * 16) * 64] = m_run;
+            dst[(FB * 16 + 1) * 64] = l;
+        }
+        __syncthreads();
+        if (ksi > 0) return;
+        float m_all = m_run;
+#pragma unroll
+        for (int j = 0; j < KS - 1; ++j)
+            m_all = fmaxf(m_all, comb[(static_cast<size_t>(j * RB + rb) * PER_LANE + FB * 16) * 64 + lane]);
+        const float m_ref = m_all == -INFINITY ? 0.f : m_all;
+        const float w0 = __builtin_amdgcn_exp2f((m_run - m_ref) * scale2);
+        l *= w0;
+#pragma unroll
+        for (int f = 0; f < FB; ++f)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[f][e] *= w0;
+#pragma unroll
+        for (int j = 0; j < KS - 1; ++j) {
+            const float* src = comb + (static_cast<size_t>(j * RB + rb) * PER_LANE) * 64 + lane;
+            const float wj = __builtin_amdgcn_exp2f((src[(FB * 16) * 64] - m_ref) * scale2);
+            l += src[(FB * 16 + 1) * 64] * wj;
+#pragma unroll
+            for (int f = 0; f < FB; ++f)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[f][e] += src[(f * 16 + e) * 64] * wj;
+        }
+    }
+    if (valid) {
+        // element e of block f is feature f * 32 + (e / 4) * 8 + lh * 4 + e % 4: runs of four features
+        const float inv = 1.0f / l;
+        bf16_t* op = out + (static_cast<size_t>(tok) * nq + head) * HD + lh * 4;
+#pragma unroll
+        for (int f = 0; f < FB; ++f)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 packed;
+                packed.x = f32_to_bf16_bits(o[f][g * 4] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[f][g * 4 + 1] * inv)) << 16);
+                packed.y = f32_to_bf16_bits(o[f][g * 4 + 2] * inv) | (static_cast<uint32_t>(f32_to_bf16_bits(o[f][g * 4 + 3] * inv)) << 16);
+                *reinterpret_cast<uint2*>(op + f * 32 + g * 8) = packed;
+            }
     }
 }
 
@@ -1012,6 +1317,19 @@ static void launch_tiled(const void* qkv, void* out, const void* k_cache, const 
         page_size, page_shift, scale, window);
 }
 
+template <int HD, int RB, int KS>
+static void launch_rows32(const void* qkv, void* out, const void* k_cache, const void* v_cache,
+                          const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
+                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size,
+                          int page_shift, float scale, int window, hipStream_t s) {
+    const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (32 * RB) + n_seqs;   // upper bound
+    dim3 grid(static_cast<unsigned>(groups), nkv);
+    attention_rows32_kernel<HD, RB, KS><<<grid, 64 * RB * KS, 0, s>>>(
+        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
+        static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
+        page_size, page_shift, scale, window);
+}
+
 extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                                           const int32_t* block_table, int table_width, const int32_t* q_start,
                                           const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens,
@@ -1030,9 +1348,18 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
 #define EGPT_TILED(HD_, RT_, KS_)                                                                                  \
     launch_tiled<HD_, RT_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,      \
                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, s)
-    // shape = 10 * row tiles + key splits of a workgroup
+#define EGPT_ROWS32(HD_, RB_, KS_)                                                                                 \
+    launch_rows32<HD_, RB_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,     \
+                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, s)
+    // shape = 10 * row tiles + key splits of a workgroup; 100 + 10 * blocks of 32 rows + key splits: the kernel of
+    // 32-row blocks
     if (hd == 64) {
         switch (shape) {
+            case 121: EGPT_ROWS32(64, 2, 1); break;
+            case 122: EGPT_ROWS32(64, 2, 2); break;
+            case 124: EGPT_ROWS32(64, 2, 4); break;
+            case 141: EGPT_ROWS32(64, 4, 1); break;
+            case 142: EGPT_ROWS32(64, 4, 2); break;
             case 41: EGPT_TILED(64, 4, 1); break;
             case 42: EGPT_TILED(64, 4, 2); break;
             case 44: EGPT_TILED(64, 4, 4); break;
@@ -1042,6 +1369,9 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
         }
     } else {
         switch (shape) {
+            case 121: EGPT_ROWS32(128, 2, 1); break;
+            case 122: EGPT_ROWS32(128, 2, 2); break;
+            case 141: EGPT_ROWS32(128, 4, 1); break;
             case 41: EGPT_TILED(128, 4, 1); break;
             case 42: EGPT_TILED(128, 4, 2); break;
             case 22: EGPT_TILED(128, 2, 2); break;
@@ -1049,6 +1379,7 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
         }
     }
 #undef EGPT_TILED
+#undef EGPT_ROWS32
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }

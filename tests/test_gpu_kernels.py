@@ -694,7 +694,8 @@ def test_float32_attention_gives_the_same_bits_however_the_rows_are_cut(k, hd, p
     assert torch.equal(single, whole[3 : 3 + n])
 
 
-@pytest.mark.parametrize("hd,shape", [(64, 41), (64, 42), (64, 44), (64, 22), (64, 24), (128, 41), (128, 42), (128, 22)])
+@pytest.mark.parametrize("hd,shape", [(64, 41), (64, 42), (64, 44), (64, 22), (64, 24), (128, 41), (128, 42), (128, 22),
+                                      (64, 121), (64, 122), (64, 124), (64, 141), (64, 142), (128, 121), (128, 122), (128, 141)])
 @pytest.mark.parametrize("window,ps", [(0, 16), (0, 64), (100, 32), (300, 16)])
 def test_paged_attention_tiled_workgroup_shapes(k, hd, shape, window, ps):
     # every workgroup shape of the LDS-tiled kernel (row tiles x key splits): prompts over several row groups and
@@ -704,7 +705,7 @@ def test_paged_attention_tiled_workgroup_shapes(k, hd, shape, window, ps):
     assert run_paged(k, seqs, 7, 1, hd, ps, torch.bfloat16, window=window, tiled_shape=shape, q_scale=6.0, seed=3) <= 4e-2
 
 
-@pytest.mark.parametrize("hd,shape", [(64, None), (64, 44), (128, None), (128, 41)])
+@pytest.mark.parametrize("hd,shape", [(64, None), (64, 44), (128, None), (128, 41), (64, 142), (64, 124), (128, 122)])
 @pytest.mark.parametrize("window", [0, 4099])
 def test_paged_attention_long_prefixes(k, hd, shape, window):
     # prompt portions behind thousands of cached keys: many key tiles for each row tile, block tables hundreds of pages wide
