@@ -606,6 +606,12 @@ class HipKernels(KernelBackend):
                     shape = 24 if hd == 64 else 22
                 elif row_tiles <= 2048:
                     shape = 44 if hd == 64 else 42
+                elif hd == 64 and row_tiles > 4096:
+                    # many rows of head size 64: the kernel of 32-row blocks (measured at 14 query heads on 2: 8,192
+                    # tokens in 239 us against 292, 32,640 in 3.26 ms against 3.84; 2,048 tokens, 1,792 tiles, are
+                    # faster in 16-row tiles, 32.1 us against 32.9; at head size 128 its registers leave a SIMD one
+                    # wavefront and it loses everywhere: 564 us against 527 for 8,192 tokens of 12 heads on 2)
+                    shape = 142
                 else:
                     shape = 42
                 self._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(),
