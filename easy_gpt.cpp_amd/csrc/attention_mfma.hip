@@ -531,9 +531,15 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
 // supplies eight of them, the same eight that it holds, so a page's values are staged into LDS in that order (within 16
 // keys: [h][b % 2][v]).  Against the kernel of 16-row tiles, a score costs half the matrix instructions, half the LDS
 // reads and half the staging and loop instructions; what is left per score is its exponential, a multiply-add, a
-// maximum and half a conversion, which is the vector pipe's floor for a softmax in float32.  A workgroup takes RB blocks
-// of rows; KS wavefronts per block split each tile of 64 * KS keys and are combined through LDS at the end.
+// maximum and half a conversion, and the kernel is bound by the issue of these vector instructions (an exponential
+// takes a wavefront's issue slot for about 8.5 cycles, the others for 4.4, a matrix instruction for 8 of its 32: with
+// 32 scores to a lane and tile that is about 1,000 cycles a wavefront and tile, against 640 of the matrix cores), so
+// the loop below is built to keep the vector pipe issuing while the matrix cores work.  A workgroup takes RB blocks
+// of rows; KS wavefronts per block split each tile of 64 * KS keys and are combined through LDS at the end.  The tiles
+// of 64 keys must be whole pages (page sizes 16, 32, 64).
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;      // (native vectors: arrays of them stay in registers)
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 // max(a, b, c) in one instruction.  (fmaxf quiets signalling NaNs first, which costs an instruction per operand that
 // comes from the matrix cores; scores are never NaN here.)
@@ -634,129 +640,228 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) zero16[e] = 0.f;
 
+    // The loop is a pipeline of three stages over the tiles.  In the iteration of tile i a wavefront issues, as one
+    // straight line of code, the score product of tile i + 1, the exponentials of tile i and the output product of tile
+    // i - 1: the matrix instructions of the two products alternate with the vector instructions of the softmax between
+    // them, so that both pipes work at once.  (With a tile's products on either side of its softmax, and the
+    // wavefronts of a workgroup in step from barrier to barrier, the pipes took turns: at 8,192 tokens the SIMDs issued
+    // vector instructions half of the time and did nothing for much of the rest.)  What does not fit into a straight
+    // line is kept out of it: masking (tiles on the diagonal or a window's edge) comes before it, and the accumulated
+    // output is rescaled after it, and only when a row's maximum has grown by more than 2^kSlack since the last time:
+    // until then the exponentials are taken against the old maximum, so they may reach 2^kSlack instead of 1, which
+    // float32 sums and bfloat16 probabilities (the same relative precision at any magnitude) do not mind.
+    // LDS holds the keys of tiles i + 1 and i + 2 and the values of tiles i - 1 and i, two slots each; the keys of tile
+    // i + 3 and the values of tile i + 1 are on their way from memory meanwhile.
+    constexpr float kSlack = 8.0f;
     const int page_mask = page_size - 1;             // page sizes here are powers of two
     const int k_row = tid / RB, k_col = (tid % RB) * CH * 8;                 // key within the tile, first feature
     const int v_key = (tid % (KT / 8)) * 8, v_row = tid / (KT / 8);          // first of eight keys, feature (+ 8 RB u)
     // where a run of eight keys goes within its 16 keys of a value row: the first four to half 0, the others to half 1
     const int v_pos = (v_key / 16) * 16 + ((v_key % 16) / 8) * 4;
-    uint4 k_regs[CH], v_regs[CH];
-    int k_page, v_page;                              // -1: nothing to read (zeros)
-    auto lookup = [&](int tile) {
-        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
-        k_page = (kk <= blk_p_hi && kk >= blk_lo) ? table[kk >> page_shift] : -1;
-        v_page = (vk <= blk_p_hi && vk + 7 >= blk_lo) ? table[vk >> page_shift] : -1;
+    // Loads without branches, so that they can stand in the straight line: a thread's key row and its run of eight
+    // values lie at the same place of their page in every tile (a tile is whole pages), so a load's address is the
+    // page's number times the pages' stride plus a constant of the thread.  The index into the block table is clamped
+    // to the pages that hold the workgroup's keys, so every load reads memory of this request; what lies outside the
+    // keys that the rows see is replaced by zeros when a tile at either end is put into LDS.
+    u32x4 k_regs[CH], v_regs[CH];
+    int k_page, v_page;
+    const long page_stride = static_cast<long>(nkv) * page_size * HD;
+    const bf16_t* const k_base = k_cache + (static_cast<long>(kh) * page_size + (k_row & page_mask)) * HD + k_col;
+    const bf16_t* const v_base = v_cache + (static_cast<long>(kh) * HD + v_row) * page_size + (v_key & page_mask);
+    const int idx_lo = blk_lo >> page_shift, idx_hi = blk_p_hi >> page_shift, idx_step = KT >> page_shift;
+    const int k_sub = k_row >> page_shift, v_sub = v_key >> page_shift;
+    auto clamped = [&](int idx) { return min(max(idx, idx_lo), idx_hi); };
+    auto lookup_k = [&](int tile) { k_page = max(table[clamped(tile * idx_step + k_sub)], 0); };
+    auto lookup_v = [&](int tile) { v_page = max(table[clamped(tile * idx_step + v_sub)], 0); };
+    auto fetch_k = [&]() {
+        const bf16_t* src = k_base + k_page * page_stride;
+#pragma unroll
+        for (int u = 0; u < CH; ++u) k_regs[u] = *reinterpret_cast<const u32x4*>(src + u * 8);
     };
-    auto fetch = [&](int tile) {
-        const int kk = tile * KT + k_row, vk = tile * KT + v_key;
-        if (k_page >= 0) {
-            const bf16_t* src = k_cache + ((static_cast<long>(k_page) * nkv + kh) * page_size + (kk & page_mask)) * HD + k_col;
+    auto fetch_v = [&]() {
+        const bf16_t* src = v_base + v_page * page_stride;
 #pragma unroll
-            for (int u = 0; u < CH; ++u) k_regs[u] = *reinterpret_cast<const uint4*>(src + u * 8);
-        } else {
+        for (int u = 0; u < CH; ++u)
+            v_regs[u] = *reinterpret_cast<const u32x4*>(src + static_cast<long>(u) * (8 * RB) * page_size);
+    };
+    auto at_an_end = [&](int tile) { return tile * KT < blk_lo || tile * KT + KT - 1 > blk_p_hi; };
+    auto trim_k = [&](int tile) {            // zeros for the keys of this tile that no row of the workgroup sees
+        if (at_an_end(tile)) {
+            const int kk = tile * KT + k_row;
+            if (!(kk <= blk_p_hi && kk >= blk_lo)) {
 #pragma unroll
-            for (int u = 0; u < CH; ++u) k_regs[u] = uint4{0u, 0u, 0u, 0u};
-        }
-        if (v_page >= 0) {
-            const bf16_t* src = v_cache + ((static_cast<long>(v_page) * nkv + kh) * HD + v_row) * page_size + (vk & page_mask);
-#pragma unroll
-            for (int u = 0; u < CH; ++u)
-                v_regs[u] = *reinterpret_cast<const uint4*>(src + static_cast<long>(u) * (8 * RB) * page_size);
-        } else {
-#pragma unroll
-            for (int u = 0; u < CH; ++u) v_regs[u] = uint4{0u, 0u, 0u, 0u};
+                for (int u = 0; u < CH; ++u) k_regs[u] = u32x4{0u, 0u, 0u, 0u};
+            }
         }
     };
-    bf16_t* const k_put[2] = {smem + k_row * KROW + k_col, smem + STAGE + k_row * KROW + k_col};
-    bf16_t* const v_put[2] = {smem + KT * KROW + v_row * VROW + v_pos, smem + STAGE + KT * KROW + v_row * VROW + v_pos};
-    const bf16_t* const k_get[2] = {smem + (ksi * 64 + lr) * KROW + lh * 8, smem + STAGE + (ksi * 64 + lr) * KROW + lh * 8};
-    const bf16_t* const v_get[2] = {smem + KT * KROW + lr * VROW + ksi * 64 + lh * 8,
-                                    smem + STAGE + KT * KROW + lr * VROW + ksi * 64 + lh * 8};
-    auto stash = [&](auto stage_c) {
-        constexpr int stage = decltype(stage_c)::value;
+    auto trim_v = [&](int tile) {
+        if (at_an_end(tile)) {
+            const int vk = tile * KT + v_key;
+            if (!(vk <= blk_p_hi && vk + 7 >= blk_lo)) {
+#pragma unroll
+                for (int u = 0; u < CH; ++u) v_regs[u] = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+    };
+    // the slots: keys [2][KT][KROW], then values [2][HD][VROW]
+    constexpr int KSLOT = KT * KROW, VSLOT = HD * VROW;
+    static_assert(2 * (KSLOT + VSLOT) == 2 * STAGE, "the slots fill the two stages");
+    bf16_t* const k_put[2] = {smem + k_row * KROW + k_col, smem + KSLOT + k_row * KROW + k_col};
+    bf16_t* const v_put[2] = {smem + 2 * KSLOT + v_row * VROW + v_pos, smem + 2 * KSLOT + VSLOT + v_row * VROW + v_pos};
+    const bf16_t* const k_get[2] = {smem + (ksi * 64 + lr) * KROW + lh * 8, smem + KSLOT + (ksi * 64 + lr) * KROW + lh * 8};
+    const bf16_t* const v_get[2] = {smem + 2 * KSLOT + lr * VROW + ksi * 64 + lh * 8,
+                                    smem + 2 * KSLOT + VSLOT + lr * VROW + ksi * 64 + lh * 8};
+    auto stash_k = [&](auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+#pragma unroll
+        for (int u = 0; u < CH; ++u) *reinterpret_cast<u32x4*>(k_put[slot] + u * 8) = k_regs[u];
+    };
+    auto stash_v = [&](auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
 #pragma unroll
         for (int u = 0; u < CH; ++u) {
-            *reinterpret_cast<uint4*>(k_put[stage] + u * 8) = k_regs[u];
-            bf16_t* vp = v_put[stage] + u * 8 * RB * VROW;
-            *reinterpret_cast<uint2*>(vp) = uint2{v_regs[u].x, v_regs[u].y};
-            *reinterpret_cast<uint2*>(vp + 8) = uint2{v_regs[u].z, v_regs[u].w};
+            bf16_t* vp = v_put[slot] + u * 8 * RB * VROW;
+            *reinterpret_cast<u32x2*>(vp) = u32x2{v_regs[u][0], v_regs[u][1]};
+            *reinterpret_cast<u32x2*>(vp + 8) = u32x2{v_regs[u][2], v_regs[u][3]};
         }
     };
-    auto walk = [&](auto stage_c, int tile) {
-        constexpr int stage = decltype(stage_c)::value;
-        fetch(tile + 1);           // past the last tile every page number is -1: nothing is read
-        lookup(tile + 2);
-        const int key0 = tile * KT + ksi * 64;       // this wavefront's 64 keys
-        if (wave_any && key0 <= w_p_hi && key0 + 63 >= w_lo_first) {     // else nothing visible to these rows
-            f32x16 acc[2];
+    // the scores of a tile from a key slot
+    auto scores = [&](auto slot_c, f32x16 (&acc)[2]) {
+        constexpr int slot = decltype(slot_c)::value;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-                for (int j = 0; j < NQ; ++j) {
-                    const uint4 kk = *reinterpret_cast<const uint4*>(k_get[stage] + kb * 32 * KROW + j * 16);
-                    acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), q[j],
-                                                                      j == 0 ? zero16 : acc[kb], 0, 0, 0);
+            for (int j = 0; j < NQ; ++j) {
+                const u32x4 kk = *reinterpret_cast<const u32x4*>(k_get[slot] + kb * 32 * KROW + j * 16);
+                acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), q[j],
+                                                                  j == 0 ? zero16 : acc[kb], 0, 0, 0);
+            }
+        }
+    };
+    // the output product of a tile from a value slot
+    auto outputs = [&](auto slot_c, const bf16x8 (&pb)[4]) {
+        constexpr int slot = decltype(slot_c)::value;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[t], o_sum, 0, 0, 0);
+#pragma unroll
+        for (int f = 0; f < FB; ++f)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const u32x4 a = *reinterpret_cast<const u32x4*>(v_get[slot] + f * 32 * VROW + t * 16);
+                o[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb[t], o[f], 0, 0, 0);
+            }
+    };
+    const float slack = kSlack / scale2;
+    // Iteration of tile i, whose parity relative to the first tile is PAR.  The keys of tile i + 1 lie in key slot
+    // PAR ^ 1, the values of tile i - 1 in value slot PAR ^ 1; `cur` holds the scores of tile i, `nxt` takes those of
+    // tile i + 1; `pb_prev` holds the probabilities of tile i - 1, `pb_new` takes those of tile i.
+    auto iterate = [&](auto par_c, int tile, f32x16 (&cur)[2], f32x16 (&nxt)[2], const bf16x8 (&pb_prev)[4],
+                       bf16x8 (&pb_new)[4]) {
+        constexpr int par = decltype(par_c)::value;
+        // what the iteration before has loaded goes into the slots that it has read for the last time (the barrier
+        // at its end lies between); the loads of this iteration have all of it to arrive
+        trim_k(tile + 2);
+        stash_k(std::integral_constant<int, par>{});     // read from the next iteration on
+        trim_v(tile);
+        stash_v(std::integral_constant<int, par>{});
+        fetch_k();                   // tile i + 3, whose page number the iteration before looked up
+        fetch_v();                   // tile i + 1
+        lookup_k(tile + 4);
+        lookup_v(tile + 2);
+        const int key0 = tile * KT + ksi * 64;
+        if (!(wave_any && key0 + 63 <= w_p_min && key0 >= w_lo_max)) {   // the diagonal, a window's edge, or nothing at all
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = key0 + kb * 32 + (e / 4) * 8 + lh * 4 + e % 4;
+                    if (!(key <= p_row && key >= lo_row)) cur[kb][e] = -INFINITY;
                 }
-            }
-            if (!(key0 + 63 <= w_p_min && key0 >= w_lo_max)) {           // on the diagonal or the window's edge
+        }
+        float mx = max3(cur[0][0], cur[0][1], cur[0][2]), mx1 = max3(cur[1][0], cur[1][1], cur[1][2]);
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+        for (int e = 3; e < 15; e += 2) {
+            mx = max3(mx, cur[0][e], cur[0][e + 1]);
+            mx1 = max3(mx1, cur[1][e], cur[1][e + 1]);
+        }
+        mx = max3(mx, mx1, cur[0][15]);
+        mx = fmaxf(mx, cur[1][15]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        // (without a branch, which would cut the straight line in two)
+        const bool rescale = __any(mx > m_run + slack);       // (-inf + slack is -inf: the first key a row sees counts)
+        const float m_new = rescale ? fmaxf(m_run, mx) : m_run;
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
+        m_run = m_new;
+        const float shift = -m_use * scale2;
+        // the straight line
+        scores(std::integral_constant<int, par ^ 1>{}, nxt);
+        // the second product's steps of 16 keys: step t takes elements 8 (t % 2) .. + 7 of block t / 2 from a lane
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        const int key = key0 + kb * 32 + (e / 4) * 8 + lh * 4 + e % 4;
-                        if (!(key <= p_row && key >= lo_row)) acc[kb][e] = -INFINITY;
-                    }
-            }
-            float mx = max3(acc[0][0], acc[0][1], acc[0][2]), mx1 = max3(acc[1][0], acc[1][1], acc[1][2]);
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int e = 3; e < 15; e += 2) {
-                mx = max3(mx, acc[0][e], acc[0][e + 1]);
-                mx1 = max3(mx1, acc[1][e], acc[1][e + 1]);
-            }
-            mx = max3(mx, mx1, acc[0][15]);
-            mx = fmaxf(mx, acc[1][15]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-            const float m_new = fmaxf(m_run, mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            if (__any(m_new != m_run)) {             // some row's maximum moved: rescale what is accumulated
-                const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
-                o_sum[0] *= alpha;
+            for (int e = 0; e < 8; ++e)
+                pb_new[t][e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(cur[t / 2][(t % 2) * 8 + e], scale2, shift)));
+        outputs(std::integral_constant<int, par ^ 1>{}, pb_prev);
+        // the order asked of the scheduler: a matrix instruction, then its share of the vector instructions (an
+        // exponential, its multiply-add, half a conversion for each of the 32 scores of a lane) and of the LDS reads
+        constexpr int N_MATRIX = 2 * NQ + 4 + 4 * FB;
+        constexpr int PER = (80 + 48 + N_MATRIX - 1) / N_MATRIX;   // (48: the maximum, the addresses of the loads)
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-                for (int f = 0; f < FB; ++f)
+        for (int g = 0; g < N_MATRIX; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x402, PER, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        // (the probabilities are first used in the next iteration; this keeps the compiler from moving their
+        // computation out of the straight line, behind the branch below)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) o[f][e] *= alpha;
-                m_run = m_new;
-            }
-            const float shift = -m_use * scale2;
-            // the second product's steps of 16 keys: step t takes elements 8 (t % 2) .. + 7 of block t / 2 from a lane
-            bf16x8 pb[4];
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    pb[t][e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(acc[t / 2][(t % 2) * 8 + e], scale2, shift)));
-#pragma unroll
-            for (int t = 0; t < 4; ++t) o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb[t], o_sum, 0, 0, 0);
+        for (int t = 0; t < 4; ++t) asm volatile("" : "+v"(pb_new[t]));
+        if (rescale) {               // what is accumulated, the product of tile i - 1 included, in units of the new maximum
+            o_sum[0] *= alpha;
 #pragma unroll
             for (int f = 0; f < FB; ++f)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const uint4 a = *reinterpret_cast<const uint4*>(v_get[stage] + f * 32 * VROW + t * 16);
-                    o[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), pb[t], o[f], 0, 0, 0);
-                }
+                for (int e = 0; e < 16; ++e) o[f][e] *= alpha;
         }
-        stash(std::integral_constant<int, stage ^ 1>{});
         __syncthreads();
     };
 
-    lookup(t_begin);
-    fetch(t_begin);
-    lookup(t_begin + 1);
-    stash(std::integral_constant<int, 0>{});
+    f32x16 acc_a[2], acc_b[2];
+    bf16x8 pb_a[4], pb_b[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb_b[t][e] = static_cast<__bf16>(0.0f);
+    lookup_k(t_begin);
+    fetch_k();
+    lookup_k(t_begin + 1);
+    trim_k(t_begin);
+    stash_k(std::integral_constant<int, 0>{});
+    fetch_k();
+    lookup_k(t_begin + 2);
+#pragma unroll
+    for (int u = 0; u < CH; ++u) v_regs[u] = u32x4{0u, 0u, 0u, 0u};
+    stash_v(std::integral_constant<int, 1>{});       // the first iteration multiplies this slot by probabilities of zero
+    lookup_v(t_begin);
+    fetch_v();
+    lookup_v(t_begin + 1);
+    trim_k(t_begin + 1);
+    stash_k(std::integral_constant<int, 1>{});
+    fetch_k();                                       // tile 2, for the first iteration to put into slot 0
+    lookup_k(t_begin + 3);
     __syncthreads();
+    scores(std::integral_constant<int, 0>{}, acc_a);
+    __syncthreads();                 // every wavefront has read the first tile's keys before their slot is written again
     for (int tile = t_begin; tile < t_end; tile += 2) {
-        walk(std::integral_constant<int, 0>{}, tile);
-        if (tile + 1 < t_end) walk(std::integral_constant<int, 1>{}, tile + 1);
+        iterate(std::integral_constant<int, 0>{}, tile, acc_a, acc_b, pb_b, pb_a);
+        if (tile + 1 < t_end) iterate(std::integral_constant<int, 1>{}, tile + 1, acc_b, acc_a, pb_a, pb_b);
     }
+    // the output product of the last tile
+    if ((t_end - t_begin) & 1) outputs(std::integral_constant<int, 0>{}, pb_a);
+    else outputs(std::integral_constant<int, 1>{}, pb_b);
+    if constexpr (KS > 1) __syncthreads();           // the combination below writes over the tiles
     // the row's sum: feature 0 of the block of ones, which lane lr of half 0 holds
     float l = __shfl(o_sum[0], lr, kWave);
     if constexpr (KS > 1) {
@@ -1341,6 +1446,7 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
         return EGPT_BAD_ARGUMENT;
     if ((hd != 64 && hd != 128) || page_size < 16 || (page_size & (page_size - 1)) != 0 || nkv > 65535)
         return EGPT_UNSUPPORTED_SIZE;
+    if (shape >= 100 && page_size > 64) return EGPT_UNSUPPORTED_SIZE;     // its tiles of 64 keys are whole pages
     if (n_tokens == 0) return EGPT_OK;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;

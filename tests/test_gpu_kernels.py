@@ -559,9 +559,10 @@ def paged_reference(q, keys, vals, nq, nkv, scale, window):
     return out
 
 
-def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
+def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3, ramp=0.0):
     """seqs: list of (q_len, kv_len).  Returns everything paged_attention needs, with pages handed out in a
-    shuffled order and unused slots filled with huge values (reading one would wreck the result)."""
+    shuffled order and unused slots filled with huge values (reading one would wreck the result).  ramp: the keys'
+    first feature is ramp * position instead of random."""
     g = torch.Generator().manual_seed(seed)
     n_pages = sum(-(-kv // ps) for _, kv in seqs) + extra_pages
     order = torch.randperm(n_pages, generator=g).tolist()
@@ -573,6 +574,8 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
     for b, (_, kv) in enumerate(seqs):
         kk = torch.randn(kv, nkv, hd, generator=g).to(dtype)
         vv = torch.randn(kv, nkv, hd, generator=g).to(dtype)
+        if ramp:
+            kk[:, :, 0] = (ramp * torch.arange(kv, dtype=torch.float32))[:, None].to(dtype)
         keys.append(kk)
         vals.append(vv)
         n = -(-kv // ps)
@@ -586,11 +589,14 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3):
     return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
 
 
-def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None):
-    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed)
+def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None, ramp=0.0):
+    kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed, ramp=ramp)
     t = sum(q for q, _ in seqs)
     g = torch.Generator().manual_seed(seed + 100)
-    qkv = (torch.randn(t, (nq + 2 * nkv) * hd, generator=g) * q_scale).to(dtype).to(DEV)
+    qkv = torch.randn(t, (nq + 2 * nkv) * hd, generator=g) * q_scale
+    if ramp:
+        qkv.view(t, nq + 2 * nkv, hd)[:, :nq, 0] = 1.0        # every query weighs the keys' ramp alike
+    qkv = qkv.to(dtype).to(DEV)
     q_len = torch.tensor([q for q, _ in seqs], dtype=torch.int32)
     q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
     kv_len = torch.tensor([kv for _, kv in seqs], dtype=torch.int32)
@@ -713,10 +719,24 @@ def test_paged_attention_long_prefixes(k, hd, shape, window):
     assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, window=window, tiled_shape=shape, seed=5) <= 1.2e-2
 
 
+@pytest.mark.parametrize("hd,shape", [(64, 142), (64, 121), (128, 141), (64, 42), (128, 42)])
+@pytest.mark.parametrize("ramp", [0.26, 0.9, -0.26, 4.0])
+def test_prompt_attention_with_scores_that_grow_along_the_keys(k, hd, shape, ramp):
+    # the kernel of 32-row blocks rescales what it has accumulated only when a row's maximum has grown by more than a
+    # margin, and takes the exponentials against the old maximum until then.  Scores that rise by about 3 (in powers
+    # of two) from one tile of 64 keys to the next keep it just below the margin for several tiles in a row; a rise
+    # of 10 a tile goes over it in every tile, 45 a tile by far; falling scores never rescale after the first tile.
+    seqs = [(300, 1500), (64, 64), (33, 700)]
+    r = ramp * math.sqrt(hd / 64)
+    assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, tiled_shape=shape, seed=9, ramp=r) <= 1.2e-2
+    assert run_paged(k, seqs, 6, 2, hd, 32, torch.bfloat16, window=200, tiled_shape=shape, seed=10, ramp=r) <= 1.2e-2
+
+
 def test_paged_attention_tiled_refuses_other_page_sizes(k):
     z = torch.zeros(64, device=DEV)
     p = z.data_ptr()
-    for ps, shape in ((48, 42), (8, 42), (16, 43)):          # not a power of two, too small, no such shape
+    # not a power of two, too small, no such shape, pages larger than the tiles of the kernel of 32-row blocks
+    for ps, shape in ((48, 42), (8, 42), (16, 43), (128, 142)):
         with pytest.raises(RuntimeError):
             k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, None)
 
