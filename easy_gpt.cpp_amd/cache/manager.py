@@ -25,6 +25,7 @@ step costs no calls into the library.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 
 from ..parts.base import CacheNeed
@@ -51,7 +52,7 @@ def _library():
         from ..csrc import build
 
         lib = ctypes.CDLL(build.ensure_host_built())
-        if lib.egh_abi_version() != 2:
+        if lib.egh_abi_version() != 3:
             raise RuntimeError("the host library has an unexpected ABI version")
         vp, i = ctypes.c_void_p, ctypes.c_int
         sigs = {
@@ -60,7 +61,7 @@ def _library():
             "egh_version": ([vp, i], i), "egh_table_len": ([vp, i, i], i), "egh_table": ([vp, i, i, vp, i], i),
             "egh_pages_needed": ([vp, i, i, vp], i), "egh_free_pages": ([vp, i], i), "egh_used_pages": ([vp, i], i),
             "egh_num_pages": ([vp, i], i), "egh_high_water": ([vp, i], i), "egh_free_slots": ([vp], i),
-            "egh_reserve": ([vp, i, vp, vp, vp], i), "egh_commit": ([vp, i, vp, vp], i),
+            "egh_reserve": ([vp, i, vp, vp, vp], i), "egh_commit": ([vp, i, vp, vp], i), "egh_unreserve": ([vp, i, vp], i),
             "egh_slot_index": ([vp, i, i, i], i), "egh_check": ([vp, vp, i], i),
             "egh_fill_decode": ([vp, i, vp, vp, vp, vp, vp], i),
             "egh_fill_decode_rows": ([vp, i, i, vp, vp, vp, vp, vp], i),
@@ -215,6 +216,31 @@ class CacheManager:
             want = -(-(rc.num_tokens + n) // ps)
             rc.table_lens = [max(want, have) for have in rc.table_lens]
         self._refresh()
+
+    def unreserve_step(self, rcs) -> None:
+        """Gives back what `reserve_step` took for tokens that were not committed (the step failed in between):
+        every request keeps the pages of its committed tokens, the pools are as before the reservation."""
+        live = [rc for rc in rcs if rc.live]
+        code = self._lib.egh_unreserve(self._core, len(live), _ints([rc.handle for rc in live]))
+        if code != 0:
+            raise RuntimeError(f"unreserve failed with code {code}")
+        ps = self.page_size
+        for rc in live:
+            keep = -(-rc.num_tokens // ps)
+            rc.table_lens = [min(keep, have) for have in rc.table_lens]
+        self._refresh()
+
+    @contextlib.contextmanager
+    def reserved(self, rcs, counts):
+        """`with cache.reserved(rcs, counts): run the step`: pages for the step's tokens, committed when the body
+        ends and given back when it raises."""
+        self.reserve_step(rcs, counts)
+        try:
+            yield
+        except BaseException:
+            self.unreserve_step(rcs)
+            raise
+        self.commit_step(rcs, counts)
 
     def commit(self, rc: RequestCache, n_new: int) -> None:
         self.commit_step([rc], [n_new])

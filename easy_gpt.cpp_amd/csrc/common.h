@@ -46,10 +46,18 @@ __device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, 
 // a product's k range add their partial results straight into it with integer atomics: integer addition does not
 // care for the order, so the sum is the same bits whatever the scheduling, and the kernels that read the stream
 // read one small tensor instead of every workgroup's partial sums.  A float32 value times 2^32 is an integer for
-// every magnitude of 2^-8 and above and is rounded to one below; the stream holds magnitudes below 2^31.
+// every magnitude of 2^-8 and above and is rounded to one below (an absolute error of at most 2^-33, whatever the
+// other values of the stream are); the stream holds magnitudes below 2^31.  What does not fit is not hidden as
+// a small number: a magnitude of 2^31 or more, an infinity or a NaN enters as the largest magnitude of its sign
+// (NaN: the negative one), which the norm behind it turns into a row of zeros and one entry of +-sqrt(width) - a
+// step of more than 16 rows, and the float32 path, keep such values in float32 and show them as they are.
 typedef long long fixed_t;
 constexpr float kFixedOne = 4294967296.0f;
-__device__ __forceinline__ fixed_t to_fixed(float v) { return __float2ll_rn(v * kFixedOne); }
+constexpr float kFixedLimit = 2147483648.0f;          // 2^31
+__device__ __forceinline__ fixed_t to_fixed(float v) {
+    if (!(fabsf(v) < kFixedLimit)) return v > 0.f ? 0x7fffffffffffffffLL : -0x7fffffffffffffffLL - 1;
+    return __float2ll_rn(v * kFixedOne);
+}
 __device__ __forceinline__ float fixed_to_float(fixed_t v) { return __ll2float_rn(v) * (1.0f / kFixedOne); }
 __device__ __forceinline__ void fixed_add(fixed_t* p, float v) {
     atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(to_fixed(v)));

@@ -66,7 +66,7 @@ struct EghCore {
 
 extern "C" {
 
-int egh_abi_version(void) { return 2; }
+int egh_abi_version(void) { return 3; }
 
 EghCore* egh_create(int n_groups, const int32_t* windows, const int32_t* num_pages, int page_size, int max_requests) {
     if (n_groups < 0 || page_size < 1 || max_requests < 0 || (n_groups > 0 && (!windows || !num_pages))) return nullptr;
@@ -187,6 +187,29 @@ int egh_reserve(EghCore* c, int n, const int32_t* handles, const int32_t* counts
             const int need = std::max(0, want - static_cast<int>(r->tables[g].size()));
             for (int j = 0; j < need; ++j) r->tables[g].push_back(c->pools[g].take());
             if (need) r->version += 1;
+        }
+    }
+    return EGH_OK;
+}
+
+int egh_unreserve(EghCore* c, int n, const int32_t* handles) {
+    if (!c || n < 0 || (n > 0 && !handles)) return EGH_BAD_ARGUMENT;
+    for (int i = 0; i < n; ++i)
+        if (!c->get(handles[i])) return EGH_BAD_HANDLE;
+    // in the reverse of the order in which egh_reserve took them, so that the free lists are as before it
+    for (int i = n - 1; i >= 0; --i) {
+        Request* r = c->get(handles[i]);
+        const int keep = c->pages_for(r->num_tokens);
+        for (int g = c->n_groups() - 1; g >= 0; --g) {
+            std::vector<int32_t>& table = r->tables[g];
+            bool changed = false;
+            while (static_cast<int>(table.size()) > keep) {
+                const int32_t p = table.back();
+                if (p >= 0 && !c->pools[g].give_back(p)) return EGH_INVARIANT;
+                table.pop_back();
+                changed = true;
+            }
+            if (changed) r->version += 1;
         }
     }
     return EGH_OK;

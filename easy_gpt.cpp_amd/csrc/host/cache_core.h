@@ -36,6 +36,10 @@ int egh_num_pages(const EghCore* c, int g);
 int egh_high_water(const EghCore* c, int g);
 int egh_free_slots(const EghCore* c);
 
+// Gives back the pages that egh_reserve took for tokens that were never committed (a step that failed between the
+// two): every request keeps the pages of its committed tokens.
+int egh_unreserve(EghCore* c, int n, const int32_t* handles);
+
 // Pages for the next counts[i] tokens of each request, in every group: all of them or none.
 // On EGH_OUT_OF_PAGES detail = {index of the request, group, pages it needs there, free pages there}.
 int egh_reserve(EghCore* c, int n, const int32_t* handles, const int32_t* counts, int32_t* detail);

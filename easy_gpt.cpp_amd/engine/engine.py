@@ -178,10 +178,9 @@ class Engine:
             return self._step_padded(entries)
         rcs = self._check(entries)
         counts = [len(e.tokens) for e in entries]
-        self.cache.reserve_step(rcs, counts)               # all of the step's pages or none
-        ctx = self._build_context(rcs, entries)
-        logits = self.model.forward(ctx)
-        self.cache.commit_step(rcs, counts)
+        with self.cache.reserved(rcs, counts):             # all of the step's pages or none; given back if it fails
+            ctx = self._build_context(rcs, entries)
+            logits = self.model.forward(ctx)
         return logits
 
     def _check(self, entries) -> list[RequestCache]:
@@ -310,6 +309,13 @@ class Engine:
         starters = [rc for rc in rcs if rc.num_tokens % ps == 0]
         if starters:
             self.cache.reserve_step(starters, [1] * len(starters))
+        try:
+            return self._decode_reserved(rcs, tokens, device_tokens)
+        except BaseException:
+            self.cache.unreserve_step(starters)            # a step that fails leaves the pools as it found them
+            raise
+
+    def _decode_reserved(self, rcs, tokens, device_tokens) -> torch.Tensor:
         b = len(rcs)
         # Beyond 16 requests the batch is padded to a multiple of 8 with rows of one token at position 0 on a page
         # that no request owns: requests finish one by one, and every batch size would otherwise be a graph of its
@@ -381,15 +387,14 @@ class Engine:
         models with per-request state, whose parts walk a portion token after token."""
         rcs = self._check(entries)
         counts = [len(e.tokens) for e in entries]
-        self.cache.reserve_step(rcs, counts)
         t = sum(counts)
-        widths = self._table_widths(rcs)
-        kv_bound = -(-max(rc.num_tokens + n for rc, n in zip(rcs, counts)) // 512) * 512
-        key = (t, tuple(widths), kv_bound)
-        plan = self._plan(self._row_plans, key, lambda: _DecodePlan(self, t, widths, kv_bound, rows_independent=False))
-        plan.fill_rows(rcs, entries, counts)
-        logits = self._run(plan)
-        self.cache.commit_step(rcs, counts)
+        with self.cache.reserved(rcs, counts):
+            widths = self._table_widths(rcs)
+            kv_bound = -(-max(rc.num_tokens + n for rc, n in zip(rcs, counts)) // 512) * 512
+            key = (t, tuple(widths), kv_bound)
+            plan = self._plan(self._row_plans, key, lambda: _DecodePlan(self, t, widths, kv_bound, rows_independent=False))
+            plan.fill_rows(rcs, entries, counts)
+            logits = self._run(plan)
         want, base = [], 0
         for e, n in zip(entries, counts):
             want.extend(base + int(w) for w in e.want)
@@ -412,7 +417,10 @@ class Engine:
         whatever its size; from the graph it takes its device time."""
         rcs = self._check(entries)
         counts = [len(e.tokens) for e in entries]
-        self.cache.reserve_step(rcs, counts)
+        with self.cache.reserved(rcs, counts):
+            return self._padded_reserved(rcs, entries, counts)
+
+    def _padded_reserved(self, rcs, entries, counts) -> torch.Tensor | None:
         t = sum(counts)
         step = 16 if t <= 256 else self.PAD_TO          # small steps are padded less: their time grows with their rows
         t_pad = -(-t // step) * step
@@ -428,7 +436,6 @@ class Engine:
         plan = self._plan(self._padded_plans, key, lambda: _PaddedPlan(self, t_pad, b_pad, r_pad, widths))
         n_want = plan.fill(rcs, entries, counts)
         logits = self._run(plan)
-        self.cache.commit_step(rcs, counts)
         return logits[:n_want] if n_want else None
 
 

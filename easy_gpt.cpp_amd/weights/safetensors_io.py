@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import json
 import mmap
+import warnings
 import os
 import struct
 from dataclasses import dataclass
@@ -117,8 +118,14 @@ class SafetensorsFile:
         dtype, _ = _DTYPES[e.dtype]
         if e.end == e.begin:
             return torch.empty(e.shape, dtype=dtype)
-        raw = self._mm[self._data_start + e.begin : self._data_start + e.end]
-        return torch.frombuffer(bytearray(raw), dtype=dtype).reshape(e.shape)
+        # one copy, from the mapped file into the tensor (the view itself must not outlive the mapping)
+        view = memoryview(self._mm)[self._data_start + e.begin : self._data_start + e.end]
+        try:
+            with warnings.catch_warnings():
+                warnings.simplefilter("ignore", UserWarning)          # "the given buffer is not writable"
+                return torch.frombuffer(view, dtype=dtype).reshape(e.shape).clone()
+        finally:
+            view.release()
 
     def close(self) -> None:
         try:

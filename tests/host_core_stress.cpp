@@ -105,10 +105,17 @@ int main(int argc, char** argv) {
                         for (int i = 0; i < b; ++i) REQUIRE(small[1 * b + i] == positions[i] && small[4 * b + i] == kv_len[i]);
                         for (int i = 0; i < tab_size; ++i) REQUIRE(tab[i] == tables[i]);
                     }
-                    REQUIRE(egh_commit(c, b, handles.data(), counts.data()) == EGH_OK);
-                    for (int i = 0; i < b; ++i) {
-                        live[chosen[i]].tokens += counts[i];
-                        REQUIRE(egh_num_tokens(c, handles[i]) == live[chosen[i]].tokens);
+                    if (pick(0, 6) == 0) {
+                        // the step fails: what it reserved goes back and the pools are as before
+                        REQUIRE(egh_unreserve(c, b, handles.data()) == EGH_OK);
+                        for (int g = 0; g < n_groups; ++g) REQUIRE(egh_free_pages(c, g) == free_before[g]);
+                        for (int i = 0; i < b; ++i) REQUIRE(egh_num_tokens(c, handles[i]) == live[chosen[i]].tokens);
+                    } else {
+                        REQUIRE(egh_commit(c, b, handles.data(), counts.data()) == EGH_OK);
+                        for (int i = 0; i < b; ++i) {
+                            live[chosen[i]].tokens += counts[i];
+                            REQUIRE(egh_num_tokens(c, handles[i]) == live[chosen[i]].tokens);
+                        }
                     }
                 }
             } else if (!live.empty()) {

@@ -160,6 +160,18 @@ class PlainCacheManager:
                 table.extend(pool.take(n))
                 rc.version += 1
 
+    def unreserve_step(self, rcs) -> None:
+        """Gives back the pages taken for tokens that were not committed, in the reverse of the order of taking."""
+        for rc in reversed(list(rcs)):
+            keep = _ceil_div(rc.num_tokens, self.page_size)
+            for pool, table in reversed(list(zip(self.pools, rc.tables))):
+                changed = False
+                while len(table) > keep:
+                    pool.give_back([table.pop()])
+                    changed = True
+                if changed:
+                    rc.version += 1
+
     def commit(self, rc: PlainRequestCache, n_new: int) -> None:
         rc.num_tokens += n_new
         if _ceil_div(rc.num_tokens, self.page_size) > min((len(t) for t in rc.tables), default=10**18):

@@ -142,7 +142,11 @@ def test_random_orders_keep_the_invariants_and_both_managers_agree(seed):
             assert m.can_reserve(rc, n) == ref.can_reserve(pc, n)
             if m.can_reserve(rc, n):
                 m.reserve(rc, n), ref.reserve(pc, n)
-                m.commit(rc, n), ref.commit(pc, n)
+                if rng.random() < 0.15:                   # the step fails: what it took goes back
+                    m.unreserve_step([rc]), ref.unreserve_step([pc])
+                    assert [list(t) for t in rc.tables] == before
+                else:
+                    m.commit(rc, n), ref.commit(pc, n)
             else:
                 with pytest.raises(OutOfPages):
                     m.reserve(rc, n)
@@ -172,6 +176,33 @@ def test_a_step_reserves_for_all_its_requests_or_for_none():
     with pytest.raises(RuntimeError, match="without reserve"):
         m.commit(a, 1)
     m.check()
+
+
+@pytest.mark.parametrize("Manager,OutOfPages,NoFreeSlot", BOTH, ids=["native", "plain"])
+def test_a_failed_step_gives_back_what_it_reserved(Manager, OutOfPages, NoFreeSlot):
+    m = Manager([FULL, WIN], page_size=4, num_pages=[12, 6], max_requests=3)
+    a, b = m.admit("a"), m.admit("b")
+    snapshot = lambda: ([list(t) for t in a.tables], [list(t) for t in b.tables])
+    for rc, n in ((a, 6), (b, 3)):
+        m.reserve(rc, n)
+        m.commit(rc, n)
+    free, tables = m.free_pages(), snapshot()
+    m.reserve(a, 9), m.reserve(b, 2)                   # a: two more pages in each group, b: one more
+    taken = snapshot()
+    assert m.free_pages() == [free[0] - 3, free[1] - 3]
+    m.unreserve_step([a, b])                           # the step failed: nothing was committed
+    assert m.free_pages() == free and snapshot() == tables
+    assert (a.num_tokens, b.num_tokens) == (6, 3)
+    m.check()
+    m.reserve(a, 9), m.reserve(b, 2)                   # the same pages come again, in the same order
+    assert snapshot() == taken
+    m.commit(a, 9), m.commit(b, 2)
+    after = snapshot()
+    m.unreserve_step([a, b])                           # nothing to give back: every page holds committed tokens
+    assert snapshot() == after
+    m.release(a), m.release(b)
+    m.check()
+    assert m.free_pages() == [12, 6]
 
 
 def test_the_library_writes_a_steps_metadata():

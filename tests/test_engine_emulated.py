@@ -78,3 +78,35 @@ def test_step_checks_and_out_of_pages_leaves_the_cache_unchanged(tiny_models):
     with pytest.raises(ValueError, match="max_position_embeddings"):
         eng.finish("b")
         eng.step([StepEntry("a", list(range(200)), [])])
+
+
+def test_a_step_that_fails_leaves_the_cache_as_it_found_it(tiny_models):
+    # an error between the reservation of a step's pages and their commit (here: the model raises) gives the pages
+    # back, and the same step can be run again
+    cfg = TINY["A"][0]
+    reqs = H.make_requests(cfg["vocab_size"], [23, 9], seed=5)
+    ref = H.plain_rows(tiny_models["A"], reqs)
+    eng = Engine.from_dir(tiny_models["A"], dtype="float32", device="cpu", page_size=4, max_tokens=64, max_requests=2)
+    ids = list(reqs)
+    for rid in ids:
+        eng.add_request(rid)
+    eng.step([StepEntry(rid, reqs[rid][:5], [4]) for rid in ids])
+    free = eng.cache.free_pages()
+    forward = eng.model.forward
+
+    def broken(ctx):
+        raise RuntimeError("the device is gone")
+
+    eng.model.forward = broken
+    second = [StepEntry(ids[0], reqs[ids[0]][5:], [0]), StepEntry(ids[1], reqs[ids[1]][5:6], [0])]
+    with pytest.raises(RuntimeError, match="gone"):
+        eng.step(second)
+    assert eng.cache.free_pages() == free
+    eng.cache.check()
+    eng.model.forward = forward
+    logits = eng.step(second)
+    for row, rid in zip(logits, ids):
+        assert float((row.double().cpu() - ref[rid][5]).abs().max()) <= 1e-5 * float(ref[rid][5].abs().max())
+    for rid in ids:
+        eng.finish(rid)
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]

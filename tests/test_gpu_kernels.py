@@ -288,6 +288,47 @@ def test_residual_stream_in_fixed_point(k, t, hid, inter, nq, hd):
     assert k.product(x, w_down, residual=hf).dim() == 3
 
 
+def test_residual_stream_in_fixed_point_over_its_range(k):
+    # magnitudes from 1e-6 to 1e6 side by side (models have channels of 1e3 to 1e5 beside ones of 1e-3): every value
+    # keeps its own precision through the embedding, the norm's addition and the products' atomics; a value that the
+    # stream cannot hold enters as the largest magnitude of its sign
+    dtype, t, hid, inter = torch.bfloat16, 6, 256, 512
+    g = torch.Generator().manual_seed(31)
+    wide = lambda *shape: (10.0 ** (torch.rand(*shape, generator=g) * 12 - 6)) * (torch.randint(0, 2, shape, generator=g) * 2 - 1)
+    table = wide(40, hid).to(dtype).to(DEV)
+    ids = torch.arange(t, dtype=torch.int32, device=DEV) * 5
+    h = torch.empty(t, hid, dtype=torch.int64, device=DEV)
+    k.embed(ids, table, h)
+    assert torch.equal(h, to_fixed(table[ids.long()].float()))                # bfloat16 values of these sizes are exact
+    # the norm adds float32 values of any of these sizes to any other
+    nw = (1 + rnd(hid, seed=2, scale=0.1)).to(dtype)
+    delta = wide(2, t, hid).float().to(DEV)
+    hh = h.clone()
+    out = torch.empty(t, hid, dtype=dtype, device=DEV)
+    k.add_rmsnorm(hh, delta, nw, 1e-6, out)
+    want = from_fixed(h) + delta.double().sum(0)
+    err = (from_fixed(hh) - want).abs()
+    size = from_fixed(h).abs() + delta.double().abs().sum(0)                  # (the additions are float32 ones)
+    assert bool((err <= 2e-7 * size + 2.0 ** -32).all())                      # per element, not against the row's largest
+    ref = plain.rms_norm(want.cpu(), nw.double().cpu(), 1e-6)
+    assert float((out.double().cpu() - ref).abs().max()) <= 1.6e-2 * float(ref.abs().max())
+    # partial products of every size are added as the integers they are
+    x = (torch.randn(t, inter, generator=g) * torch.tensor([1e-5, 1e-3, 1e-1, 1e1, 1e3, 1e4])[:, None]).to(dtype).to(DEV)
+    w_down = rnd(hid, inter, dtype=dtype, seed=6, scale=0.05)
+    parts = k.product(x, w_down)
+    assert float(parts.abs().max()) > 1e2 and float(parts.abs().min()) < 1e-3
+    hh = h.clone()
+    assert k.product(x, w_down, residual=hh) is hh
+    assert torch.equal(hh, h + sum(to_fixed(p) for p in parts))
+    # what does not fit: 2^31 and beyond, infinities and NaN become the largest magnitude
+    odd = torch.tensor([[3e9, -3e9, float("inf"), float("-inf"), float("nan"), 2.0 ** 31, 2.0 ** 31 - 128, 1.0]],
+                       dtype=torch.float32, device=DEV).repeat(1, hid // 8)
+    hz = torch.zeros(1, hid, dtype=torch.int64, device=DEV)
+    k.add_rmsnorm(hz, odd.view(1, 1, hid), nw, 1e-6, torch.empty(1, hid, dtype=dtype, device=DEV))
+    top, low = 2 ** 63 - 1, -(2 ** 63)
+    assert hz[0, :8].tolist() == [top, low, top, low, low, top, (2 ** 31 - 128) * 2 ** 32, 2 ** 32]
+
+
 @pytest.mark.parametrize("t,hid,n,d_splits", [(1, 896, 1152, 0), (8, 896, 9728, 4), (16, 200, 130, 3), (5, 1536, 2048, 13),
                                               (8, 3584, 4608, 19), (3, 1536, 17920, 12), (16, 256, 26000, 2)])
 def test_product_with_norm_folded_in(k, t, hid, n, d_splits):
