@@ -234,6 +234,12 @@ class HipKernels(KernelBackend):
             return True
         if n < k:
             return False
+        if m <= 32 and n >= 65536:
+            # an output matrix over a whole vocabulary, up to 32 rows: the own kernel with four wavefronts (measured
+            # on 151,936 x 896: 51 / 53 / 59 us at 17 / 24 / 32 rows against the library's 58 / 57 / 59; on 152,064 x
+            # 3,584: 215 / 218 / 223 against 243 / 248 / 255; at 48 and 64 rows the library wins, 71 against 100 us and
+            # 217 against 246, and workgroups of 8 or 16 wavefronts are slower than either)
+            return False
         return n * k >= (2 << 20 if m > 32 else 16 << 20)
 
     def linear(self, x, w, bias, out):
@@ -252,11 +258,10 @@ class HipKernels(KernelBackend):
         if x.dtype == _BF16 and k % 8 == 0:
             to_f32 = out.dtype == _F32
             if not self._library_rows(m, n, k):
-                # weight-streaming MFMA kernel (a very wide output with more than one tile of rows: workgroups
-                # of 8 wavefronts stage x half as often)
+                # weight-streaming MFMA kernel
                 self._run("egpt_gemm_skinny", x.data_ptr(), w.data_ptr(), self._ptr(bias),
                           out.data_ptr() if to_f32 else None, None if to_f32 else out.data_ptr(), None, m, n, k, 1,
-                          8 if (m > 16 and n >= 65536) else 4, self._stream())
+                          4, self._stream())
                 return out
             # many rows: the library's matrix product; float32 output (logits) unrounded
             if to_f32:
@@ -696,6 +701,14 @@ class HipKernels(KernelBackend):
             # workgroups of eight wavefronts, 1.66 with 440 and 480 of four; 1.57 either way at batch 40)
             if pairs * n_splits > 256:
                 n_waves = 0
+        if not n_waves and 128 < 2 * pairs <= 256 and key_blocks <= 288:
+            # two key ranges of eight wavefronts while that gives every workgroup a CU of its own (measured at the 0.5B
+            # sizes against the best shape of four wavefronts: batch 64 behind 2,048 tokens 1.727 ms a step against 1.765
+            # (4 ranges; 1.811 with the 5 that the rule below gives), batch 56 1.680 against 1.725, batch 48 1.618 against
+            # 1.626, batch 64 behind 3,584 tokens 1.923 against 1.962, behind 8,192 tokens 2.599 against 2.624; at the
+            # 1.5B sizes, head size 128: batch 64 3.12 against 3.21, batch 48 3.02 against 3.04; folding the two parts'
+            # combination into the output projection at these rows gave nothing: 1.752 against 1.728 at batch 64)
+            n_splits, n_waves = 2, 8
         if not n_waves:
             n_splits, n_waves = splits_for(4), 4
             # head size 128: eight wavefronts as well while every workgroup has a CU of its own (its 71 KB of LDS are
@@ -711,7 +724,7 @@ class HipKernels(KernelBackend):
         # but 1.99 -> 2.03 at batch 8 and 32,000 tokens, 31 blocks per wavefront).  Head size 128: from one and a
         # half workgroups per CU on (fewer: 1 to 2% slower than the full variant).
         per_wave = -(-key_blocks // (n_splits * n_waves))
-        lean = per_wave <= 16 if hd == 64 else pairs * n_splits > 384
+        lean = per_wave <= 17 if hd == 64 else pairs * n_splits > 384
         return n_splits, n_waves, 1 if lean else 0
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
