@@ -299,7 +299,10 @@ class HipKernels(KernelBackend):
         The count depends on the matrix alone, never on the rows, so that a row's partial sums, and with them
         every value of the 32-bit path, are the same bits in whatever batch the row is computed."""
         steps = -(-k // 64)
-        s = min(steps, max(1, 512 // -(-n // 64)), 8)
+        # at most 12 ranges: a step of few rows wants many workgroups, a prompt pays for every range with a float32
+        # copy of its output (measured at the 0.5B sizes, decode step at batch 8 / 2,048-token prefill: 1.73 / 24.4 ms
+        # with at most 8 ranges, 1.65 / 24.6 with 12, 1.58 / 26.5 with 16)
+        s = min(steps, max(1, 512 // -(-n // 64)), 12)
         per = -(-steps // s)
         return -(-steps // per)
 
