@@ -712,6 +712,13 @@ class HipKernels(KernelBackend):
             # 1.5B sizes, head size 128: batch 64 3.12 against 3.21, batch 48 3.02 against 3.04; folding the two parts'
             # combination into the output projection at these rows gave nothing: 1.752 against 1.728 at batch 64)
             n_splits, n_waves = 2, 8
+        elif not n_waves and 128 < pairs <= 512 and key_blocks <= 288:
+            # more pairs than half the CUs: no key ranges at all (and no combination of parts), eight wavefronts while
+            # every workgroup has a CU of its own, four beyond (measured, ms a step against the rule below: batch 128
+            # at the 0.5B sizes 2.44 against 2.52 behind 2,048 tokens and 4.04 against 4.21 behind 8,192, batch 256
+            # 3.11 against 3.27; at the 1.5B sizes batch 128 4.03 against 4.20; at the 7B sizes, four kv heads, batch
+            # 64 6.56 against 6.71 and batch 128 9.87 against 10.06)
+            n_splits, n_waves = 1, 8 if pairs <= 256 else 4
         if not n_waves:
             n_splits, n_waves = splits_for(4), 4
             # head size 128: eight wavefronts as well while every workgroup has a CU of its own (its 71 KB of LDS are
@@ -726,8 +733,9 @@ class HipKernels(KernelBackend):
         # at batch 8 and 2,048-token contexts, 0.872 -> 0.853 at batch 1, 1.135 -> 1.102 at batch 8 and 8,192 tokens,
         # but 1.99 -> 2.03 at batch 8 and 32,000 tokens, 31 blocks per wavefront).  Head size 128: from one and a
         # half workgroups per CU on (fewer: 1 to 2% slower than the full variant).
+        # (with more pairs than half the CUs also behind 8,192 tokens, 34 blocks per wavefront: 4.04 against 4.13 at batch 128)
         per_wave = -(-key_blocks // (n_splits * n_waves))
-        lean = per_wave <= 17 if hd == 64 else pairs * n_splits > 384
+        lean = (per_wave <= 17 or pairs > 128) if hd == 64 else pairs * n_splits > 384
         return n_splits, n_waves, 1 if lean else 0
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
