@@ -704,13 +704,14 @@ class HipKernels(KernelBackend):
             # workgroups of eight wavefronts, 1.66 with 440 and 480 of four; 1.57 either way at batch 40)
             if pairs * n_splits > 256:
                 n_waves = 0
-        if not n_waves and 128 < 2 * pairs <= 256 and key_blocks <= 288:
+        if not n_waves and 128 < 2 * pairs <= 256:
             # two key ranges of eight wavefronts while that gives every workgroup a CU of its own (measured at the 0.5B
             # sizes against the best shape of four wavefronts: batch 64 behind 2,048 tokens 1.727 ms a step against 1.765
             # (4 ranges; 1.811 with the 5 that the rule below gives), batch 56 1.680 against 1.725, batch 48 1.618 against
             # 1.626, batch 64 behind 3,584 tokens 1.923 against 1.962, behind 8,192 tokens 2.599 against 2.624; at the
             # 1.5B sizes, head size 128: batch 64 3.12 against 3.21, batch 48 3.02 against 3.04; folding the two parts'
-            # combination into the output projection at these rows gave nothing: 1.752 against 1.728 at batch 64)
+            # combination into the output projection at these rows gave nothing: 1.752 against 1.728 at batch 64; behind
+            # 32,000 tokens batch 64 takes 5.77 against 5.78 to 5.87 with 4 to 12 ranges of four wavefronts)
             n_splits, n_waves = 2, 8
         elif not n_waves and 128 < pairs <= 512 and key_blocks <= 288:
             # more pairs than half the CUs: no key ranges at all (and no combination of parts), eight wavefronts while
@@ -735,7 +736,8 @@ class HipKernels(KernelBackend):
         # half workgroups per CU on (fewer: 1 to 2% slower than the full variant).
         # (with more pairs than half the CUs also behind 8,192 tokens, 34 blocks per wavefront: 4.04 against 4.13 at batch 128)
         per_wave = -(-key_blocks // (n_splits * n_waves))
-        lean = (per_wave <= 17 or pairs > 128) if hd == 64 else pairs * n_splits > 384
+        # (and with 65 to 128 pairs behind 32,000 tokens: 5.77 against 5.85 at batch 64)
+        lean = (per_wave <= 17 or pairs > 64) if hd == 64 else pairs * n_splits > 384
         return n_splits, n_waves, 1 if lean else 0
 
     def attention_decode_fused(self, prod, row_ss, hidden, eps, bias, positions, inv_freq, rotary_dim, slots, out,
