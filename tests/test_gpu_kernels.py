@@ -772,6 +772,9 @@ def test_prompt_attention_with_scores_that_grow_along_the_keys(k, hd, shape, ram
     r = ramp * math.sqrt(hd / 64)
     assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, tiled_shape=shape, seed=9, ramp=r) <= 1.2e-2
     assert run_paged(k, seqs, 6, 2, hd, 32, torch.bfloat16, window=200, tiled_shape=shape, seed=10, ramp=r) <= 1.2e-2
+    # one head to a group, and sixteen
+    assert run_paged(k, seqs, 3, 3, hd, 64, torch.bfloat16, tiled_shape=shape, seed=11, ramp=r) <= 1.2e-2
+    assert run_paged(k, [(90, 400), (1, 77)], 16, 1, hd, 16, torch.bfloat16, tiled_shape=shape, seed=12, ramp=r) <= 1.2e-2
 
 
 def test_paged_attention_tiled_refuses_other_page_sizes(k):
