@@ -240,7 +240,10 @@ class HipKernels(KernelBackend):
             # 3,584: 215 / 218 / 223 against 243 / 248 / 255; at 48 and 64 rows the library wins, 71 against 100 us and
             # 217 against 246, and workgroups of 8 or 16 wavefronts are slower than either)
             return False
-        return n * k >= (2 << 20 if m > 32 else 16 << 20)
+        # (33 to 64 rows, measured with the weights coming from memory: 2,048 x 1,536 in 7.8 us against the library's 9.8,
+        # 1,536 x 1,536 7.7 against 9.2, 2,560 x 2,048 8.9 against 12.0, 2,048 x 2,048 8.1 against 11.8; 4,608 x 3,584 18.9
+        # either way, 3,584 x 3,584 14.2 against 13.7, 7,168 x 5,120 25.8 against 22.7)
+        return n * k >= (6 << 20 if m > 32 else 16 << 20)
 
     def linear(self, x, w, bias, out):
         m, k = x.shape
@@ -319,6 +322,11 @@ class HipKernels(KernelBackend):
         # matrix (measured inside the model at 896 x 4,864: 1.291 -> 1.260 ms a step at batch 24 and 1.790 -> 1.771 at 64
         # with 13 ranges instead of 10, 1.853 with 19; at 1,536 x 8,960, 13 ranges cost 3 to 7 %)
         s = min(steps, max(1, most // n_blocks), max(1, k // (2 * m)), 20 if m <= 16 else 13 if n * k <= 8 << 20 else 10)
+        if m > 16 and steps <= 16:
+            # a short k range and more than one tile of rows: no more workgroups than CUs (measured at 64 rows: 2,048 x
+            # 1,536 in 7.8 us with 6 ranges, 192 workgroups, against 9.0 with 12; 2,560 x 2,048 8.9 with 6 against 11.3 with
+            # 8, 320 workgroups; 2,048 x 2,048 8.1 with 8, 256 workgroups; at 32 rows 5.6 against 6.3 and 7.0 against 7.9)
+            s = min(s, max(1, 256 // n_blocks))
         per = -(-steps // s)
         return -(-steps // per)
 

@@ -167,7 +167,7 @@ def test_which_products_go_to_the_library():
     assert not lib(17, 151936, 896) and not lib(32, 152064, 3584)         # an output matrix at up to 32 rows: the own kernel
     assert not lib(64, 896, 4864) and not lib(17, 3584, 18944)            # split-k shapes stay with the own kernels
     assert not lib(32, 9728, 896) and lib(32, 17920, 1536)                # small matrices with up to 32 rows, too
-    assert not lib(64, 1152, 896) and lib(64, 4608, 3584)
+    assert not lib(64, 1152, 896) and lib(64, 4608, 3584) and not lib(64, 2048, 1536) and not lib(64, 2560, 2048)
 
 
 def test_consumers_add_partial_sums_up(k):
