@@ -15,6 +15,7 @@
 // second product.  With n_splits > 1 each split of the key range writes an unnormalised partial result
 // and its (maximum, sum), which attention_reduce_kernel combines.
 #include <type_traits>
+#include <utility>
 
 #include "api.h"
 #include "common.h"
@@ -549,6 +550,16 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
     return r;
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in this order
+template <int... I, class F>
+__device__ __forceinline__ void static_for_each(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_each(std::make_integer_sequence<int, N>{}, f);
+}
+
 template <int HD, int RB, int KS>
 __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
@@ -643,7 +654,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     // The loop is a pipeline of three stages over the tiles.  In the iteration of tile i a wavefront issues, as one
     // straight line of code, the score product of tile i + 1, the exponentials of tile i and the output product of tile
     // i - 1: the matrix instructions of the two products alternate with the vector instructions of the softmax between
-    // them, so that both pipes work at once.  (With a tile's products on either side of its softmax, and the
+    // them (in groups whose order scheduling fences keep), so that both pipes work at once.  (With a tile's products on either side of its softmax, and the
     // wavefronts of a workgroup in step from barrier to barrier, the pipes took turns: at 8,192 tokens the SIMDs issued
     // vector instructions half of the time and did nothing for much of the rest.)  What does not fit into a straight
     // line is kept out of it: masking (tiles on the diagonal or a window's edge) comes before it, and the accumulated
@@ -764,10 +775,6 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
         stash_k(std::integral_constant<int, par>{});     // read from the next iteration on
         trim_v(tile);
         stash_v(std::integral_constant<int, par>{});
-        fetch_k();                   // tile i + 3, whose page number the iteration before looked up
-        fetch_v();                   // tile i + 1
-        lookup_k(tile + 4);
-        lookup_v(tile + 2);
         const int key0 = tile * KT + ksi * 64;
         if (!(wave_any && key0 + 63 <= w_p_min && key0 >= w_lo_max)) {   // the diagonal, a window's edge, or nothing at all
 #pragma unroll
@@ -778,42 +785,78 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
                     if (!(key <= p_row && key >= lo_row)) cur[kb][e] = -INFINITY;
                 }
         }
-        float mx = max3(cur[0][0], cur[0][1], cur[0][2]), mx1 = max3(cur[1][0], cur[1][1], cur[1][2]);
+        // The straight line, group by group: a matrix instruction, the LDS read of the operand that the matrix
+        // instruction three groups on will take, and a share of the vector work; a scheduling fence after every group
+        // keeps them in this order.  The matrix instructions: 2 NQ for the scores of tile i + 1, four that sum the rows
+        // of tile i - 1, 4 FB for its output.  The vector work: the rows' maxima of tile i in the first four groups (with
+        // the loads of the tiles to come, whose addresses are a few instructions), the new maximum and what follows
+        // from it in the fifth, then the 32 exponentials of a lane dealt over the groups that are left.
+        constexpr int N_QK = 2 * NQ, N_MATRIX = N_QK + 4 + 4 * FB, AHEAD = 3, MAX_GROUPS = 4;
+        constexpr int EXP_GROUPS = N_MATRIX - MAX_GROUPS - 1;
+        u32x4 operand[AHEAD + 1];
+        // (consecutive matrix instructions go to different accumulators: one that adds to the result of the one before
+        // it would wait for it)
+        auto read_operand = [&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            if constexpr (g < N_QK) {
+                operand[g % (AHEAD + 1)] =
+                    *reinterpret_cast<const u32x4*>(k_get[par ^ 1] + (g % 2) * 32 * KROW + (g / 2) * 16);
+            } else if constexpr (g < N_MATRIX && (g - N_QK) % (1 + FB) != 0) {
+                constexpr int t = (g - N_QK) / (1 + FB), f = (g - N_QK) % (1 + FB) - 1;
+                operand[g % (AHEAD + 1)] = *reinterpret_cast<const u32x4*>(v_get[par ^ 1] + f * 32 * VROW + t * 16);
+            }
+        };
+        float mx = -INFINITY, mx1 = -INFINITY, alpha = 1.0f, shift = 0.0f;
+        bool rescale = false;
+        auto group = [&](auto g_c) {
+            constexpr int g = decltype(g_c)::value;
+            read_operand(std::integral_constant<int, g + AHEAD>{});
+            const bf16x8 from_lds = __builtin_bit_cast(bf16x8, operand[g % (AHEAD + 1)]);
+            if constexpr (g < N_QK) {
+                nxt[g % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(from_lds, q[g / 2], g / 2 == 0 ? zero16 : nxt[g % 2],
+                                                                     0, 0, 0);
+            } else if constexpr ((g - N_QK) % (1 + FB) == 0) {
+                o_sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb_prev[(g - N_QK) / (1 + FB)], o_sum, 0, 0, 0);
+            } else {
+                constexpr int t = (g - N_QK) / (1 + FB), f = (g - N_QK) % (1 + FB) - 1;
+                o[f] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(from_lds, pb_prev[t], o[f], 0, 0, 0);
+            }
+            if constexpr (g < MAX_GROUPS) {
+                // a quarter of the 32 scores of a lane: four of each of its two blocks
 #pragma unroll
-        for (int e = 3; e < 15; e += 2) {
-            mx = max3(mx, cur[0][e], cur[0][e + 1]);
-            mx1 = max3(mx1, cur[1][e], cur[1][e + 1]);
-        }
-        mx = max3(mx, mx1, cur[0][15]);
-        mx = fmaxf(mx, cur[1][15]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        // (without a branch, which would cut the straight line in two)
-        const bool rescale = __any(mx > m_run + slack);       // (-inf + slack is -inf: the first key a row sees counts)
-        const float m_new = rescale ? fmaxf(m_run, mx) : m_run;
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
-        m_run = m_new;
-        const float shift = -m_use * scale2;
-        // the straight line
-        scores(std::integral_constant<int, par ^ 1>{}, nxt);
-        // the second product's steps of 16 keys: step t takes elements 8 (t % 2) .. + 7 of block t / 2 from a lane
+                for (int e = 4 * g; e < 4 * g + 4; e += 2) {
+                    mx = max3(mx, cur[0][e], cur[0][e + 1]);
+                    mx1 = max3(mx1, cur[1][e], cur[1][e + 1]);
+                }
+                if constexpr (g == 0) fetch_k();          // tile i + 3, whose page number the iteration before looked up
+                if constexpr (g == 1) fetch_v();          // tile i + 1
+                if constexpr (g == 2) lookup_k(tile + 4);
+                if constexpr (g == 3) lookup_v(tile + 2);
+            } else if constexpr (g == MAX_GROUPS) {
+                mx = fmaxf(mx, mx1);
+                mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+                // (without a branch, which would cut the straight line in two)
+                rescale = __any(mx > m_run + slack);      // (-inf + slack is -inf: the first key a row sees counts)
+                const float m_new = rescale ? fmaxf(m_run, mx) : m_run;
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale2);
+                m_run = m_new;
+                shift = -m_use * scale2;
+            } else {
+                // the second product's steps of 16 keys: step t takes elements 8 (t % 2) .. + 7 of block t / 2 from a lane
+                constexpr int eg = g - MAX_GROUPS - 1;
+                constexpr int first = eg * 32 / EXP_GROUPS, last = (eg + 1) * 32 / EXP_GROUPS;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                pb_new[t][e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(cur[t / 2][(t % 2) * 8 + e], scale2, shift)));
-        outputs(std::integral_constant<int, par ^ 1>{}, pb_prev);
-        // the order asked of the scheduler: a matrix instruction, then its share of the vector instructions (an
-        // exponential, its multiply-add, half a conversion for each of the 32 scores of a lane) and of the LDS reads
-        constexpr int N_MATRIX = 2 * NQ + 4 + 4 * FB;
-        constexpr int PER = (80 + 48 + N_MATRIX - 1) / N_MATRIX;   // (48: the maximum, the addresses of the loads)
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-        for (int g = 0; g < N_MATRIX; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x402, PER, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
+                for (int i = first; i < last; ++i) {
+                    const int t = i / 8, e = i % 8;
+                    pb_new[t][e] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(cur[t / 2][(t % 2) * 8 + e], scale2, shift)));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        static_for<AHEAD>(read_operand);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<N_MATRIX>(group);
         // (the probabilities are first used in the next iteration; this keeps the compiler from moving their
         // computation out of the straight line, behind the branch below)
 #pragma unroll

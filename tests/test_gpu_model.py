@@ -367,13 +367,13 @@ def test_wide_layers_with_many_requests_replay_the_library_products_in_the_graph
     from easy_gpt.cpp_amd.weights import write_random_model
 
     cfg = {
-        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 256,
-        "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 4112, "vocab_size": 8300,
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 2, "hidden_size": 512,
+        "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64, "intermediate_size": 6160, "vocab_size": 12400,
         "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 64,
     }
     kernels.use_backend(None)
     k = kernels.backend()
-    assert k._library_rows(40, 2 * 4112, 256) and k._library_rows(40, 8300, 256) and not k._library_rows(40, 256, 4112)
+    assert k._library_rows(40, 2 * 6160, 512) and k._library_rows(40, 12400, 512) and not k._library_rows(40, 512, 6160)
     sharp = str(tmp_path)              # plain random weights: this test is about the replays, not about far keys
     write_random_model(sharp, cfg, seed=9)
     n_req, prompt, steps = 40, 9, 7
