@@ -618,21 +618,21 @@ class HipKernels(KernelBackend):
                 # a workgroup.  Few rows: small workgroups whose wavefronts split the keys, so that the GPU
                 # has enough of them; many rows: 64 rows per workgroup, which read the keys fewer times.
                 row_tiles = -(-t * (nq // nkv) // 16) * nkv
-                # Measured (us for one layer's prompt; row tiles of 16 rows; shape = row tiles x key splits of a
-                # workgroup, 1xx the kernel of 32-row blocks, whose tiles of 64 keys must be whole pages):
-                #   head size 64, 14 heads on 2:   448 tiles 24: 9.7, 44: 10.5 |  896 tiles 24: 17.9, 44: 15.4, 142: 17.3
-                #     1,344 tiles 44: 20.5, 142: 22.4 | 1,792 tiles 44: 29.6, 142: 27.6 | 3,584 tiles 42: 75, 142: 56
-                #     7,168 tiles (8,192 tokens) 42: 292, 142: 183 | 28,560 tiles (32,640 tokens) 42: 3,840, 142: 2,504
-                #   head size 128, 12 heads on 2:  768 tiles 22: 31.1, 42: 25.8 | 1,536 tiles 42: 47.2, 141: 56.7
-                #     3,072 tiles 42: 157, 141: 108;  28 heads on 4: 896 tiles 22: 28.4, 42: 16.9 | 1,792 tiles 42: 41.0,
-                #     141: 34.6 | 7,168 tiles 42: 336, 141: 227;  40 heads on 8: 1,280 tiles 42: 22.8, 141: 21.8
+                # Measured (us for one layer's prompt on a GPU that is warm; row tiles of 16 rows; shape = row tiles x key
+                # splits of a workgroup, 1xx the kernel of 32-row blocks, whose tiles of 64 keys must be whole pages):
+                #   head size 64, 14 heads on 2:   448 tiles 24: 9.4, 44: 10.4 |  896 tiles 24: 16.9, 44: 14.7, 142: 16.4
+                #     1,344 tiles 44: 20.0, 142: 21.3 | 1,792 tiles 44: 29.7, 142: 26.2 | 3,584 tiles 42: 76, 142: 53
+                #     7,168 tiles (8,192 tokens) 42: 292, 142: 175 | 28,560 tiles (32,640 tokens) 42: 3,840, 142: 2,400
+                #   head size 128, 12 heads on 2:  768 tiles 22: 31.0, 42: 26.1, 141: 27.8 | 1,536 tiles 42: 47.1, 141: 47.3
+                #     3,072 tiles 42: 158, 141: 87;  28 heads on 4: 896 tiles 22: 28.8, 42: 16.3, 141: 19.3 | 1,792 tiles
+                #     42: 40.7, 141: 30.0 | 7,168 tiles 42: 341, 141: 190;  40 heads on 8: 1,280 tiles 42: 23.2, 141: 19.6
                 blocks_of_32 = page_size <= 64
                 if hd == 64:
                     shape = 24 if row_tiles <= 512 else 44 if row_tiles <= 1536 or not blocks_of_32 else 142
                     if shape == 44 and row_tiles > 2048:
                         shape = 42
                 else:
-                    shape = 22 if row_tiles <= 192 else 42 if row_tiles <= 1536 or not blocks_of_32 else 141
+                    shape = 22 if row_tiles <= 192 else 42 if row_tiles <= 1024 or not blocks_of_32 else 141
                 self._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(),
                           v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(),
                           kv_len.data_ptr(), b, t, nq, nkv, hd, page_size, float(scale), int(window), shape,
