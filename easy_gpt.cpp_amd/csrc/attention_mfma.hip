@@ -654,9 +654,10 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     // The loop is a pipeline of three stages over the tiles.  In the iteration of tile i a wavefront issues, as one
     // straight line of code, the score product of tile i + 1, the exponentials of tile i and the output product of tile
     // i - 1: the matrix instructions of the two products alternate with the vector instructions of the softmax between
-    // them (in groups whose order scheduling fences keep), so that both pipes work at once.  (With a tile's products on either side of its softmax, and the
-    // wavefronts of a workgroup in step from barrier to barrier, the pipes took turns: at 8,192 tokens the SIMDs issued
-    // vector instructions half of the time and did nothing for much of the rest.)  What does not fit into a straight
+    // them (in groups whose order scheduling fences keep), so that both pipes work at once.  (With a tile's products on
+    // either side of its softmax, and the wavefronts of a workgroup in step from barrier to barrier, the pipes took
+    // turns: at 8,192 tokens the SIMDs issued vector instructions half of the time and did nothing for much of the
+    // rest.)  What does not fit into a straight
     // line is kept out of it: masking (tiles on the diagonal or a window's edge) comes before it, and the accumulated
     // output is rescaled after it, and only when a row's maximum has grown by more than 2^kSlack since the last time:
     // until then the exponentials are taken against the old maximum, so they may reach 2^kSlack instead of 1, which
