@@ -70,11 +70,12 @@ def serve_workload(engine, args, vocab: int, name: str = "Qwen2.5-0.5B") -> dict
     from easy_gpt.cpp_amd.sampling import SamplingParams
 
     rnd = random.Random(0)
-    lens = [rnd.randint(128, 2048) for _ in range(SERVE_REQUESTS)]
+    lo, hi = (int(v) for v in args.serve_prompts.split(","))
+    lens = [rnd.randint(lo, hi) for _ in range(args.serve_requests)]
     g = torch.Generator().manual_seed(0)
     results = []
     for rep in range(2):                                       # the first pass warms up (graphs, library choices)
-        sched = Scheduler(engine, SchedulerConfig(max_active=SERVE_REQUESTS, max_admit_per_step=8,
+        sched = Scheduler(engine, SchedulerConfig(max_active=args.serve_requests, max_admit_per_step=8,
                                                   max_tokens_per_step=args.serve_budget,
                                                   prefill_chunk=min(SERVE_CHUNK, args.serve_budget)), eos_token_id=-1)
         if args.no_lookahead:
@@ -90,14 +91,14 @@ def serve_workload(engine, args, vocab: int, name: str = "Qwen2.5-0.5B") -> dict
         results.append((time.perf_counter() - t0, sched.stats))
         print(f"[bench] serve pass {rep}: {results[-1][0]:.2f} s, {sched.stats.steps} steps", file=sys.stderr, flush=True)
     sec, st = results[-1]
-    total = sum(lens) + SERVE_REQUESTS * SERVE_NEW_TOKENS
+    total = sum(lens) + args.serve_requests * SERVE_NEW_TOKENS
     return {
         "metric": f"tokens/s through the scheduler, prompts and generated ({name})", "value": round(total / sec, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(sec / st.steps * 1e3, 3),
         "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "generated_per_s": round(SERVE_REQUESTS * SERVE_NEW_TOKENS / sec, 1), "seconds": round(sec, 3),
+        "generated_per_s": round(args.serve_requests * SERVE_NEW_TOKENS / sec, 1), "seconds": round(sec, 3),
         "data": "synthetic: uniform-random token ids, random weights N(0, 0.02) from seed 0",
-        "config": {"model": f"{name} layer sizes", "requests": SERVE_REQUESTS, "prompt_tokens": sum(lens),
+        "config": {"model": f"{name} layer sizes", "requests": args.serve_requests, "prompt_tokens": sum(lens),
                    "new_tokens_each": SERVE_NEW_TOKENS, "prefill_chunk": min(SERVE_CHUNK, args.serve_budget),
                    "max_tokens_per_step": args.serve_budget,
                    "preemptions": st.preemptions, "steps_launched_ahead": st.steps_ahead, "sampling": "greedy"},
@@ -367,6 +368,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="tokens of the prompt that --prefill-only feeds in one step (the record's prefill is 2,048)")
     ap.add_argument("--serve-budget", type=int, default=2048, help="with --serve: the token budget of one step")
+    ap.add_argument("--serve-requests", type=int, default=SERVE_REQUESTS, help="with --serve: requests, submitted together")
+    ap.add_argument("--serve-prompts", default="128,2048", help="with --serve: prompt lengths are uniform in LOW,HIGH")
     ap.add_argument("--serve", action="store_true",
                     help="instead of fixed batches: 64 requests with prompts of 128 to 2,048 tokens and 256 new tokens "
                          "each through the scheduler, prompts in portions of 512 (the mixed serving workload)")
@@ -420,7 +423,8 @@ def main() -> int:
     new_tokens = max(NEW_TOKENS, args.warmup + args.steps)        # a longer run than the default decodes further
     tokens_per_request = -(-(PREFIX + new_tokens) // page_size) * page_size
     if args.serve:
-        max_batch, tokens_per_request = SERVE_REQUESTS, -(-(2048 + SERVE_NEW_TOKENS) // page_size) * page_size
+        longest = int(args.serve_prompts.split(",")[1])
+        max_batch, tokens_per_request = args.serve_requests, -(-(longest + SERVE_NEW_TOKENS) // page_size) * page_size
     engine = Engine.from_dir(tmp, dtype=args.dtype, device="cuda:0", page_size=page_size,
                              max_tokens=max_batch * tokens_per_request + max(PREFILL_TOKENS, args.prefill_tokens),
                              max_requests=max_batch + 1, tune_products=not args.no_tune)

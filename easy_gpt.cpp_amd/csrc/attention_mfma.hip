@@ -268,7 +268,7 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
-    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window) {
+    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window, int skip_single) {
     constexpr int KD = HD / 32, DT = HD / 16;
     constexpr int ROWS = 16 * RT;                // rows per workgroup
     constexpr int KT = 64 * KS;                  // keys per LDS tile
@@ -289,7 +289,8 @@ __global__ __launch_bounds__(64 * RT * KS) void attention_tiled_kernel(
 
     int b = 0, grp = blockIdx.x;
     for (; b < n_seqs; ++b) {
-        const int groups = (q_len[b] * group_size + ROWS - 1) / ROWS;
+        // (skip_single: requests of one token are the decode kernel's, which spreads their keys over wavefronts)
+        const int groups = (skip_single && q_len[b] == 1) ? 0 : (q_len[b] * group_size + ROWS - 1) / ROWS;
         if (grp < groups) {
             grp = groups - 1 - grp;          // the last rows first: they have the most keys to walk
             break;
@@ -565,7 +566,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
-    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window) {
+    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window, int skip_single) {
     constexpr int NQ = HD / 16;                  // steps of 16 features of the score product
     constexpr int FB = HD / 32;                  // blocks of 32 output features
     constexpr int ROWS = 32 * RB;
@@ -586,7 +587,8 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
 
     int b = 0, grp = blockIdx.x;
     for (; b < n_seqs; ++b) {
-        const int groups = (q_len[b] * group_size + ROWS - 1) / ROWS;
+        // (skip_single: requests of one token are the decode kernel's, which spreads their keys over wavefronts)
+        const int groups = (skip_single && q_len[b] == 1) ? 0 : (q_len[b] * group_size + ROWS - 1) / ROWS;
         if (grp < groups) {
             grp = groups - 1 - grp;          // the last rows first: they have the most keys to walk
             break;
@@ -994,9 +996,12 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ kv_len, int n_tokens, int nq, int nkv, int page_size, float scale, int window,
-    int n_splits, FusedQkv f) {
+    int n_splits, FusedQkv f, const int32_t* __restrict__ q_len) {
     constexpr int KD = HD / 32, DT = HD / 16;
     constexpr int kRow = HD + 2;
+    // q_len given: a step that also holds portions of prompts; this kernel takes its requests of one token, parts are
+    // kept by request (n_tokens is the number of requests then) and the rest is another kernel's
+    if (q_len != nullptr && q_len[blockIdx.x] != 1) return;
     extern __shared__ float wave_state[];          // [n_waves][16][HD + 2]: O, then maximum, then sum
     const int lane = threadIdx.x % kWave, n_waves = blockDim.x / kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // known to be the same for the wavefront
@@ -1300,7 +1305,8 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
         if (n_splits == 1) {
             out[(row0 + r) * HD + d] = from_float<bf16_t>(num / den);
         } else {
-            const size_t prow = static_cast<size_t>(split) * n_tokens * nq + row0 + r;
+            const size_t prow = static_cast<size_t>(split) * n_tokens * nq +
+                                (q_len != nullptr ? static_cast<size_t>(b) * nq + kh * group_size : row0) + r;
             part_o[prow * HD + d] = num;
             if (d == 0) {
                 part_ml[prow * 2] = mx;
@@ -1315,8 +1321,18 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
 // round of loads; the partial outputs are then read eight splits at a time.
 __global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __restrict__ part_o,
                                                               const float* __restrict__ part_ml,
-                                                              bf16_t* __restrict__ out, int n_rows, int hd, int n_splits) {
+                                                              bf16_t* __restrict__ out, int n_rows, int hd, int n_splits,
+                                                              const int32_t* __restrict__ q_start = nullptr,
+                                                              const int32_t* __restrict__ q_len = nullptr, int nq = 1) {
     const int row = blockIdx.x, lane = threadIdx.x;
+    // q_start given: the parts are kept by request, of which only those of one token have any, and the result goes
+    // to that token's row
+    int out_row = row;
+    if (q_start != nullptr) {
+        const int seq = row / nq;
+        if (q_len[seq] != 1) return;
+        out_row = q_start[seq] * nq + row % nq;
+    }
     // the first eight splits' parts are asked for together with their weights' inputs, not behind them (a part of a
     // split without visible keys may hold anything: it is read and then dropped)
     float first[8][4];
@@ -1362,7 +1378,7 @@ __global__ __launch_bounds__(64) void attention_reduce_kernel(const float* __res
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int d = lane + r * kWave;
-        if (d < hd) out[static_cast<size_t>(row) * hd + d] = from_float<bf16_t>(acc[r] * inv);
+        if (d < hd) out[static_cast<size_t>(out_row) * hd + d] = from_float<bf16_t>(acc[r] * inv);
     }
 }
 
@@ -1395,7 +1411,8 @@ template <int HD, int PF>
 static int launch_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,
                          const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size, float scale,
-                         int window, int n_splits, int n_waves, int combine, const FusedQkv* fused, hipStream_t s) {
+                         int window, int n_splits, int n_waves, int combine, const FusedQkv* fused,
+                         const int32_t* q_len, hipStream_t s) {
     dim3 grid(n_seqs, nkv, n_splits);
     size_t lds = static_cast<size_t>(n_waves) * 16 * (HD + 2) * sizeof(float);
     if (fused) lds += 18 * HD * sizeof(bf16_t);          // 16 query heads, the new key and value
@@ -1417,16 +1434,16 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
         attention_decode_kernel<HD, PF, true><<<grid, n_waves * kWave, lds, s>>>(
             nullptr, static_cast<bf16_t*>(out), part_o, part_ml, static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, kv_len, n_tokens, nq, nkv,
-            page_size, scale, window, n_splits, fq);
+            page_size, scale, window, n_splits, fq, nullptr);
     else
         attention_decode_kernel<HD, PF, false><<<grid, n_waves * kWave, lds, s>>>(
             static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
             static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
-            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq);
+            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq, q_len);
     EGPT_CHECK_LAUNCH();
     if (n_splits > 1 && combine) {
         attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
-                                                             HD, n_splits);
+                                                             HD, n_splits, q_len ? q_start : nullptr, q_len, nq);
         EGPT_CHECK_LAUNCH();
     }
     return EGPT_OK;
@@ -1436,11 +1453,12 @@ static int dispatch_decode(const void* qkv, void* out, float* part_o, float* par
                            const void* v_cache, const int32_t* block_table, int table_width, const int32_t* q_start,
                            const int32_t* kv_len, int n_seqs, int nq, int nkv, int hd, int page_size, float scale,
                            int window, int n_splits, int n_waves, int combine, bool lean, const FusedQkv* fused,
-                           hipStream_t s) {
+                           const int32_t* q_len, hipStream_t s) {
     // lean: the variant with half the loads in flight and fewer registers (the caller's choice, see the wrapper)
-#define EGPT_LAUNCH_DECODE(HD_, PF_)                                                                             \
+#define EGPT_LAUNCH_DECODE(HD_, PF_)                                                                                \
     launch_decode<HD_, PF_>(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len, \
-                            n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, fused, s)
+                            n_seqs, n_seqs, nq, nkv, page_size, scale, window, n_splits, n_waves, combine, fused,   \
+                            q_len, s)
     if (hd == 64) return lean ? EGPT_LAUNCH_DECODE(64, 2) : EGPT_LAUNCH_DECODE(64, 4);
     return lean ? EGPT_LAUNCH_DECODE(128, 1) : EGPT_LAUNCH_DECODE(128, 2);
 #undef EGPT_LAUNCH_DECODE
@@ -1457,39 +1475,46 @@ template <int HD, int RT, int KS>
 static void launch_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                          const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
                          const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size,
-                         int page_shift, float scale, int window, hipStream_t s) {
+                         int page_shift, float scale, int window, int skip_single, hipStream_t s) {
     const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (16 * RT) + n_seqs;   // upper bound
     dim3 grid(static_cast<unsigned>(groups), nkv);
     attention_tiled_kernel<HD, RT, KS><<<grid, 64 * RT * KS, 0, s>>>(
         static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
         static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
-        page_size, page_shift, scale, window);
+        page_size, page_shift, scale, window, skip_single);
 }
 
 template <int HD, int RB, int KS>
 static void launch_rows32(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                           const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
                           const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size,
-                          int page_shift, float scale, int window, hipStream_t s) {
+                          int page_shift, float scale, int window, int skip_single, hipStream_t s) {
     const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (32 * RB) + n_seqs;   // upper bound
     dim3 grid(static_cast<unsigned>(groups), nkv);
     attention_rows32_kernel<HD, RB, KS><<<grid, 64 * RB * KS, 0, s>>>(
         static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
         static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
-        page_size, page_shift, scale, window);
+        page_size, page_shift, scale, window, skip_single);
 }
 
 extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                                           const int32_t* block_table, int table_width, const int32_t* q_start,
                                           const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens,
                                           int nq, int nkv, int hd, int page_size, float scale, int window,
-                                          int shape, void* stream) {
+                                          int shape, float* part_o, float* part_ml, int single_splits,
+                                          int single_waves, int single_lean, void* stream) {
     if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
         return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0)
         return EGPT_BAD_ARGUMENT;
     if ((hd != 64 && hd != 128) || page_size < 16 || (page_size & (page_size - 1)) != 0 || nkv > 65535)
         return EGPT_UNSUPPORTED_SIZE;
+    const int skip_single = single_waves != 0;
+    if (skip_single) {
+        if (single_waves < 0 || single_splits < 1 || (single_splits > 1 && (!part_o || !part_ml)))
+            return EGPT_BAD_ARGUMENT;
+        if (nq / nkv > 16 || single_splits > 64 || single_waves > 8) return EGPT_UNSUPPORTED_SIZE;
+    }
     if (shape >= 100 && page_size > 64) return EGPT_UNSUPPORTED_SIZE;     // its tiles of 64 keys are whole pages
     if (n_tokens == 0) return EGPT_OK;
     int page_shift = 0;
@@ -1497,10 +1522,10 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define EGPT_TILED(HD_, RT_, KS_)                                                                                  \
     launch_tiled<HD_, RT_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,      \
-                                n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, s)
+                                n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, skip_single, s)
 #define EGPT_ROWS32(HD_, RB_, KS_)                                                                                 \
     launch_rows32<HD_, RB_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,     \
-                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, s)
+                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, skip_single, s)
     // shape = 10 * row tiles + key splits of a workgroup; 100 + 10 * blocks of 32 rows + key splits: the kernel of
     // 32-row blocks
     if (hd == 64) {
@@ -1531,6 +1556,10 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
 #undef EGPT_TILED
 #undef EGPT_ROWS32
     EGPT_CHECK_LAUNCH();
+    if (skip_single)
+        return dispatch_decode(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
+                               n_seqs, nq, nkv, hd, page_size, scale, window, single_splits, single_waves, 1,
+                               single_lean != 0, nullptr, q_len, s);
     return EGPT_OK;
 }
 
@@ -1550,7 +1579,7 @@ extern "C" int egpt_paged_attention_decode(const void* qkv, void* out, float* pa
         return EGPT_UNSUPPORTED_SIZE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_decode(qkv, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, nullptr, s);
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, nullptr, nullptr, s);
 }
 
 // The same with the QKV epilogue folded in: the queries, and the new token's key and value, are computed from
@@ -1584,7 +1613,7 @@ extern "C" int egpt_attention_decode_fused(const float* qkv_prod, int in_splits,
     f.k_cache_w = static_cast<bf16_t*>(k_cache); f.v_cache_w = static_cast<bf16_t*>(v_cache);
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_decode(nullptr, out, part_o, part_ml, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, &f, s);
+                           n_seqs, nq, nkv, hd, page_size, scale, window, n_splits, n_waves, combine, lean != 0, &f, nullptr, s);
 }
 
 // bfloat16 only; head size 64 or 128; page size a multiple of 16.  rows_per_wave: 16 (decoded tokens) or 32.

@@ -616,4 +616,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 14; }
+extern "C" int egpt_abi_version(void) { return 15; }

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 14:
+    if lib.egpt_abi_version() != 15:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -85,7 +85,8 @@ class HipKernels(KernelBackend):
             "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
-            "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp],
+            "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp, vp, i, i, i,
+                                           vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, i, vp],
             "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
                                             i, i, f, i, i, i, i, i, vp],
@@ -633,10 +634,20 @@ class HipKernels(KernelBackend):
                         shape = 42
                 else:
                     shape = 22 if row_tiles <= 192 else 42 if row_tiles <= 1024 or not blocks_of_32 else 141
+                # Requests that bring one token (decoded tokens beside the portions) go to the decode kernel in a second
+                # launch: here one workgroup would walk all of such a request's keys, 128 or 256 per iteration of some
+                # 1.7 us, and the longest of them sets the launch's time
+                part_o = part_ml = None
+                n_splits = n_waves = lean = 0
+                if b > 1 and nq // nkv <= 16 and max_kv_len > self.singles_apart_beyond:
+                    n_splits, n_waves, lean = self._decode_shape(b, nkv, hd, max_kv_len, True)
+                    if n_splits > 1:
+                        part_o = torch.empty((n_splits, b, nq, hd), dtype=_F32, device=qkv.device)
+                        part_ml = torch.empty((n_splits, b, nq, 2), dtype=_F32, device=qkv.device)
                 self._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(),
                           v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(),
                           kv_len.data_ptr(), b, t, nq, nkv, hd, page_size, float(scale), int(window), shape,
-                          self._stream())
+                          self._ptr(part_o), self._ptr(part_ml), n_splits, n_waves, lean, self._stream())
                 return None
             n_splits = max(1, min(1024 // (b * nkv), -(-max_kv_len // 64), 64))
             part_o = part_ml = None
@@ -669,6 +680,13 @@ class HipKernels(KernelBackend):
                   block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(), kv_len.data_ptr(), b, t,
                   nq, nkv, hd, page_size, float(scale), int(window), dt, self._stream())
 
+    # A mixed step's requests of one token go to the decode kernel when the step's longest context is beyond this: the
+    # second launch (and a third that combines key ranges) costs some 8 us, a workgroup of the tiled kernel that walks
+    # 4,000 keys alone some 30.  Measured, us for one layer's attention of the 0.5B sizes, tiled kernel alone against
+    # the two: one portion of 512 tokens beside 8 decoded tokens behind 600 keys each 11.0 against 18.3, behind 1,300
+    # 16.2 against 18.6, behind 4,000 33.2 against 20.5, behind 16,000 122 against 32; four portions beside 24 decoded
+    # tokens behind 1,300 keys 36.7 against 38.1, behind 4,000 61.6 against 43.5, behind 16,000 152 against 66
+    singles_apart_beyond = 2048
     attention_segment = 64       # keys per segment of the decode kernel for any head size (kSegment in attention_any.hip)
 
     @staticmethod

@@ -631,7 +631,8 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3, ramp=0.0):
     return kc.to(DEV), vc.to(DEV), table.to(DEV), keys, vals
 
 
-def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None, ramp=0.0):
+def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None, ramp=0.0,
+              singles=(0, 0, 0)):
     kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed, ramp=ramp)
     t = sum(q for q, _ in seqs)
     g = torch.Generator().manual_seed(seed + 100)
@@ -649,10 +650,14 @@ def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, ti
                           scale, window, int(q_len.max()), int(kv_len.max()))
     else:
         # the LDS-tiled kernel with a given workgroup shape (the wrapper picks one by the amount of work)
+        # singles = (key ranges, wavefronts, lean variant) of the decode kernel that takes the requests of one token
         qs, ql, kl = q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV)
+        part_o = torch.full((singles[0], len(seqs), nq, hd), float("nan"), device=DEV)
+        part_ml = torch.full((singles[0], len(seqs), nq, 2), float("nan"), device=DEV)
+        out.fill_(float("nan"))
         k._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), kc.data_ptr(), vc.data_ptr(),
                table.data_ptr(), table.shape[1], qs.data_ptr(), ql.data_ptr(), kl.data_ptr(), len(seqs), t, nq, nkv,
-               hd, ps, scale, window, tiled_shape, k._stream())
+               hd, ps, scale, window, tiled_shape, k._ptr(part_o), k._ptr(part_ml), *singles, k._stream())
         torch.cuda.synchronize()
     got = out.double().cpu().view(t, nq, hd)
     worst = 0.0
@@ -783,7 +788,27 @@ def test_paged_attention_tiled_refuses_other_page_sizes(k):
     # not a power of two, too small, no such shape, pages larger than the tiles of the kernel of 32-row blocks
     for ps, shape in ((48, 42), (8, 42), (16, 43), (128, 142)):
         with pytest.raises(RuntimeError):
-            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, None)
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, None, None,
+                   0, 0, 0, None)
+    # single tokens to the decode kernel: more than 16 heads to a group, key ranges without room for their parts
+    for nq, splits, parts in ((17, 1, None), (2, 2, None), (2, 65, p)):
+        with pytest.raises(RuntimeError):
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, nq, 1, 64, 16, 0.1, 0, 42, parts, parts,
+                   splits, 4, 0, None)
+
+
+@pytest.mark.parametrize("hd,shape", [(64, 24), (64, 44), (64, 142), (128, 42), (128, 141)])
+@pytest.mark.parametrize("singles", [(1, 8, 0), (1, 1, 1), (3, 4, 1), (7, 8, 0)])
+def test_a_mixed_step_hands_its_single_tokens_to_the_decode_kernel(k, hd, shape, singles):
+    # portions beside requests of one token behind short and long contexts; the key ranges' parts are kept by
+    # request, the results go to the tokens' rows; the keys' ramp makes every far key count
+    seqs = [(70, 300), (1, 2500), (1, 77), (33, 33), (1, 1), (1, 4100), (2, 900), (1, 64)]
+    r = 8.0 / 4100
+    assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, tiled_shape=shape, singles=singles, seed=21, ramp=r) <= 1.2e-2
+    assert run_paged(k, seqs, 16, 1, hd, 32, torch.bfloat16, window=700, tiled_shape=shape, singles=singles, seed=22) <= 1.2e-2
+    # nothing but single tokens and one portion at the end; no single tokens at all
+    assert run_paged(k, [(1, 500)] * 5 + [(40, 1000)], 3, 3, hd, 64, torch.bfloat16, tiled_shape=shape, singles=singles, seed=23) <= 1.2e-2
+    assert run_paged(k, [(5, 500), (40, 1000)], 4, 2, hd, 16, torch.bfloat16, tiled_shape=shape, singles=singles, seed=24) <= 1.2e-2
 
 
 @pytest.mark.parametrize("nq,nkv,hd", [(14, 2, 64), (12, 2, 128), (3, 1, 64)])

@@ -94,6 +94,27 @@ def test_mixed_batches_with_page_reuse(sharp_models, name, dtype):
         assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16"])
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_mixed_batches_whose_single_tokens_go_to_the_decode_kernel(sharp_models, name, dtype, monkeypatch):
+    # what steps with contexts beyond some thousand tokens do, here at every length: the requests that bring one
+    # token are left out by the kernel of the portions and taken by the decode kernel in a launch of its own
+    from easy_gpt.cpp_amd.kernels import hip
+
+    monkeypatch.setattr(hip.HipKernels, "singles_apart_beyond", 0)
+    cfg = TINY[name][0]
+    cap = cfg["max_position_embeddings"]
+    reqs = H.make_requests(cfg["vocab_size"], [min(n, cap) for n in (70, 23, 110, 64, 37, 90, 128, 16)], seed=33)
+    ref = H.plain_rows(sharp_models[name], reqs, bf16_weights=True)
+    trace = H.trace_mixed(reqs, seed=3, decode_tail=20)
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, round_to=16))
+    H.assert_rows_match(H.replay(eng, trace), ref, tol_of(dtype), f"{name} mixed, single tokens apart")
+    assert any(len(r["entries"]) > 1 and {len(e["tokens"]) for e in r["entries"]} > {1} for r in trace)
+    # the same steps kernel by kernel, not from replayed graphs
+    eng = engine_for(sharp_models[name], dtype, max_tokens=H.max_live_tokens(trace, round_to=16), use_graphs=False)
+    H.assert_rows_match(H.replay(eng, trace), ref, tol_of(dtype), f"{name} mixed, single tokens apart, no graphs")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["B", "D"])
 def test_the_general_step_kernel_by_kernel(sharp_models, name, dtype):
