@@ -439,6 +439,12 @@ class HipKernels(KernelBackend):
         n, k = w.shape
         if w.dtype != _BF16 or k != nq * hd or not 0 < t <= self.fused_rows or hd % 8 or a_splits > 64:
             return None
+        if n * k > 16 << 20:
+            # every workgroup combines the parts of its range of k before it has anything to multiply, and on a matrix
+            # this large there are some 40 columns of workgroups that each do so: a kernel that combines the parts once
+            # and the plain product are faster (measured, us for 8 rows: 5,120 x 5,120 28.3 against 18.2; 3,584 x 3,584
+            # 11.7 against 11.8, 2,048 x 2,048 6.2 against 8.8, 896 x 896 4.1 against 6.6)
+            return None
         self._need(part_o, "part_o", _F32)
         self._need(part_ml, "part_ml", _F32, (a_splits, t, nq, 2))
         self._need(w, "w", _BF16)
@@ -746,6 +752,13 @@ class HipKernels(KernelBackend):
             # 3.11 against 3.27; at the 1.5B sizes batch 128 4.03 against 4.20; at the 7B sizes, four kv heads, batch
             # 64 6.56 against 6.71 and batch 128 9.87 against 10.06)
             n_splits, n_waves = 1, 8 if pairs <= 256 else 4
+        elif not n_waves and 32 < pairs <= 64 and key_blocks >= 64:
+            # and with 33 to 64 pairs as many key ranges of eight wavefronts as give every workgroup a CU of its own
+            # (measured, ms a step against the rule below, which takes 8 ranges of four wavefronts: at the 1.5B sizes
+            # behind 2,048 tokens batch 32 2.31 against 2.42 and batch 24 2.21 against 2.27; at the 7B sizes behind 4,096
+            # tokens batch 16 5.04 against 5.23; at the 14B sizes, eight kv heads, batch 8 9.00 against 9.50; at the 0.5B
+            # sizes behind 8,192 tokens batch 32 1.82 against 1.87 and batch 24 1.63 against 1.67)
+            n_splits, n_waves = 256 // pairs, 8
         if not n_waves:
             n_splits, n_waves = splits_for(4), 4
             # head size 128: eight wavefronts as well while every workgroup has a CU of its own (its 71 KB of LDS are

@@ -782,6 +782,14 @@ def test_prompt_attention_with_scores_that_grow_along_the_keys(k, hd, shape, ram
     assert run_paged(k, [(90, 400), (1, 77)], 16, 1, hd, 16, torch.bfloat16, tiled_shape=shape, seed=12, ramp=r) <= 1.2e-2
 
 
+def test_attention_parts_before_a_large_output_projection_are_combined_apart(k):
+    # the product that combines the parts itself is for matrices on which that pays; beyond, the caller combines
+    po = torch.zeros(2, 1, 40, 128, device=DEV)
+    pml = torch.zeros(2, 1, 40, 2, device=DEV)
+    assert k.product_attention(po, pml, torch.empty(5120, 5120, dtype=torch.bfloat16, device=DEV)) is None
+    assert k.product_attention(po, pml, torch.zeros(1024, 5120, dtype=torch.bfloat16, device=DEV)) is not None
+
+
 def test_paged_attention_tiled_refuses_other_page_sizes(k):
     z = torch.zeros(64, device=DEV)
     p = z.data_ptr()
