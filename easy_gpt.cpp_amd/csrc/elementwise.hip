@@ -59,10 +59,11 @@ __global__ void add_rmsnorm_kernel(R* __restrict__ h, ProductView<T> delta,
     const bool has_delta = delta.present();
     const size_t dbase = src * hidden;
     const bool write_back = (rows == nullptr) && has_delta;
-    // A row of up to four values per thread stays in registers, with its norm weight: all of a thread's loads are
+    // A row of up to eight values per thread stays in registers, with its norm weight: all of a thread's loads are
     // issued together, and the sum over the workgroup is the only wait between them and the stores.  (A loop over
-    // the row instead waits for memory once per round: 10 us for a row of 3,584 values with 512 threads.)
-    constexpr int KEEP = 4;
+    // the row instead waits for memory once per round: 10 us for a row of 3,584 values with 512 threads, 9 us for
+    // one of 5,120 with 1,024.)
+    constexpr int KEEP = 8;
     if (hidden <= KEEP * static_cast<int>(blockDim.x)) {
         float v[KEEP], w[KEEP];
 #pragma unroll
@@ -456,7 +457,7 @@ extern "C" int egpt_add_rmsnorm(void* h, int fixed, const void* delta, int delta
     if (n_rows == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for; and
-    // enough threads for a row to stay in registers (four values a thread)
+    // enough threads for a row to stay in registers (up to eight values a thread)
     const int threads = (delta_splits > 1 || hidden > 2048) ? 1024 : (hidden > 1024 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
     if (dtype == 1 && delta_splits <= 1 && hidden % 8 == 0 && n_rows >= 32 && !fixed) {

@@ -45,7 +45,8 @@ def test_embed(k, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hidden,eps,n_rows", [(72, 1e-6, 7), (896, 1e-5, 7), (3000, 1e-2, 7), (896, 1e-6, 70), (3000, 1e-5, 33),
                                                (100, 1e-6, 40), (896, 1e-6, 601), (1536, 1e-5, 512), (2000, 1e-6, 513),
-                                               (2056, 1e-6, 600), (5000, 1e-6, 7), (4104, 1e-5, 33), (8192, 1e-6, 7)])
+                                               (2056, 1e-6, 600), (5000, 1e-6, 7), (4104, 1e-5, 33), (8192, 1e-6, 7), (5120, 1e-6, 8),
+                                               (8200, 1e-6, 3), (12288, 1e-5, 2)])
 def test_add_rmsnorm(k, dtype, hidden, eps, n_rows):
     h = rnd(n_rows, hidden, seed=1, scale=2.0)
     delta = rnd(n_rows, hidden, dtype=dtype, seed=2)
