@@ -63,15 +63,20 @@ int egpt_paged_attention_mfma(const void* qkv, void* out, float* part_o, float* 
 // Prompt portions: the wavefronts of a workgroup share key/value tiles through LDS (n_splits == 1 semantics);
 // page sizes that are powers of two; shape = 10 * row tiles + key splits per workgroup (41, 42, 44, 22, 24), or
 // 100 + 10 * blocks of 32 rows + key splits (121, 122, 124, 141, 142; page sizes up to 64).
+// key_splits > 1 (shapes from 100 on): the tiles of keys that a block of rows walks are dealt over as many workgroups,
+// whose results part_o [key_splits][n_tokens][nq][hd] and part_ml [key_splits][n_tokens][nq][2] (float32) hold until a
+// second kernel has combined them.
 // single_waves > 0 (needs nq / nkv <= 16): the requests of the step that bring one token are left out here and taken
-// by the decode kernel in a second launch, which spreads a request's keys over the single_waves (1..8) wavefronts of a
+// by the decode kernel in a launch behind, which spreads a request's keys over the single_waves (1..8) wavefronts of a
 // workgroup and over single_splits key ranges; with single_splits > 1, part_o [single_splits][n_seqs][nq][hd] and
-// part_ml [single_splits][n_seqs][nq][2] (float32) hold those ranges' results until they are combined.
+// part_ml [single_splits][n_seqs][nq][2] hold those ranges' results until they are combined (the same memory as
+// above, used after it: it must hold the larger of the two).
 int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                                const int32_t* block_table, int table_width, const int32_t* q_start,
                                const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv,
-                               int hd, int page_size, float scale, int window, int shape, float* part_o,
-                               float* part_ml, int single_splits, int single_waves, int single_lean, void* stream);
+                               int hd, int page_size, float scale, int window, int shape, int key_splits,
+                               float* part_o, float* part_ml, int single_splits, int single_waves, int single_lean,
+                               void* stream);
 // One decoded token per request: workgroups of n_waves wavefronts per (request, kv head, key split); lean != 0: the
 // variant with half the loads in flight per round and fewer registers.
 int egpt_paged_attention_decode(const void* qkv, void* out, float* part_o, float* part_ml, const void* k_cache,

@@ -566,7 +566,8 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ kv_len,
-    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window, int skip_single) {
+    int n_seqs, int nq, int nkv, int page_size, int page_shift, float scale, int window, int skip_single,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int n_tokens) {
     constexpr int NQ = HD / 16;                  // steps of 16 features of the score product
     constexpr int FB = HD / 32;                  // blocks of 32 output features
     constexpr int ROWS = 32 * RB;
@@ -606,7 +607,12 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const int blk_p_hi = kv - n + blk_last / group_size;
     const int blk_first_pos = kv - n + blk_first / group_size;
     const int blk_lo = window > 0 ? max(0, blk_first_pos - window + 1) : 0;
-    const int t_begin = blk_lo / KT, t_end = blk_p_hi / KT + 1;
+    // n_splits > 1: the tiles of keys are dealt over as many workgroups (blockIdx.z), each of which leaves its rows'
+    // unnormalised result with its maximum and sum in part_o / part_ml for the kernel that combines them
+    const int t_first = blk_lo / KT, t_last = blk_p_hi / KT + 1;
+    const int t_per = max((t_last - t_first + n_splits - 1) / n_splits, 4);    // (a few tiles are not worth sharing)
+    const int t_begin = t_first + static_cast<int>(blockIdx.z) * t_per, t_end = min(t_last, t_begin + t_per);
+    const size_t part_row0 = static_cast<size_t>(blockIdx.z) * n_tokens * nq;
 
     // this wavefront's block of 32 rows, this lane's row
     const int row_base = blk_first + rb * 32;
@@ -633,6 +639,14 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
         }
     }
     const float scale2 = scale * 1.4426950408889634f;
+    if (t_begin >= t_end) {                  // (n_splits > 1 only) no tile of keys is left for this workgroup
+        if (valid && ksi == 0 && lh == 0) {
+            float* ml = part_ml + (part_row0 + static_cast<size_t>(tok) * nq + head) * 2;
+            ml[0] = -INFINITY;
+            ml[1] = 0.f;
+        }
+        return;
+    }
 
     f32x16 o[FB];
 #pragma unroll
@@ -910,6 +924,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     if constexpr (KS > 1) __syncthreads();           // the combination below writes over the tiles
     // the row's sum: feature 0 of the block of ones, which lane lr of half 0 holds
     float l = __shfl(o_sum[0], lr, kWave);
+    float m_part = m_run;                            // the maximum that o and l are in units of
     if constexpr (KS > 1) {
         // The wavefronts of one block of rows hold partial results over their keys: those with ks > 0 leave
         // theirs in LDS (the tiles are no longer read: the loop ended with a barrier), ks == 0 adds them up.
@@ -929,6 +944,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
 #pragma unroll
         for (int j = 0; j < KS - 1; ++j)
             m_all = fmaxf(m_all, comb[(static_cast<size_t>(j * RB + rb) * PER_LANE + FB * 16) * 64 + lane]);
+        m_part = m_all;
         const float m_ref = m_all == -INFINITY ? 0.f : m_all;
         const float w0 = __builtin_amdgcn_exp2f((m_run - m_ref) * scale2);
         l *= w0;
@@ -946,6 +962,25 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
 #pragma unroll
                 for (int e = 0; e < 16; ++e) o[f][e] += src[(f * 16 + e) * 64] * wj;
         }
+    }
+    if (n_splits > 1) {
+        // (element e of block f is feature f * 32 + (e / 4) * 8 + lh * 4 + e % 4: runs of four features; the maximum
+        // goes out in units of the exponent's argument, as the combining kernel takes it; -inf: no key seen)
+        if (valid) {
+            const size_t prow = part_row0 + static_cast<size_t>(tok) * nq + head;
+            float* po = part_o + prow * HD + lh * 4;
+#pragma unroll
+            for (int f = 0; f < FB; ++f)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    *reinterpret_cast<float4*>(po + f * 32 + g * 8) =
+                        float4{o[f][g * 4], o[f][g * 4 + 1], o[f][g * 4 + 2], o[f][g * 4 + 3]};
+            if (lh == 0) {
+                part_ml[prow * 2] = m_part * scale;
+                part_ml[prow * 2 + 1] = l;
+            }
+        }
+        return;
     }
     if (valid) {
         // element e of block f is feature f * 32 + (e / 4) * 8 + lh * 4 + e % 4: runs of four features
@@ -1488,21 +1523,27 @@ template <int HD, int RB, int KS>
 static void launch_rows32(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                           const int32_t* block_table, int table_width, const int32_t* q_start, const int32_t* q_len,
                           const int32_t* kv_len, int n_seqs, int n_tokens, int nq, int nkv, int page_size,
-                          int page_shift, float scale, int window, int skip_single, hipStream_t s) {
+                          int page_shift, float scale, int window, int skip_single, float* part_o, float* part_ml,
+                          int n_splits, hipStream_t s) {
     const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (32 * RB) + n_seqs;   // upper bound
-    dim3 grid(static_cast<unsigned>(groups), nkv);
+    dim3 grid(static_cast<unsigned>(groups), nkv, n_splits);
     attention_rows32_kernel<HD, RB, KS><<<grid, 64 * RB * KS, 0, s>>>(
         static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
         static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
-        page_size, page_shift, scale, window, skip_single);
+        page_size, page_shift, scale, window, skip_single, part_o, part_ml, n_splits, n_tokens);
+    // (the rows of requests that were left out have no parts: what is combined for them is written over by the
+    // kernel that takes them, which runs behind this one)
+    if (n_splits > 1)
+        attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
+                                                             HD, n_splits);
 }
 
 extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void* k_cache, const void* v_cache,
                                           const int32_t* block_table, int table_width, const int32_t* q_start,
                                           const int32_t* q_len, const int32_t* kv_len, int n_seqs, int n_tokens,
                                           int nq, int nkv, int hd, int page_size, float scale, int window,
-                                          int shape, float* part_o, float* part_ml, int single_splits,
-                                          int single_waves, int single_lean, void* stream) {
+                                          int shape, int key_splits, float* part_o, float* part_ml,
+                                          int single_splits, int single_waves, int single_lean, void* stream) {
     if (!qkv || !out || !k_cache || !v_cache || !block_table || !q_start || !q_len || !kv_len)
         return EGPT_BAD_ARGUMENT;
     if (n_seqs <= 0 || n_tokens < 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || table_width <= 0 || window < 0)
@@ -1516,6 +1557,8 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
         if (nq / nkv > 16 || single_splits > 64 || single_waves > 8) return EGPT_UNSUPPORTED_SIZE;
     }
     if (shape >= 100 && page_size > 64) return EGPT_UNSUPPORTED_SIZE;     // its tiles of 64 keys are whole pages
+    if (key_splits < 1 || (key_splits > 1 && (!part_o || !part_ml))) return EGPT_BAD_ARGUMENT;
+    if (key_splits > 64 || (key_splits > 1 && shape < 100)) return EGPT_UNSUPPORTED_SIZE;
     if (n_tokens == 0) return EGPT_OK;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
@@ -1525,7 +1568,8 @@ extern "C" int egpt_paged_attention_tiled(const void* qkv, void* out, const void
                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, skip_single, s)
 #define EGPT_ROWS32(HD_, RB_, KS_)                                                                                 \
     launch_rows32<HD_, RB_, KS_>(qkv, out, k_cache, v_cache, block_table, table_width, q_start, q_len, kv_len,     \
-                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, skip_single, s)
+                                 n_seqs, n_tokens, nq, nkv, page_size, page_shift, scale, window, skip_single,     \
+                                 part_o, part_ml, key_splits, s)
     // shape = 10 * row tiles + key splits of a workgroup; 100 + 10 * blocks of 32 rows + key splits: the kernel of
     // 32-row blocks
     if (hd == 64) {

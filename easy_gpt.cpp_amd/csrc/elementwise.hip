@@ -617,4 +617,4 @@ extern "C" const char* egpt_error_string(int code) {
     }
 }
 
-extern "C" int egpt_abi_version(void) { return 15; }
+extern "C" int egpt_abi_version(void) { return 16; }

@@ -28,7 +28,7 @@ def _load_library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except (build.BuildError, OSError) as e:
         raise KernelsUnavailable(f"the HIP kernel library could not be built or loaded: {e}") from e
-    if lib.egpt_abi_version() != 15:
+    if lib.egpt_abi_version() != 16:
         raise KernelsUnavailable(f"{path} has an unexpected ABI version")
     return lib
 
@@ -85,8 +85,8 @@ class HipKernels(KernelBackend):
             "egpt_gemm_skinny_swiglu": [vp, i, vp, i, i, f, vp, vp, vp, i, i, i, i, i, vp],
             "egpt_gemm_skinny_attn": [vp, vp, i, i, i, vp, vp, vp, i, i, i, i, vp],
             "egpt_attention_combine": [vp, vp, vp, i, i, i, vp],
-            "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, vp, vp, i, i, i,
-                                           vp],
+            "egpt_paged_attention_tiled": [vp, vp, vp, vp, vp, i, vp, vp, vp, i, i, i, i, i, i, f, i, i, i, vp, vp, i, i,
+                                           i, vp],
             "egpt_paged_attention_decode": [vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i, i, i, f, i, i, i, i, i, vp],
             "egpt_attention_decode_fused": [vp, i, vp, i, i, f, vp, vp, vp, vp, vp, vp, vp, vp, vp, i, vp, vp, i, i, i,
                                             i, i, f, i, i, i, i, i, vp],
@@ -640,6 +640,22 @@ class HipKernels(KernelBackend):
                         shape = 42
                 else:
                     shape = 22 if row_tiles <= 192 else 42 if row_tiles <= 1024 or not blocks_of_32 else 141
+                # Portions behind a prefix walk many keys per row and are few blocks of rows: the kernel of 32-row blocks
+                # with 128 rows to a workgroup, and the tiles of keys of a block of rows dealt over as many workgroups
+                # as give every CU one.  Measured (us, a layer; shape x workgroups that share the keys): head size 64,
+                # 14 heads on 2, 512 tokens behind 4,096 / 8,192 / 32,768 keys 24x1: 35 / 70 / 257, 124x1: 32 / 59 / 196,
+                # 142x1: 45 / 84 / 300, 142x4: 27 / 38 / 98; 256 tokens behind 32,768 124x1: 195, 124x4: 66, 142x8: 57; 64
+                # tokens 124x1: 201, 142x16: 40; behind 2,048 keys nothing is gained (24x1: 24, 142x4: 23) and a prompt
+                # without a prefix loses (2,048 tokens 142x1: 28, 142x2: 47); three portions of 512 behind 30,000 keys
+                # 142x1: 283, 124x1: 397.  Head size 128, 12 heads on 2, 512 tokens behind 2,048 / 32,768 keys 42x1: 59 /
+                # 643, 141x1: 59 / 665, 141x4: 30 / 185; 28 heads on 4: 141x1: 61 / 671, 141x2: 48 / 378; 40 heads on 8
+                # (160 workgroups): 141x1: 103 / 679.
+                key_splits = 1
+                if blocks_of_32 and max_kv_len >= (self.prefix_keys if hd == 64 else self.prefix_keys // 2):
+                    shape = 142 if hd == 64 else 141
+                    workgroups = -(-row_tiles // 8)
+                    tiles = -(-max_kv_len // (64 * (shape % 10)))
+                    key_splits = max(1, min(256 // workgroups, tiles // 4, 16))
                 # Requests that bring one token (decoded tokens beside the portions) go to the decode kernel in a second
                 # launch: here one workgroup would walk all of such a request's keys, 128 or 256 per iteration of some
                 # 1.7 us, and the longest of them sets the launch's time
@@ -647,12 +663,13 @@ class HipKernels(KernelBackend):
                 n_splits = n_waves = lean = 0
                 if b > 1 and nq // nkv <= 16 and max_kv_len > self.singles_apart_beyond:
                     n_splits, n_waves, lean = self._decode_shape(b, nkv, hd, max_kv_len, True)
-                    if n_splits > 1:
-                        part_o = torch.empty((n_splits, b, nq, hd), dtype=_F32, device=qkv.device)
-                        part_ml = torch.empty((n_splits, b, nq, 2), dtype=_F32, device=qkv.device)
+                parts_rows = max(n_splits * b if n_splits > 1 else 0, key_splits * t if key_splits > 1 else 0)
+                if parts_rows:
+                    part_o = torch.empty((parts_rows, nq, hd), dtype=_F32, device=qkv.device)
+                    part_ml = torch.empty((parts_rows, nq, 2), dtype=_F32, device=qkv.device)
                 self._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), k_cache.data_ptr(),
                           v_cache.data_ptr(), block_table.data_ptr(), width, q_start.data_ptr(), q_len.data_ptr(),
-                          kv_len.data_ptr(), b, t, nq, nkv, hd, page_size, float(scale), int(window), shape,
+                          kv_len.data_ptr(), b, t, nq, nkv, hd, page_size, float(scale), int(window), shape, key_splits,
                           self._ptr(part_o), self._ptr(part_ml), n_splits, n_waves, lean, self._stream())
                 return None
             n_splits = max(1, min(1024 // (b * nkv), -(-max_kv_len // 64), 64))
@@ -693,6 +710,7 @@ class HipKernels(KernelBackend):
     # 16.2 against 18.6, behind 4,000 33.2 against 20.5, behind 16,000 122 against 32; four portions beside 24 decoded
     # tokens behind 1,300 keys 36.7 against 38.1, behind 4,000 61.6 against 43.5, behind 16,000 152 against 66
     singles_apart_beyond = 2048
+    prefix_keys = 4096           # a step's longest context from which its portions are taken to lie behind a prefix
     attention_segment = 64       # keys per segment of the decode kernel for any head size (kSegment in attention_any.hip)
 
     @staticmethod

@@ -46,7 +46,7 @@ def test_embed(k, dtype):
 @pytest.mark.parametrize("hidden,eps,n_rows", [(72, 1e-6, 7), (896, 1e-5, 7), (3000, 1e-2, 7), (896, 1e-6, 70), (3000, 1e-5, 33),
                                                (100, 1e-6, 40), (896, 1e-6, 601), (1536, 1e-5, 512), (2000, 1e-6, 513),
                                                (2056, 1e-6, 600), (5000, 1e-6, 7), (4104, 1e-5, 33), (8192, 1e-6, 7), (5120, 1e-6, 8),
-                                               (8200, 1e-6, 3), (12288, 1e-5, 2)])
+                                               (8200, 1e-6, 7), (12288, 1e-5, 7)])
 def test_add_rmsnorm(k, dtype, hidden, eps, n_rows):
     h = rnd(n_rows, hidden, seed=1, scale=2.0)
     delta = rnd(n_rows, hidden, dtype=dtype, seed=2)
@@ -633,7 +633,7 @@ def build_paged(seqs, nkv, hd, ps, dtype, seed=0, extra_pages=3, ramp=0.0):
 
 
 def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, tiled_shape=None, ramp=0.0,
-              singles=(0, 0, 0)):
+              singles=(0, 0, 0), key_splits=1):
     kc, vc, table, keys, vals = build_paged(seqs, nkv, hd, ps, dtype, seed, ramp=ramp)
     t = sum(q for q, _ in seqs)
     g = torch.Generator().manual_seed(seed + 100)
@@ -653,12 +653,14 @@ def run_paged(k, seqs, nq, nkv, hd, ps, dtype, window=0, seed=0, q_scale=1.0, ti
         # the LDS-tiled kernel with a given workgroup shape (the wrapper picks one by the amount of work)
         # singles = (key ranges, wavefronts, lean variant) of the decode kernel that takes the requests of one token
         qs, ql, kl = q_start.to(DEV), q_len.to(DEV), kv_len.to(DEV)
-        part_o = torch.full((singles[0], len(seqs), nq, hd), float("nan"), device=DEV)
-        part_ml = torch.full((singles[0], len(seqs), nq, 2), float("nan"), device=DEV)
+        # key_splits: workgroups that share the keys of a block of rows; both leave parts in the same memory
+        part_rows = max(singles[0] * len(seqs), key_splits * t if key_splits > 1 else 0)
+        part_o = torch.full((part_rows, nq, hd), float("nan"), device=DEV)
+        part_ml = torch.full((part_rows, nq, 2), float("nan"), device=DEV)
         out.fill_(float("nan"))
         k._run("egpt_paged_attention_tiled", qkv.data_ptr(), out.data_ptr(), kc.data_ptr(), vc.data_ptr(),
                table.data_ptr(), table.shape[1], qs.data_ptr(), ql.data_ptr(), kl.data_ptr(), len(seqs), t, nq, nkv,
-               hd, ps, scale, window, tiled_shape, k._ptr(part_o), k._ptr(part_ml), *singles, k._stream())
+               hd, ps, scale, window, tiled_shape, key_splits, k._ptr(part_o), k._ptr(part_ml), *singles, k._stream())
         torch.cuda.synchronize()
     got = out.double().cpu().view(t, nq, hd)
     worst = 0.0
@@ -783,6 +785,23 @@ def test_prompt_attention_with_scores_that_grow_along_the_keys(k, hd, shape, ram
     assert run_paged(k, [(90, 400), (1, 77)], 16, 1, hd, 16, torch.bfloat16, tiled_shape=shape, seed=12, ramp=r) <= 1.2e-2
 
 
+@pytest.mark.parametrize("hd,shape", [(64, 124), (64, 142), (64, 122), (64, 121), (128, 141), (128, 122)])
+@pytest.mark.parametrize("key_splits", [2, 3, 7])
+def test_portions_whose_blocks_of_rows_share_their_keys_among_workgroups(k, hd, shape, key_splits):
+    # portions behind prefixes of different lengths (one with fewer tiles of keys than workgroups that share them), a
+    # fresh prompt, a window; the keys' ramp makes every far key count, so a range that is left out or taken twice shows
+    seqs = [(70, 1300), (33, 33), (5, 2100), (130, 130), (40, 700)]
+    r = 8.0 / 2100
+    assert run_paged(k, seqs, 6, 2, hd, 16, torch.bfloat16, tiled_shape=shape, key_splits=key_splits, seed=31, ramp=r) <= 1.2e-2
+    assert run_paged(k, seqs, 7, 1, hd, 64, torch.bfloat16, window=500, tiled_shape=shape, key_splits=key_splits, seed=32) <= 1.2e-2
+    assert run_paged(k, seqs, 4, 4, hd, 32, torch.bfloat16, tiled_shape=shape, key_splits=key_splits, seed=33, q_scale=5.0) <= 4e-2
+    # with the requests of one token taken by the decode kernel behind it, parts in the same memory
+    mixed = [(70, 1300), (1, 2500), (1, 77), (33, 33), (1, 1), (2, 900)]
+    for singles in ((1, 8, 0), (5, 4, 1)):
+        assert run_paged(k, mixed, 6, 2, hd, 16, torch.bfloat16, tiled_shape=shape, key_splits=key_splits, singles=singles,
+                         seed=34, ramp=8.0 / 2500) <= 1.2e-2
+
+
 def test_attention_parts_before_a_large_output_projection_are_combined_apart(k):
     # the product that combines the parts itself is for matrices on which that pays; beyond, the caller combines
     po = torch.zeros(2, 1, 40, 128, device=DEV)
@@ -797,12 +816,17 @@ def test_paged_attention_tiled_refuses_other_page_sizes(k):
     # not a power of two, too small, no such shape, pages larger than the tiles of the kernel of 32-row blocks
     for ps, shape in ((48, 42), (8, 42), (16, 43), (128, 142)):
         with pytest.raises(RuntimeError):
-            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, None, None,
-                   0, 0, 0, None)
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, ps, 0.1, 0, shape, 1, None,
+                   None, 0, 0, 0, None)
+    # shared keys: only in the kernel of 32-row blocks, and with room for the parts
+    for shape, splits, parts in ((42, 2, p), (142, 2, None), (142, 0, p), (142, 65, p)):
+        with pytest.raises(RuntimeError):
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, 2, 1, 64, 16, 0.1, 0, shape, splits, parts,
+                   parts, 0, 0, 0, None)
     # single tokens to the decode kernel: more than 16 heads to a group, key ranges without room for their parts
     for nq, splits, parts in ((17, 1, None), (2, 2, None), (2, 65, p)):
         with pytest.raises(RuntimeError):
-            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, nq, 1, 64, 16, 0.1, 0, 42, parts, parts,
+            k._run("egpt_paged_attention_tiled", p, p, p, p, p, 1, p, p, p, 1, 1, nq, 1, 64, 16, 0.1, 0, 42, 1, parts, parts,
                    splits, 4, 0, None)
 
 

@@ -200,6 +200,51 @@ def test_decoding_behind_a_long_prefix_splits_the_keys_many_times(models_0p5b, d
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_portions_of_a_long_prompt_beside_decoded_tokens(models_0p5b, dtype):
+    # a prompt of 9,000 tokens in portions of 512 and less, every step beside the decoded tokens of two requests behind
+    # 3,000 tokens: in bfloat16 the portions' blocks of rows share their keys among several workgroups once the
+    # prefix is long, and the requests of one token go to the decode kernel; the steps replay the graphs of their
+    # padded sizes
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    model_dir, cfg, w = models_0p5b(dtype)
+    n_long, lens = 9000, {"b": 3011, "c": 2990}
+    cuts = [512] * 9 + [300, 512, 64, 512, 2, 512, 16] + [512] * 4
+    cuts.append(n_long - sum(cuts))
+    assert 0 < cuts[-1] <= 512
+    reqs = {"long": H.make_requests(VOCAB, [n_long], seed=80)["r0"]}
+    for i, (rid, n) in enumerate(lens.items()):
+        reqs[rid] = H.make_requests(VOCAB, [n + len(cuts)], seed=81 + i)["r0"]
+    eng = engine_for(model_dir, dtype, max_tokens=9216 + 2 * 3072, max_requests=3)
+    rows, fed = {}, {}
+    for rid, n in lens.items():
+        eng.add_request(rid)
+        for pos in range(0, n, 2048):
+            step = min(2048, n - pos)
+            eng.step([StepEntry(rid, reqs[rid][pos : pos + step], [])])
+        fed[rid] = n
+    eng.add_request("long")
+    pos = 0
+    for i, n in enumerate(cuts):
+        want = [0, n - 1] if i % 4 == 1 or i >= len(cuts) - 2 or n < 100 else []
+        entries = [StepEntry("long", reqs["long"][pos : pos + n], want)]
+        entries += [StepEntry(rid, [reqs[rid][fed[rid]]], [0]) for rid in lens]
+        out = eng.step(entries).float().cpu()
+        for j, at in enumerate(want):
+            rows[("long", pos + at)] = out[j].clone()
+        for j, rid in enumerate(lens):
+            rows[(rid, fed[rid])] = out[len(want) + j].clone()
+            fed[rid] += 1
+        pos += n
+    assert pos == n_long
+    assert any(p.graph is not None for p in eng._padded_plans.values())
+    for rid in reqs:
+        eng.finish(rid)
+    compare(rows, cfg, w, reqs, tol_of(dtype), f"0.5B sizes {dtype} portions of a long prompt beside decoded tokens")
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_decoding_behind_32000_tokens(models_0p5b, dtype):
     # the longest context of the benchmark's record: a request of 32,000 tokens, its prompt fed in one step of that
     # many tokens (no graph covers it) and, again, in portions of 2,048 (replayed from the graph of that size); then
