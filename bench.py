@@ -178,6 +178,10 @@ def further_points(args, model_dir: str, cfg: dict, g) -> dict:
     decode_runs(engine, sampler, cfg["vocab_size"], "", PREFIX, FURTHER_BATCHES)
     for label, prefix, batches in FURTHER_CONTEXTS:
         rate(f"{label}_prefill", prefix, prefill_seconds(engine, cfg["vocab_size"], prefix, g, reps=3), per_step=False)
+        if label == "ctx32k":
+            # the same prompt as the scheduler feeds it under a budget of 512 tokens a step
+            rate(f"{label}_prefill_in_512s", prefix,
+                 prefill_in_portions_seconds(engine, cfg["vocab_size"], prefix, SERVE_CHUNK, g), per_step=False)
         decode_runs(engine, sampler, cfg["vocab_size"], label, prefix, batches)
     # ---- the mixed serving workload through the scheduler (what `--serve` prints)
     serve = serve_workload(engine, args, cfg["vocab_size"])
@@ -223,6 +227,28 @@ def prefill_seconds(engine, vocab: int, tokens: int, g, reps: int = 10) -> float
         times.append(time.perf_counter() - t0)
         engine.finish("prefill")
     return sorted(times[1:])[len(times[1:]) // 2]
+
+
+def prefill_in_portions_seconds(engine, vocab: int, tokens: int, portion: int, g, reps: int = 2) -> float:
+    """One prompt of `tokens` tokens in steps of `portion` tokens each, as the scheduler feeds a long prompt under a token
+    budget; logits at its last place: the fastest of `reps` passes after one warm-up."""
+    import torch
+
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    ids = torch.randint(0, vocab, (tokens,), generator=g).tolist()
+    times = []
+    for rep in range(reps + 1):
+        engine.add_request("prefill")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for pos in range(0, tokens, portion):
+            n = min(portion, tokens - pos)
+            engine.step([StepEntry("prefill", ids[pos : pos + n], [n - 1] if pos + n == tokens else [])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.finish("prefill")
+    return min(times[1:])
 
 
 def fill_requests(engine, sampler, vocab: int, prefix: int, batch: int, g):

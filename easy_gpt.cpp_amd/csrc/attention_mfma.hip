@@ -561,7 +561,7 @@ __device__ __forceinline__ void static_for(F&& f) {
     static_for_each(std::make_integer_sequence<int, N>{}, f);
 }
 
-template <int HD, int RB, int KS>
+template <int HD, int RB, int KS, bool SPLIT>
 __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_width,
@@ -609,10 +609,12 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const int blk_lo = window > 0 ? max(0, blk_first_pos - window + 1) : 0;
     // n_splits > 1: the tiles of keys are dealt over as many workgroups (blockIdx.z), each of which leaves its rows'
     // unnormalised result with its maximum and sum in part_o / part_ml for the kernel that combines them
+    // (SPLIT is a parameter of the template so that the kernel without it is compiled as if this were not here)
     const int t_first = blk_lo / KT, t_last = blk_p_hi / KT + 1;
-    const int t_per = max((t_last - t_first + n_splits - 1) / n_splits, 4);    // (a few tiles are not worth sharing)
-    const int t_begin = t_first + static_cast<int>(blockIdx.z) * t_per, t_end = min(t_last, t_begin + t_per);
-    const size_t part_row0 = static_cast<size_t>(blockIdx.z) * n_tokens * nq;
+    const int t_per = SPLIT ? max((t_last - t_first + n_splits - 1) / n_splits, 4) : t_last - t_first;    // (a few tiles are not worth sharing)
+    const int t_begin = SPLIT ? t_first + static_cast<int>(blockIdx.z) * t_per : t_first;
+    const int t_end = SPLIT ? min(t_last, t_begin + t_per) : t_last;
+    [[maybe_unused]] const size_t part_row0 = SPLIT ? static_cast<size_t>(blockIdx.z) * n_tokens * nq : 0;
 
     // this wavefront's block of 32 rows, this lane's row
     const int row_base = blk_first + rb * 32;
@@ -639,13 +641,15 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
         }
     }
     const float scale2 = scale * 1.4426950408889634f;
-    if (t_begin >= t_end) {                  // (n_splits > 1 only) no tile of keys is left for this workgroup
-        if (valid && ksi == 0 && lh == 0) {
-            float* ml = part_ml + (part_row0 + static_cast<size_t>(tok) * nq + head) * 2;
-            ml[0] = -INFINITY;
-            ml[1] = 0.f;
+    if constexpr (SPLIT) {
+        if (t_begin >= t_end) {              // no tile of keys is left for this workgroup
+            if (valid && ksi == 0 && lh == 0) {
+                float* ml = part_ml + (part_row0 + static_cast<size_t>(tok) * nq + head) * 2;
+                ml[0] = -INFINITY;
+                ml[1] = 0.f;
+            }
+            return;
         }
-        return;
     }
 
     f32x16 o[FB];
@@ -924,7 +928,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     if constexpr (KS > 1) __syncthreads();           // the combination below writes over the tiles
     // the row's sum: feature 0 of the block of ones, which lane lr of half 0 holds
     float l = __shfl(o_sum[0], lr, kWave);
-    float m_part = m_run;                            // the maximum that o and l are in units of
+    [[maybe_unused]] float m_part = m_run;           // the maximum that o and l are in units of
     if constexpr (KS > 1) {
         // The wavefronts of one block of rows hold partial results over their keys: those with ks > 0 leave
         // theirs in LDS (the tiles are no longer read: the loop ended with a barrier), ks == 0 adds them up.
@@ -944,7 +948,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
 #pragma unroll
         for (int j = 0; j < KS - 1; ++j)
             m_all = fmaxf(m_all, comb[(static_cast<size_t>(j * RB + rb) * PER_LANE + FB * 16) * 64 + lane]);
-        m_part = m_all;
+        if constexpr (SPLIT) m_part = m_all;
         const float m_ref = m_all == -INFINITY ? 0.f : m_all;
         const float w0 = __builtin_amdgcn_exp2f((m_run - m_ref) * scale2);
         l *= w0;
@@ -963,7 +967,7 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
                 for (int e = 0; e < 16; ++e) o[f][e] += src[(f * 16 + e) * 64] * wj;
         }
     }
-    if (n_splits > 1) {
+    if constexpr (SPLIT) {
         // (element e of block f is feature f * 32 + (e / 4) * 8 + lh * 4 + e % 4: runs of four features; the maximum
         // goes out in units of the exponent's argument, as the combining kernel takes it; -inf: no key seen)
         if (valid) {
@@ -1025,7 +1029,7 @@ struct FusedQkv {
 // qkv_rope_store_kernel, so the same bits) and keeps the queries in LDS.  The workgroup whose key range ends
 // with the new token does the same for that token's key and value, writes them to the cache and, because
 // its own loads of that cache line may have been issued before, puts them into its operands itself.
-template <int HD, int PF, bool FUSED>
+template <int HD, int PF, bool FUSED, bool MIXED = false>
 __global__ __launch_bounds__(512) void attention_decode_kernel(
     const bf16_t* __restrict__ qkv, bf16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -1034,9 +1038,12 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
     int n_splits, FusedQkv f, const int32_t* __restrict__ q_len) {
     constexpr int KD = HD / 32, DT = HD / 16;
     constexpr int kRow = HD + 2;
-    // q_len given: a step that also holds portions of prompts; this kernel takes its requests of one token, parts are
-    // kept by request (n_tokens is the number of requests then) and the rest is another kernel's
-    if (q_len != nullptr && q_len[blockIdx.x] != 1) return;
+    // MIXED: a step that also holds portions of prompts; this kernel takes its requests of one token, parts are kept
+    // by request (n_tokens is the number of requests then) and the rest is another kernel's.  (A parameter of the
+    // template, so that the kernel of the decode step is compiled as if this were not here.)
+    if constexpr (MIXED) {
+        if (q_len[blockIdx.x] != 1) return;
+    }
     extern __shared__ float wave_state[];          // [n_waves][16][HD + 2]: O, then maximum, then sum
     const int lane = threadIdx.x % kWave, n_waves = blockDim.x / kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // known to be the same for the wavefront
@@ -1341,7 +1348,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(
             out[(row0 + r) * HD + d] = from_float<bf16_t>(num / den);
         } else {
             const size_t prow = static_cast<size_t>(split) * n_tokens * nq +
-                                (q_len != nullptr ? static_cast<size_t>(b) * nq + kh * group_size : row0) + r;
+                                (MIXED ? static_cast<size_t>(b) * nq + kh * group_size : row0) + r;
             part_o[prow * HD + d] = num;
             if (d == 0) {
                 part_ml[prow * 2] = mx;
@@ -1454,11 +1461,12 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
     if (lds > kDecodeLdsMost) return EGPT_UNSUPPORTED_SIZE;
     if (lds > 64 * 1024) {
         // (eight wavefronts at head size 128: more than a kernel may take without being asked; once per instance)
-        static bool raised_fused = false, raised_plain = false;
-        bool& raised = fused ? raised_fused : raised_plain;
+        static bool raised_fused = false, raised_plain = false, raised_mixed = false;
+        bool& raised = fused ? raised_fused : q_len ? raised_mixed : raised_plain;
         if (!raised) {
-            const void* fn = fused ? reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, true>)
-                                   : reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, false>);
+            const void* fn = fused   ? reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, true>)
+                             : q_len ? reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, false, true>)
+                                     : reinterpret_cast<const void*>(&attention_decode_kernel<HD, PF, false>);
             if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsMost) != hipSuccess)
                 return EGPT_UNSUPPORTED_SIZE;
             raised = true;
@@ -1470,11 +1478,16 @@ static int launch_decode(const void* qkv, void* out, float* part_o, float* part_
             nullptr, static_cast<bf16_t*>(out), part_o, part_ml, static_cast<const bf16_t*>(k_cache),
             static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, kv_len, n_tokens, nq, nkv,
             page_size, scale, window, n_splits, fq, nullptr);
+    else if (q_len)
+        attention_decode_kernel<HD, PF, false, true><<<grid, n_waves * kWave, lds, s>>>(
+            static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
+            static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
+            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq, q_len);
     else
         attention_decode_kernel<HD, PF, false><<<grid, n_waves * kWave, lds, s>>>(
             static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), part_o, part_ml,
             static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start,
-            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq, q_len);
+            kv_len, n_tokens, nq, nkv, page_size, scale, window, n_splits, fq, nullptr);
     EGPT_CHECK_LAUNCH();
     if (n_splits > 1 && combine) {
         attention_reduce_kernel<<<n_tokens * nq, 64, 0, s>>>(part_o, part_ml, static_cast<bf16_t*>(out), n_tokens * nq,
@@ -1527,10 +1540,13 @@ static void launch_rows32(const void* qkv, void* out, const void* k_cache, const
                           int n_splits, hipStream_t s) {
     const long groups = (static_cast<long>(n_tokens) * (nq / nkv)) / (32 * RB) + n_seqs;   // upper bound
     dim3 grid(static_cast<unsigned>(groups), nkv, n_splits);
-    attention_rows32_kernel<HD, RB, KS><<<grid, 64 * RB * KS, 0, s>>>(
-        static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),
-        static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,
-        page_size, page_shift, scale, window, skip_single, part_o, part_ml, n_splits, n_tokens);
+#define EGPT_ROWS32_ARGS                                                                                           \
+    static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_cache),               \
+        static_cast<const bf16_t*>(v_cache), block_table, table_width, q_start, q_len, kv_len, n_seqs, nq, nkv,    \
+        page_size, page_shift, scale, window, skip_single, part_o, part_ml, n_splits, n_tokens
+    if (n_splits > 1) attention_rows32_kernel<HD, RB, KS, true><<<grid, 64 * RB * KS, 0, s>>>(EGPT_ROWS32_ARGS);
+    else attention_rows32_kernel<HD, RB, KS, false><<<grid, 64 * RB * KS, 0, s>>>(EGPT_ROWS32_ARGS);
+#undef EGPT_ROWS32_ARGS
     // (the rows of requests that were left out have no parts: what is combined for them is written over by the
     // kernel that takes them, which runs behind this one)
     if (n_splits > 1)

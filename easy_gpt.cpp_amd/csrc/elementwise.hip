@@ -48,7 +48,7 @@ __global__ void embed_kernel(const int32_t* __restrict__ ids, const T* __restric
 // ss = sum x^2 (float32), inv = 1/sqrt(ss/H + eps), y = x * inv * w
 // (/root/reference/src/models/norm.cpp:47-59, /root/reference/src/cuda/ops/self_attn_detail.cuh:385-418).
 // The residual addition h += delta happens here too, in float32.
-template <typename T, typename R>
+template <typename T, typename R, int KEEP>
 __global__ void add_rmsnorm_kernel(R* __restrict__ h, ProductView<T> delta,
                                    const int32_t* __restrict__ rows, const T* __restrict__ weight, float eps,
                                    T* __restrict__ out, int hidden) {
@@ -59,11 +59,11 @@ __global__ void add_rmsnorm_kernel(R* __restrict__ h, ProductView<T> delta,
     const bool has_delta = delta.present();
     const size_t dbase = src * hidden;
     const bool write_back = (rows == nullptr) && has_delta;
-    // A row of up to eight values per thread stays in registers, with its norm weight: all of a thread's loads are
-    // issued together, and the sum over the workgroup is the only wait between them and the stores.  (A loop over
-    // the row instead waits for memory once per round: 10 us for a row of 3,584 values with 512 threads, 9 us for
-    // one of 5,120 with 1,024.)
-    constexpr int KEEP = 8;
+    // A row of up to KEEP (four or eight) values per thread stays in registers, with its norm weight: all of a
+    // thread's loads are issued together, and the sum over the workgroup is the only wait between them and the
+    // stores.  (A loop over the row instead waits for memory once per round: 10 us for a row of 3,584 values with 512
+    // threads, 7.4 us for one of 5,120 with 1,024 against 6.2 from registers; eight where four are enough cost 0.3 to
+    // 0.7 us.)
     if (hidden <= KEEP * static_cast<int>(blockDim.x)) {
         float v[KEEP], w[KEEP];
 #pragma unroll
@@ -457,7 +457,7 @@ extern "C" int egpt_add_rmsnorm(void* h, int fixed, const void* delta, int delta
     if (n_rows == 0) return EGPT_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // few rows with many partial sums each: more threads, so that each has fewer dependent loads to wait for; and
-    // enough threads for a row to stay in registers (up to eight values a thread)
+    // enough threads for a row to stay in registers (four values a thread, eight for the widest rows)
     const int threads = (delta_splits > 1 || hidden > 2048) ? 1024 : (hidden > 1024 ? 512 : 256);
     const size_t stride = static_cast<size_t>(delta_rows) * hidden;
     if (dtype == 1 && delta_splits <= 1 && hidden % 8 == 0 && n_rows >= 32 && !fixed) {
@@ -475,15 +475,22 @@ extern "C" int egpt_add_rmsnorm(void* h, int fixed, const void* delta, int delta
         return EGPT_OK;
     }
     if (dtype != 0 && dtype != 1) return EGPT_BAD_ARGUMENT;
-#define EGPT_NORM(T_, R_)                                                                                              \
-    add_rmsnorm_kernel<T_, R_><<<n_rows, threads, 0, s>>>(static_cast<R_*>(h), make_view<T_>(delta, delta_splits, stride), \
-                                                          rows, static_cast<const T_*>(weight), eps,                  \
-                                                          static_cast<T_*>(out), hidden)
+#define EGPT_NORM_KEEP(T_, R_, KEEP_)                                                                      \
+    add_rmsnorm_kernel<T_, R_, KEEP_><<<n_rows, threads, 0, s>>>(                                          \
+        static_cast<R_*>(h), make_view<T_>(delta, delta_splits, stride), rows, static_cast<const T_*>(weight), eps, \
+        static_cast<T_*>(out), hidden)
+#define EGPT_NORM(T_, R_)                                        \
+    do {                                                         \
+        /* (a wide row behind partial sums is faster in the loop: 7.7 against 8.7 us at 64 rows of 5,120) */ \
+        if (hidden <= 4 * threads || delta_splits > 1) EGPT_NORM_KEEP(T_, R_, 4);    \
+        else EGPT_NORM_KEEP(T_, R_, 8);                          \
+    } while (0)
     if (dtype == 0 && !fixed) EGPT_NORM(float, float);
     else if (dtype == 0) EGPT_NORM(float, fixed_t);
     else if (!fixed) EGPT_NORM(bf16_t, float);
     else EGPT_NORM(bf16_t, fixed_t);
 #undef EGPT_NORM
+#undef EGPT_NORM_KEEP
     EGPT_CHECK_LAUNCH();
     return EGPT_OK;
 }
