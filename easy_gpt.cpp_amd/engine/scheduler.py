@@ -38,7 +38,7 @@ class SchedulerConfig:
     max_active: int = 16            # the reference's --serve-max-active
     max_admit_per_step: int = 4     # the reference's --serve-prefill-batch
     max_tokens_per_step: int = 2048
-    prefill_chunk: int = 512
+    prefill_chunk: int = 512        # a request's share of a step's budget; what is left of the budget goes to portions too
 
     def __post_init__(self):
         for name in ("max_active", "max_admit_per_step", "max_tokens_per_step", "prefill_chunk"):
@@ -290,6 +290,25 @@ class Scheduler:
                 assert ok
                 entries.append(PlannedEntry(r, 0, count, count == r.pending()))
                 budget -= count
+            # 4. what is left of the budget goes to the portions that were cut at `prefill_chunk`, in their order: a
+            # long prompt that is alone in its step has the whole step (few tokens behind a long prefix use the GPU badly)
+            for e in entries:
+                left = e.request.pending() - e.count
+                if budget < 1:
+                    break
+                if e.samples or left < 1:
+                    continue
+                rc = self.cache.requests[e.request.request_id]
+                more = min(left, budget)
+                have = self.cache.pages_needed(rc, e.count)
+                need = [a - b for a, b in zip(self.cache.pages_needed(rc, e.count + more), have)]
+                if any(n > pool.free_count - p for n, pool, p in zip(need, self.cache.pools, promised)):
+                    continue                # (the pages are short: the portion stays as it is)
+                for g, n in enumerate(need):
+                    promised[g] += n
+                e.count += more
+                e.samples = e.count == e.request.pending()
+                budget -= more
             if entries or not self.running:
                 return entries
             # nothing can move although requests are running: free the newest one's pages

@@ -94,13 +94,43 @@ def test_budget_portions_and_decode_first():
     b = s.add(Request("b", list(range(2, 6)), GREEDY, max_new_tokens=3))
     s.run()
     assert eng.log[0] == [("a", 6, []), ("b", 4, [3])]             # chunk 6, then b gets the rest of the budget
-    assert eng.log[1] == [("b", 1, [0]), ("a", 6, [])]             # b decodes first, a goes on with its prompt
-    assert eng.log[2] == [("b", 1, [0]), ("a", 2, [1])]            # a's last portion of two tokens is sampled
+    # b decodes first; a goes on with its prompt: its share of 6, and the 2 more that the budget still holds
+    assert eng.log[1] == [("b", 1, [0]), ("a", 8, [7])]
+    assert eng.log[2] == [("a", 1, [0]), ("b", 1, [0])]
     assert all(sum(n for _, n, _ in step) <= 10 for step in eng.log)
     assert a.output == expected_output(a.prompt, 3) and b.output == expected_output(b.prompt, 3)
     assert a.finish_reason == b.finish_reason == "length"
     assert eng.cache.free_pages() == [200] and not eng.cache.requests
     assert s.stats.generated == 6 and s.stats.prompt_tokens == 18 and s.stats.finished == 2
+
+
+def test_what_is_left_of_the_budget_goes_to_the_portions():
+    # a prompt alone in its steps has the whole budget, not only its share
+    eng = FakeEngine(num_pages=200)
+    s = Scheduler(eng, SchedulerConfig(max_active=4, max_admit_per_step=4, max_tokens_per_step=10, prefill_chunk=4))
+    a = s.add(Request("a", list(range(1, 24)), GREEDY, max_new_tokens=1))
+    s.run()
+    assert [step[0][1:] for step in eng.log] == [(10, []), (10, []), (3, [2])]
+    # three prompts: each its share while the budget lasts, the rest to the first that has tokens left
+    eng = FakeEngine(num_pages=200)
+    s = Scheduler(eng, SchedulerConfig(max_active=4, max_admit_per_step=4, max_tokens_per_step=16, prefill_chunk=4))
+    rs = [s.add(Request(i, list(range(1, n + 1)), GREEDY, max_new_tokens=1)) for i, n in enumerate((3, 20, 20))]
+    s.step()
+    assert eng.log[0] == [(0, 3, [2]), (1, 9, []), (2, 4, [])]      # 3 + 4 + 4 leave 5, which request 1 takes
+    assert all(sum(n for _, n, _ in step) <= 16 for step in eng.log)
+    s.run()
+    assert all(r.output == expected_output(r.prompt, 1) for r in rs)
+    # no pages for more than the share: the portion stays as it is (4 pages of 4 tokens: b's 7 tokens take two, which
+    # leaves c's 11 one page beyond the one of its share)
+    eng = FakeEngine(num_pages=4)
+    s = Scheduler(eng, SchedulerConfig(max_active=2, max_admit_per_step=2, max_tokens_per_step=64, prefill_chunk=4))
+    b = s.add(Request("b", list(range(1, 8)), GREEDY, max_new_tokens=1))
+    c = s.add(Request("c", list(range(1, 12)), GREEDY, max_new_tokens=1))
+    s.step()
+    assert eng.log[0] == [("b", 7, [6]), ("c", 4, [])]
+    s.run()
+    assert b.output == expected_output(b.prompt, 1) and c.output == expected_output(c.prompt, 1)
+    assert eng.cache.free_pages() == [4] and not eng.cache.requests
 
 
 def test_admission_is_first_in_first_out_and_bounded():
