@@ -26,6 +26,8 @@ class StepContext:
     rows_independent       False when several of the B "requests" are tokens of one request (a portion laid out as
                            single-token rows that share a block table): a row's keys and values must then be in the
                            cache before any row's attention reads it
+    single_token_requests  False when no request of the step brings exactly one token: a kernel that takes those apart
+                           from the portions of prompts need not run
     """
 
     num_tokens: int
@@ -51,6 +53,7 @@ class StepContext:
     group_windows: list = field(default_factory=list)
     shared: dict = field(default_factory=dict)     # what parts of several layers compute once per step and share
     rows_independent: bool = True
+    single_token_requests: bool = True     # False when the step is known to hold no request of exactly one token
 
     def cache_view(self, cache_id: int, writes: bool) -> CacheView:
         g, j = self.cache_location[cache_id]

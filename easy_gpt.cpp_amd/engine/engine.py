@@ -253,6 +253,7 @@ class Engine:
         return StepContext(
             num_tokens=t, num_seqs=b, token_ids=d_tok, positions=d_pos, q_start=d_qs, q_len=d_ql, kv_len=d_kv,
             want_rows=d_want if want_rows else None, max_q_len=max(q_len), max_kv_len=max(kv_len),
+            single_token_requests=1 in q_len,
             q_start_host=q_start, q_len_host=q_len, kv_len_host=kv_len,
             state_slots=d_slot, state_slots_host=[rc.slot for rc in rcs],
             groups=groups, page_size=ps, kv_storage=self.kv, state_storage=self.states,
@@ -432,8 +433,11 @@ class Engine:
         n_wanted = sum(len(e.want) for e in entries)
         while r_pad < n_wanted:
             r_pad *= 2
-        key = (t_pad, b_pad, r_pad, tuple(widths))
-        plan = self._plan(self._padded_plans, key, lambda: _PaddedPlan(self, t_pad, b_pad, r_pad, widths))
+        # (steps with and without requests of one token have graphs of their own: the attention takes those requests
+        # apart, in a kernel that the others need not launch; the padding's tokens go either way)
+        singles = 1 in counts
+        key = (t_pad, b_pad, r_pad, tuple(widths), singles)
+        plan = self._plan(self._padded_plans, key, lambda: _PaddedPlan(self, t_pad, b_pad, r_pad, widths, singles))
         n_want = plan.fill(rcs, entries, counts)
         logits = self._run(plan)
         return logits[:n_want] if n_want else None
@@ -457,7 +461,7 @@ def _capture(graph, pool, run):
 class _PaddedPlan:
     """Static buffers, a pinned host mirror and the captured graph of one padded step size."""
 
-    def __init__(self, engine: Engine, t_pad: int, b_pad: int, r_pad: int, widths: list[int]):
+    def __init__(self, engine: Engine, t_pad: int, b_pad: int, r_pad: int, widths: list[int], singles: bool = True):
         self.t_pad, self.b_pad, self.widths = t_pad, b_pad, list(widths)
         # (no reference back to the engine: engine and plan would keep each other alive until the collector of
         # reference cycles runs, which may be in the middle of another engine's graph capture, where memory of
@@ -485,7 +489,7 @@ class _PaddedPlan:
             q_start_host=[0] * b_pad, q_len_host=[0] * b_pad, kv_len_host=[0] * b_pad,
             state_slots=view(5), state_slots_host=[0] * b_pad, groups=groups, page_size=ps, kv_storage=engine.kv,
             state_storage=engine.states, cache_location=engine.model.cache_location,
-            group_windows=[n.window for n in engine.cache.groups],
+            group_windows=[n.window for n in engine.cache.groups], single_token_requests=singles,
         )
         self.c_widths = _ints(self.widths)
         self.copied = None

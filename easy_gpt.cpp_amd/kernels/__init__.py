@@ -23,9 +23,11 @@ Methods of a backend (T tokens, B requests, R rows, act = bfloat16 or float32):
         values [P,nkv,hd,page_size]
   paged_attention(qkv, out act[T,nq*hd], k_cache, v_cache, block_table i32[B,W], q_start i32[B],
                   q_len i32[B], kv_len i32[B], nq, nkv, hd, page_size, scale, window,
-                  max_q_len, max_kv_len)
+                  max_q_len, max_kv_len, combine=True, singles=True)
         query i of request b stands at position p = kv_len[b] - q_len[b] + i and reads keys
         j <= p (and j > p - window if window > 0) of that request through its block table
+        (hints: singles=False says that no request brings exactly one token; combine=False lets the
+        caller combine the parts of a split key range, which are then returned)
   swiglu(gate_up act[T,2I], out act[T,I])        out = silu(gate_up[:, :I]) * gate_up[:, I:]
   argmax(logits f32[R,V], out i32[R])            lowest index among equal maxima
   sample(logits f32[R,V], temperature f32[R], top_k i32[R], top_p f32[R], uniform f32[R], out i32[R])

@@ -589,9 +589,10 @@ class HipKernels(KernelBackend):
         return out
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd, page_size,
-                        scale, window, max_q_len, max_kv_len, combine=True):
+                        scale, window, max_q_len, max_kv_len, combine=True, singles=True):
         """combine=False: when the kernel splits the key range, leave the parts to the caller and return
-        (part_o [S, T, nq, hd], part_ml [S, T, nq, 2]); `out` is then not written.  Returns None otherwise."""
+        (part_o [S, T, nq, hd], part_ml [S, T, nq, 2]); `out` is then not written.  Returns None otherwise.
+        singles=False: no request brings exactly one token (a hint: the kernel that takes those apart is not launched)."""
         t = qkv.shape[0]
         b, width = block_table.shape
         dt = self._act(qkv, "qkv")
@@ -661,7 +662,7 @@ class HipKernels(KernelBackend):
                 # 1.7 us, and the longest of them sets the launch's time
                 part_o = part_ml = None
                 n_splits = n_waves = lean = 0
-                if b > 1 and nq // nkv <= 16 and max_kv_len > self.singles_apart_beyond:
+                if singles and b > 1 and nq // nkv <= 16 and max_kv_len > self.singles_apart_beyond:
                     n_splits, n_waves, lean = self._decode_shape(b, nkv, hd, max_kv_len, True)
                 parts_rows = max(n_splits * b if n_splits > 1 else 0, key_splits * t if key_splits > 1 else 0)
                 if parts_rows:

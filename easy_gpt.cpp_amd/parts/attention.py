@@ -177,6 +177,7 @@ class GQAttention(Mixer):
         args = dict(
             nq=self.n_heads, nkv=self.n_kv_heads, hd=self.head_dim, page_size=cache.page_size,
             scale=self.scale, window=self.window or 0, max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len,
+            singles=getattr(ctx, "single_token_requests", True),
         )
         if want_parts:
             args["combine"] = False

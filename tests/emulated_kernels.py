@@ -82,7 +82,7 @@ class EmulatedKernels(KernelBackend):
         return qkv
 
     def paged_attention(self, qkv, out, k_cache, v_cache, block_table, q_start, q_len, kv_len, nq, nkv, hd,
-                        page_size, scale, window, max_q_len, max_kv_len):
+                        page_size, scale, window, max_q_len, max_kv_len, combine=True, singles=True):
         group = nq // nkv
         q_all = qkv.view(qkv.shape[0], nq + 2 * nkv, hd)[:, :nq].to(F64)
         for b in range(q_start.shape[0]):
