@@ -100,3 +100,48 @@ def test_cuttings_and_decoding_at_larger_sizes(larger_models, size, dtype):
         eng.finish(rid)
     compare(rows, cfg, w, reqs, tol_of(dtype), f"{size} sizes {dtype} decoding behind 1,100 tokens")
     assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size", ["1.5b", "7b"])
+def test_portions_behind_a_prefix_beside_decoded_tokens_at_larger_sizes(larger_models, size, dtype):
+    # a prompt of 3,900 tokens in portions of up to 512, every step beside the decoded tokens of two requests behind
+    # 2,300 tokens: at head size 128 the portions' blocks of rows share their keys among workgroups from 2,048 tokens
+    # on, and the requests of one token go to the decode kernel
+    from easy_gpt.cpp_amd.engine import StepEntry
+
+    model_dir, cfg, w = larger_models(size, dtype)
+    vocab = cfg["vocab_size"]
+    n_long, lens = 3900, {"b": 2311, "c": 2290}
+    cuts = [512] * 4 + [300, 512, 70, 2, 512]
+    cuts.append(n_long - sum(cuts))
+    assert 0 < cuts[-1] <= 512
+    reqs = {"long": H.make_requests(vocab, [n_long], seed=90)["r0"]}
+    for i, (rid, n) in enumerate(lens.items()):
+        reqs[rid] = H.make_requests(vocab, [n + len(cuts)], seed=91 + i)["r0"]
+    eng = engine_for(model_dir, dtype, max_tokens=4096 + 2 * 2432, max_requests=3)
+    rows, fed = {}, {}
+    for rid, n in lens.items():
+        eng.add_request(rid)
+        for pos in range(0, n, 2048):
+            step = min(2048, n - pos)
+            eng.step([StepEntry(rid, reqs[rid][pos : pos + step], [])])
+        fed[rid] = n
+    eng.add_request("long")
+    pos = 0
+    for i, n in enumerate(cuts):
+        want = [0, n - 1] if i % 3 == 1 or i >= len(cuts) - 2 or n < 100 else []
+        entries = [StepEntry("long", reqs["long"][pos : pos + n], want)]
+        entries += [StepEntry(rid, [reqs[rid][fed[rid]]], [0]) for rid in lens]
+        out = eng.step(entries).float().cpu()
+        for j, at in enumerate(want):
+            rows[("long", pos + at)] = out[j].clone()
+        for j, rid in enumerate(lens):
+            rows[(rid, fed[rid])] = out[len(want) + j].clone()
+            fed[rid] += 1
+        pos += n
+    assert pos == n_long
+    for rid in reqs:
+        eng.finish(rid)
+    compare(rows, cfg, w, reqs, tol_of(dtype), f"{size} sizes {dtype} portions behind a prefix beside decoded tokens")
+    assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools]
