@@ -652,7 +652,9 @@ class HipKernels(KernelBackend):
                 # 643, 141x1: 59 / 665, 141x4: 30 / 185; 28 heads on 4: 141x1: 61 / 671, 141x2: 48 / 378; 40 heads on 8
                 # (160 workgroups): 141x1: 103 / 679.
                 key_splits = 1
-                if blocks_of_32 and max_kv_len >= (self.prefix_keys if hd == 64 else self.prefix_keys // 2):
+                # (behind a prefix: the longest context is a few thousand tokens and at least twice the step's own)
+                if (blocks_of_32 and max_kv_len >= 2 * t
+                        and max_kv_len >= (self.prefix_keys if hd == 64 else self.prefix_keys // 2)):
                     shape = 142 if hd == 64 else 141
                     workgroups = -(-row_tiles // 8)
                     tiles = -(-max_kv_len // (64 * (shape % 10)))
