@@ -609,9 +609,10 @@ __global__ __launch_bounds__(64 * RB * KS) void attention_rows32_kernel(
     const int blk_lo = window > 0 ? max(0, blk_first_pos - window + 1) : 0;
     // n_splits > 1: the tiles of keys are dealt over as many workgroups (blockIdx.z), each of which leaves its rows'
     // unnormalised result with its maximum and sum in part_o / part_ml for the kernel that combines them
-    // (SPLIT is a parameter of the template so that the kernel without it is compiled as if this were not here)
+    // (SPLIT is a parameter of the template so that the kernel without it is compiled as if this were not here; a
+    // workgroup takes four tiles at least: fewer are not worth sharing)
     const int t_first = blk_lo / KT, t_last = blk_p_hi / KT + 1;
-    const int t_per = SPLIT ? max((t_last - t_first + n_splits - 1) / n_splits, 4) : t_last - t_first;    // (a few tiles are not worth sharing)
+    const int t_per = SPLIT ? max((t_last - t_first + n_splits - 1) / n_splits, 4) : t_last - t_first;
     const int t_begin = SPLIT ? t_first + static_cast<int>(blockIdx.z) * t_per : t_first;
     const int t_end = SPLIT ? min(t_last, t_begin + t_per) : t_last;
     [[maybe_unused]] const size_t part_row0 = SPLIT ? static_cast<size_t>(blockIdx.z) * n_tokens * nq : 0;
