@@ -105,3 +105,44 @@ def test_random_weights_are_the_same_on_every_device_and_without_a_file(tmp_path
         eng.add_request("r")
         rows.append(eng.step([StepEntry("r", ids, [0, 39])]).clone())
     assert torch.equal(rows[0], rows[1])
+
+
+def test_generation_under_page_pressure_gives_the_same_tokens_in_float32():
+    # 40 requests with prompts of 20 to 6,000 tokens on four layers of the 0.5B sizes, greedy: with room for all of them,
+    # and with so few pages that requests are preempted dozens of times (freed, queued again, their prompt and what
+    # they had generated computed again in other portions, beside other requests, on other pages).  In float32 a
+    # row's logits are the same bits however the work is cut and batched, so every request must get exactly the
+    # tokens it got with room
+    import random
+
+    from easy_gpt.cpp_amd import kernels
+    from easy_gpt.cpp_amd.engine import Engine
+    from easy_gpt.cpp_amd.engine.engine import load_random_model
+    from easy_gpt.cpp_amd.engine.scheduler import Request, Scheduler, SchedulerConfig
+    from easy_gpt.cpp_amd.sampling import SamplingParams
+
+    kernels.use_backend(None)
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 4, "hidden_size": 896,
+           "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
+           "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "max_position_embeddings": 32768,
+           "hidden_act": "silu", "torch_dtype": "bfloat16"}
+    model = load_random_model(cfg, seed=3, dtype="float32", device="cuda:0")
+    rnd = random.Random(5)
+    lens = [rnd.choice([rnd.randint(20, 300), rnd.randint(500, 3000), rnd.randint(4000, 6000)]) for _ in range(40)]
+    new = [rnd.choice([8, 40, 100]) for _ in lens]
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for n in lens]
+    outputs = {}
+    for label, max_tokens in (("room", sum(lens) + sum(new) + 4096), ("pressure", 10000)):
+        eng = Engine(model, page_size=16, max_tokens=max_tokens, max_requests=33)
+        sched = Scheduler(eng, SchedulerConfig(max_active=32, max_admit_per_step=4, max_tokens_per_step=2048,
+                                               prefill_chunk=512), eos_token_id=-1)
+        reqs = [sched.add(Request(i, p, SamplingParams(greedy=True), max_new_tokens=n, ignore_eos=True))
+                for i, (p, n) in enumerate(zip(prompts, new))]
+        sched.run()
+        assert all(r.finish_reason == "length" and len(r.output) == n for r, n in zip(reqs, new))
+        assert eng.cache.free_pages() == [p.num_pages for p in eng.cache.pools] and not eng.cache.requests
+        assert (sched.stats.preemptions > 20) == (label == "pressure")
+        outputs[label] = [list(r.output) for r in reqs]
+        del eng, sched
+    assert outputs["pressure"] == outputs["room"]
