@@ -137,15 +137,16 @@ def shape_config(shape: str) -> tuple[dict, int]:
     return dict(QWEN25_05B, **changes, num_hidden_layers=n_layers), prefix
 
 
-def further_points(args, model_dir: str, cfg: dict, g) -> dict:
-    """The points beside the record: a flat dict of tokens a second."""
+def further_points(args, model_dir: str, cfg: dict, g, points: dict) -> None:
+    """The points beside the record, tokens a second each, into the flat dict `points` (what was measured before a
+    failure stays there)."""
     import torch
 
     from easy_gpt.cpp_amd.engine import Engine
     from easy_gpt.cpp_amd.engine.engine import load_random_model
     from easy_gpt.cpp_amd.sampling import Sampler
 
-    points, page = {}, args.page_size
+    page = args.page_size
     warm, steps = FURTHER_WARMUP, FURTHER_STEPS
 
     def rate(name, tokens, sec, per_step=True):
@@ -207,7 +208,6 @@ def further_points(args, model_dir: str, cfg: dict, g) -> dict:
                         prefix, batches)
         del engine, sampler, model
         torch.cuda.empty_cache()
-    return points
 
 
 def prefill_seconds(engine, vocab: int, tokens: int, g, reps: int = 10) -> float:
@@ -541,7 +541,12 @@ def main() -> int:
     points = {f"decode_b{b}": round(b * args.steps / results[b][0], 1) for b in batches if b != args.batch}
     del engine
     if further:
-        points.update(further_points(args, tmp, cfg, g))
+        # (the record above stands whatever happens to the points beside it: a failure there is named in the line)
+        try:
+            further_points(args, tmp, cfg, g, points)
+        except Exception as e:      # noqa: BLE001
+            line["points_error"] = f"{type(e).__name__}: {str(e)[:200]}"
+            print(f"[bench] the further points stopped: {line['points_error']}", file=sys.stderr, flush=True)
     remove_folder(tmp)
     if points:
         line["points"] = points
